@@ -1,0 +1,162 @@
+/*
+ * C ABI of libwcn_hip.so: the MI355X (gfx950) sparse-convolution forward path.
+ *
+ * Conventions shared by every entry point
+ *   - every pointer argument is a DEVICE pointer owned by the caller unless its name starts with
+ *     `host_`; nothing is allocated or freed by the library; scratch memory is passed in as a
+ *     workspace whose size comes from the matching *_bytes() query;
+ *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it and, unless stated,
+ *     the call returns without waiting for the device;
+ *   - the return value is a status: 0 = success, negative = error (wcn_status_string());
+ *   - conditions only the device can see (probe limit of the coordinate table exceeded,
+ *     coordinate range too wide to pack, more than 2^31-1 pairs) are recorded in the table
+ *     header / result block and surface through wcn_kmap_read_result(), wcn_table_read_status();
+ *   - coordinates are rows [batch, x, y, z] of int32; index outputs are int32, bit-exact with the
+ *     reference's own results.
+ *
+ * Reference interfaces replaced (paths relative to the kenomo/WarpConvNet checkout):
+ *   hash table     warpconvnet/geometry/coords/search/torch_hashmap.py:102-322 and the CuPy
+ *                  RawKernels of warpconvnet/csrc/hashmap_kernels.cu:182-301
+ *   kernel map     warpconvnet/geometry/coords/search/torch_discrete.py:80-157,244-337 and
+ *                  warpconvnet/csrc/discrete_kernels.cu:183-213,264-370
+ *   strided coords warpconvnet/geometry/coords/ops/stride.py:17-54, warpconvnet/utils/unique.py:125-144
+ *   contraction    warpconvnet/csrc/warpconvnet_pybind.cpp:1174-1247 (_C.gemm.implicit_gemm,
+ *                  _C.gemm.cutlass_gemm_AD_gather_scatter) together with the per-offset Python
+ *                  loop of warpconvnet/nn/functional/sparse_conv.py:281-311,358-415,495-544
+ */
+#ifndef WCN_HIP_H_
+#define WCN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WCN_OK 0
+#define WCN_ERR_INVALID_ARGUMENT (-1)  /* null pointer, bad size, unsupported dtype ...        */
+#define WCN_ERR_LAUNCH (-2)            /* the HIP runtime refused a launch or a copy           */
+#define WCN_ERR_TABLE_OVERFLOW (-3)    /* probe limit exceeded: rebuild with a larger capacity */
+#define WCN_ERR_COORD_RANGE (-4)       /* bounding box of the keys cannot be packed in 63 bits */
+#define WCN_ERR_TOO_MANY_PAIRS (-5)    /* kernel map would hold more than 2^31-1 pairs         */
+#define WCN_ERR_WORKSPACE (-6)         /* workspace smaller than the *_bytes() query demands   */
+
+#define WCN_DTYPE_F32 0
+#define WCN_DTYPE_F16 1
+#define WCN_DTYPE_BF16 2
+
+/* Library version (major*10000 + minor*100 + patch). */
+int wcn_version(void);
+
+/* Text for a status code; replaces gemm_status_to_string (warpconvnet_pybind.cpp:1207-1226). */
+const char* wcn_status_string(int status);
+
+/* ---------------------------------------------------------------------------------------------
+ * Coordinate table.  Replaces TorchHashTable.insert/search (torch_hashmap.py:102-170,225-300;
+ * hashmap_kernels.cu:182-253).  Same observable results: search returns the row index of a key
+ * among the inserted keys or -1; among duplicate keys the LOWEST row index is returned (the
+ * reference returns whichever thread won a race).
+ * ------------------------------------------------------------------------------------------- */
+
+/* Slot count the library would pick for n_keys keys (a power of two). */
+int64_t wcn_table_default_capacity(int64_t n_keys);
+
+/* Bytes of workspace a table of n_keys keys and `capacity` slots needs. */
+size_t wcn_table_bytes(int64_t n_keys, int64_t capacity);
+
+/* Build the table over keys (n_keys, 4) int32.  `capacity` must be a power of two >= 64. */
+int wcn_table_build(const int32_t* keys, int64_t n_keys, void* table, int64_t capacity,
+                    void* stream);
+
+/* results[i] = row index of queries[i] (num_queries, 4) among the keys, or -1. */
+int wcn_table_query(const void* table, int64_t n_keys, int64_t capacity, const int32_t* queries,
+                    int64_t num_queries, int32_t* results, void* stream);
+
+/* Waits for the stream, then returns WCN_OK or the error the build kernels recorded;
+ * host_num_blocks (may be NULL) receives the number of occupied slots. */
+int wcn_table_read_status(const void* table, int32_t* host_num_blocks, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Kernel map.  Replaces generate_kernel_map's device work (torch_discrete.py:244-337,80-157;
+ * discrete_kernels.cu:264-334,183-213) with two calls and one host read in between:
+ *
+ *   wcn_kmap_count  -> per-offset pair counts, their prefix sums (device)
+ *   wcn_kmap_read_result (waits; host learns offsets[K+1], allocates in_maps/out_maps of L)
+ *   wcn_kmap_fill   -> in_maps[L], out_maps[L] in the reference's order: offsets concatenated
+ *                      in k order (k = (i*ky + j)*kz + kk), pairs ascending in output index.
+ *
+ * Query coordinate of output m and offset k: out[m] * [1, sx, sy, sz] + (0, i-cx, j-cy, kk-cz)
+ * with c = size/2 for odd sizes and 0 for even ones (discrete_kernels.cu:291-314).
+ * ------------------------------------------------------------------------------------------- */
+
+size_t wcn_kmap_workspace_bytes(int64_t num_out, int32_t num_offsets);
+
+int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
+                   int64_t num_out, const int32_t host_kernel_size[3],
+                   const int32_t host_stride[3], void* workspace, void* stream);
+
+/* Waits for the stream.  host_offsets[K+1] receives the exclusive prefix sums of the per-offset
+ * pair counts (host_offsets[K] = L).  Returns the table status or WCN_ERR_TOO_MANY_PAIRS. */
+int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_offsets,
+                         int64_t* host_offsets, void* stream);
+
+int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
+                  int64_t num_out, const int32_t host_kernel_size[3], const int32_t host_stride[3],
+                  const void* workspace, int32_t* in_maps, int32_t* out_maps, void* stream);
+
+/* Device address, inside a kmap workspace, of the (K, ceil(num_out/64)+1) int32 table
+ * group_start[k][g] = number of pairs of offset k whose output index is below 64*g.  The
+ * contraction accepts it as `host_or_null_group_start` to skip its own search. */
+const int32_t* wcn_kmap_group_start(const void* workspace, int64_t num_out, int32_t num_offsets);
+
+/* ---------------------------------------------------------------------------------------------
+ * Strided output coordinates.  Replaces stride_coords / unique_hashmap (stride.py:17-54,
+ * unique.py:125-144): rows of floor(coords / [1,sx,sy,sz]) made unique; the representative of
+ * equal rows is the lowest source row; output rows ascend in representative index (which keeps
+ * a batch-sorted input batch-sorted).  Division is exact integer floor division.
+ * ------------------------------------------------------------------------------------------- */
+
+size_t wcn_stride_unique_workspace_bytes(int64_t n, int64_t capacity);
+
+/* `capacity` is the slot count of the internal coordinate table (wcn_table_default_capacity(n),
+ * or larger after WCN_ERR_TABLE_OVERFLOW).  out_coords (>= n rows, 4) and first_index (>= n)
+ * are written for the first M rows; M is returned through wcn_stride_unique_read_count. */
+int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_stride[3],
+                      void* workspace, int64_t capacity, int32_t* out_coords,
+                      int32_t* first_index, void* stream);
+
+/* Waits for the stream; host_count receives M.  Returns the table status. */
+int wcn_stride_unique_read_count(const void* workspace, int64_t n, int64_t capacity,
+                                 int64_t* host_count, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Feature contraction.  Replaces, in one launch sequence, the whole per-offset loop of the
+ * reference forward (sparse_conv.py:281-311 / :358-415 / :495-544) and the native calls it
+ * makes (_C.gemm.implicit_gemm, _C.gemm.cutlass_gemm_AD_gather_scatter):
+ *
+ *   out[m, :] = bias + sum_k sum_{pairs p of offset k with out_maps[p] == m} X[in_maps[p], :] @ W[k]
+ *
+ * with fp32 accumulation and ONE rounding to the feature dtype at the end.  `out` is fully
+ * written (rows without pairs become bias or zero), never accumulated into.
+ * If identity_offset >= 0 that offset is applied as out[m] += X[m] @ W[identity_offset] for
+ * every m < min(N, M) and its pairs in the map are ignored, as the reference does
+ * (sparse_conv.py:292-302).
+ * Within every offset out_maps must be strictly ascending (true for every map the reference
+ * builds except the in/out-swapped map of a transposed convolution, which the caller sorts).
+ * ------------------------------------------------------------------------------------------- */
+
+size_t wcn_conv_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_in, int32_t c_out,
+                                int32_t dtype);
+
+int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                        const void* weight, int32_t weight_dtype, int32_t num_offsets,
+                        int32_t c_out, const void* bias_or_null, const int32_t* in_maps,
+                        const int32_t* out_maps, const int64_t* host_offsets,
+                        int32_t identity_offset, const int32_t* group_start_or_null, void* out,
+                        int64_t num_out, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WCN_HIP_H_ */

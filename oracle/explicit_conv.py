@@ -1,0 +1,44 @@
+"""Torch-CPU restatement of the reference's explicit gather-GEMM-scatter forward.
+
+TEST INFRASTRUCTURE ONLY (parity checker and the benchmark's cpu_baseline leg).
+
+Follows warpconvnet/nn/functional/sparse_conv.py:281-311 operation by operation, so that the
+rounding of a low-precision run (the running output is rounded to the compute dtype after every
+kernel offset) is reproduced by torch itself:
+
+    X, W cast to compute_dtype (if given)
+    out = X @ W[iden]                      if the map carries an identity index
+          zeros(M, C_out, dtype of X)      otherwise
+    for k in range(K), skipping iden and empty offsets, in k order:
+        out[out_map_k] += X[in_map_k] @ W[k]
+    return out cast back to the dtype X came in with
+
+The bias add and the output container are applied by the caller (sparse_conv.py:1794-1805).
+"""
+from typing import Optional
+
+import torch
+
+
+def explicit_gemm_forward(in_features: torch.Tensor, weight: torch.Tensor, in_maps: torch.Tensor,
+                          out_maps: torch.Tensor, offsets, identity_map_index: Optional[int],
+                          num_out_coords: int,
+                          compute_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    x = in_features if compute_dtype is None else in_features.to(compute_dtype)
+    w = weight if compute_dtype is None else weight.to(compute_dtype)
+    offs = [int(o) for o in offsets]
+    num_offsets = len(offs) - 1
+    if identity_map_index is not None:
+        out = torch.matmul(x, w[identity_map_index])
+    else:
+        out = torch.zeros(num_out_coords, w.shape[-1], dtype=x.dtype, device=x.device)
+    for k in range(num_offsets):
+        if k == identity_map_index:
+            continue
+        lo, hi = offs[k], offs[k + 1]
+        if hi == lo:
+            continue
+        rows_in = in_maps[lo:hi].long()
+        rows_out = out_maps[lo:hi].long()
+        out[rows_out] += torch.matmul(x[rows_in], w[k])
+    return out.to(dtype=in_features.dtype)

@@ -1,0 +1,208 @@
+"""GPU parity of the feature contraction and of the public convolution entry points.
+
+Yardsticks: the C oracle's double-precision explicit gather-GEMM-scatter, and the torch-CPU
+restatement of the reference's explicit path in the reference's own operation order (which
+reproduces its per-offset rounding in low precision).
+Tolerances (max|a-b| / max|b| per tensor): 1e-5 for fp32, 1e-2 for fp16 / bf16.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import elementwise_rel_err, kaiming_weight, normal_features, rel_err
+from warpconvnet_amd.utils import synthetic
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {torch.float32: 1e-5, torch.float16: 1e-2, torch.bfloat16: 1e-2}
+
+
+def _dev_i32(a):
+    return torch.as_tensor(np.ascontiguousarray(a), dtype=torch.int32, device=DEV)
+
+
+def _voxels(items, feats, **kw):
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    offsets = np.zeros(len(items) + 1, dtype=np.int64)
+    offsets[1:] = np.cumsum([len(i) for i in items])
+    coords = torch.as_tensor(np.concatenate(items, axis=0), dtype=torch.int32, device=DEV)
+    return Voxels(coords, feats.to(DEV), offsets=torch.as_tensor(offsets), **kw)
+
+
+def _oracle_out(oracle, x, w, in_coords, out_coords, ksize, stride, bias=None):
+    im, om, off, iden = oracle.kernel_map(in_coords, out_coords, ksize, stride)
+    out = oracle.explicit_conv_f64(x.double().numpy(), w.double().numpy(), im, om, off, iden,
+                                   len(out_coords))
+    if bias is not None:
+        out = out + bias.double().numpy()
+    return out, (im, om, off, iden)
+
+
+CONV_CASES = [
+    # name, dtype, c_in, c_out, voxels per item, batch, kernel
+    ("f32_32_32", torch.float32, 32, 32, 6000, 2, (3, 3, 3)),
+    ("f16_64_64", torch.float16, 64, 64, 6000, 2, (3, 3, 3)),
+    ("bf16_96_128", torch.bfloat16, 96, 128, 4000, 1, (3, 3, 3)),
+    ("f32_7_13", torch.float32, 7, 13, 3000, 2, (3, 3, 3)),     # the reference's odd channel counts
+    ("f16_16_13", torch.float16, 16, 13, 3000, 1, (3, 3, 3)),
+    ("f16_3_32", torch.float16, 3, 32, 3000, 1, (3, 3, 3)),      # network stem
+    ("f16_256_256", torch.float16, 256, 256, 1500, 1, (3, 3, 3)),
+    ("f16_16_16_k5", torch.float16, 16, 16, 3000, 1, (5, 5, 5)),
+    ("bf16_40_72_k2", torch.bfloat16, 40, 72, 3000, 1, (2, 2, 2)),
+]
+
+
+@pytest.mark.parametrize("name,dtype,c_in,c_out,n,batch,ksize", CONV_CASES,
+                         ids=[c[0] for c in CONV_CASES])
+def test_conv_stride1_matches_oracle(oracle, name, dtype, c_in, c_out, n, batch, ksize):
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    from oracle.explicit_conv import explicit_gemm_forward
+    items = [synthetic.random_cloud(10 + b, n, 26)[:, 1:] for b in range(batch)]
+    bc = synthetic.batch_indexed(items)
+    K = int(np.prod(ksize))
+    x = normal_features(len(bc), c_in, seed=3, dtype=dtype)
+    w = kaiming_weight(K, c_in, c_out, seed=4, dtype=dtype)
+    bias = (torch.randn(c_out, generator=torch.Generator().manual_seed(5)) * 0.1).to(dtype)
+    vox = _voxels(items, x)
+    out = spatially_sparse_conv(vox, w.to(DEV), ksize, bias=bias.to(DEV))
+    assert out.feature_tensor.dtype == dtype and out.feature_tensor.shape == (len(bc), c_out)
+    assert torch.equal(out.coordinate_tensor, vox.coordinate_tensor)
+    got = out.feature_tensor.float().cpu().numpy()
+    want, (im, om, off, iden) = _oracle_out(oracle, x, w, bc, bc, ksize, (1, 1, 1), bias)
+    assert rel_err(got, want) <= TOL[dtype], name
+    # the reference's own operation order (per-offset rounding) on the CPU, same tolerance
+    ref = explicit_gemm_forward(x.float() if dtype != torch.float32 else x, w.float(),
+                                torch.as_tensor(im), torch.as_tensor(om), off, iden, len(bc))
+    ref = ref.double().numpy() + bias.double().numpy()
+    assert rel_err(got, ref) <= TOL[dtype], name
+
+
+def test_conv_dense_cube_equals_conv3d():
+    """Textbook anchor: on a fully occupied cube with zero padding the sparse convolution is
+    torch.nn.functional.conv3d (cross-correlation), W[k] <-> weight[:, :, i, j, kk].T with
+    k = (i * 3 + j) * 3 + kk."""
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    S, c_in, c_out = 12, 8, 16
+    g = torch.Generator().manual_seed(0)
+    dense = torch.randn(1, c_in, S, S, S, generator=g)
+    w = torch.randn(27, c_in, c_out, generator=g) * 0.2
+    xs, ys, zs = torch.meshgrid(torch.arange(S), torch.arange(S), torch.arange(S), indexing="ij")
+    coords = torch.stack([xs, ys, zs], dim=-1).reshape(-1, 3).int()
+    perm = torch.randperm(len(coords), generator=g)
+    coords = coords[perm]
+    feats = dense[0, :, coords[:, 0].long(), coords[:, 1].long(), coords[:, 2].long()].T.contiguous()
+    vox = _voxels([coords.numpy()], feats)
+    out = spatially_sparse_conv(vox, w.to(DEV), 3).feature_tensor.cpu()
+    w5 = w.reshape(3, 3, 3, c_in, c_out).permute(4, 3, 0, 1, 2).contiguous()
+    want = torch.nn.functional.conv3d(dense, w5, padding=1)[0]
+    want = want[:, coords[:, 0].long(), coords[:, 1].long(), coords[:, 2].long()].T
+    assert rel_err(out.numpy(), want.numpy()) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_strided_then_transposed_pair(oracle, dtype):
+    """2x2x2 stride-2 down convolution followed by its transposed convolution back onto the
+    fine coordinates; the second reuses the cached map with in/out exchanged."""
+    from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d
+    items = [synthetic.random_cloud(20 + b, 5000, 30)[:, 1:] for b in range(2)]
+    bc = synthetic.batch_indexed(items)
+    x = normal_features(len(bc), 24, seed=7, dtype=dtype)
+    fine = _voxels(items, x)
+    down = SparseConv3d(24, 40, 2, stride=2, bias=False).to(DEV)
+    up = SparseConv3d(40, 24, 2, stride=2, bias=True, transposed=True).to(DEV)
+    with torch.no_grad():
+        coarse = down(fine)
+        assert coarse.tensor_stride == (2, 2, 2)
+        assert fine.cache is not None and len(fine.cache) == 1
+        back = up(coarse, fine)
+        assert len(fine.cache) == 2  # transposed entry added, no new device map build
+    assert back.tensor_stride in (None, (1, 1, 1))
+    assert torch.equal(back.coordinate_tensor, fine.coordinate_tensor)
+    # oracle: forward map fine->coarse, then the same map with in/out exchanged
+    coarse_bc = coarse.batch_indexed_coordinates.cpu().numpy()
+    wd = down.weight.detach().cpu()
+    wu = up.weight.detach().cpu()
+    im, om, off, iden = oracle.kernel_map(bc, coarse_bc, (2, 2, 2), (2, 2, 2))
+    assert iden is None
+    xd = x.to(dtype).double().numpy()
+    mid = oracle.explicit_conv_f64(xd, wd.to(dtype).double().numpy(), im, om, off, None,
+                                   len(coarse_bc))
+    assert rel_err(coarse.feature_tensor.float().cpu().numpy(), mid) <= TOL[dtype]
+    mid_in = coarse.feature_tensor.double().cpu().numpy()  # what the GPU fed the second conv
+    want = oracle.explicit_conv_f64(mid_in, wu.to(dtype).double().numpy(), om, im, off, None,
+                                    len(bc)) + up.bias.detach().to(dtype).double().cpu().numpy()
+    assert rel_err(back.feature_tensor.float().cpu().numpy(), want) <= TOL[dtype]
+
+
+def test_transposed_adjoint_identity():
+    """<conv(x), y> == <x, conv_T(y)> when the transposed weights are W[k]^T on the same map."""
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    items = [synthetic.random_cloud(30, 4000, 28)[:, 1:]]
+    x = normal_features(len(items[0]), 16, seed=1)
+    fine = _voxels(items, x)
+    w = kaiming_weight(8, 16, 24, seed=2)
+    coarse = spatially_sparse_conv(fine, w.to(DEV), 2, stride=2)
+    y = normal_features(len(coarse), 24, seed=3).to(DEV)
+    back = spatially_sparse_conv(coarse.replace(batched_features=y), w.transpose(1, 2).contiguous().to(DEV),
+                                 2, stride=2, transposed=True, output_spatially_sparse_tensor=fine)
+    lhs = (coarse.feature_tensor.double() * y.double()).sum().item()
+    rhs = (fine.feature_tensor.double() * back.feature_tensor.double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), 1.0)
+
+
+def test_conv_linearity_and_determinism():
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    items = [synthetic.random_cloud(40, 5000, 28)[:, 1:]]
+    n = len(items[0])
+    a = normal_features(n, 32, seed=1)
+    b = normal_features(n, 32, seed=2)
+    w = kaiming_weight(27, 32, 48, seed=3).to(DEV)
+    fa = spatially_sparse_conv(_voxels(items, a), w, 3).feature_tensor
+    fb = spatially_sparse_conv(_voxels(items, b), w, 3).feature_tensor
+    fab = spatially_sparse_conv(_voxels(items, 2 * a - 3 * b), w, 3).feature_tensor
+    assert rel_err((2 * fa - 3 * fb).cpu().numpy(), fab.cpu().numpy()) <= 1e-5
+    again = spatially_sparse_conv(_voxels(items, a), w, 3).feature_tensor
+    assert torch.equal(fa, again)  # no atomics: bitwise reproducible
+
+
+def test_one_by_one_shortcut_and_errors():
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    items = [synthetic.random_cloud(50, 500, 20)[:, 1:]]
+    x = normal_features(len(items[0]), 8, seed=1)
+    vox = _voxels(items, x)
+    w = kaiming_weight(1, 8, 4, seed=2).to(DEV)
+    out = spatially_sparse_conv(vox, w, 1)
+    assert torch.allclose(out.feature_tensor, vox.feature_tensor @ w[0])
+    with pytest.raises(TypeError):
+        spatially_sparse_conv(x, w, 3)
+    with pytest.raises(AssertionError):
+        spatially_sparse_conv(vox, kaiming_weight(8, 8, 4).to(DEV), 2, stride=2, transposed=True)
+
+
+def test_module_autocast_and_backward():
+    """AMP view of the features (reference: tests/nn/test_sparse_conv.py:527-585) and gradients
+    of the autograd Function against the torch-CPU restatement."""
+    from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d
+    from oracle.explicit_conv import explicit_gemm_forward
+    items = [synthetic.random_cloud(60, 2000, 22)[:, 1:]]
+    x = normal_features(len(items[0]), 16, seed=1)
+    conv = SparseConv3d(16, 32, 3).to(DEV)
+    with torch.autocast("cuda", dtype=torch.float16):
+        out = conv(_voxels(items, x))
+    assert out.batched_features.batched_tensor.dtype == torch.float16
+    # gradients
+    xg = x.clone().to(DEV).requires_grad_(True)
+    vox = _voxels(items, xg.detach())
+    vox.batched_features.batched_tensor = xg
+    out = conv(vox)
+    out.feature_tensor.square().sum().backward()
+    bc = synthetic.batch_indexed(items)
+    from oracle import cpu_oracle
+    im, om, off, iden = cpu_oracle.kernel_map(bc, bc, (3, 3, 3))
+    xc = x.clone().requires_grad_(True)
+    wc = conv.weight.detach().cpu().clone().requires_grad_(True)
+    ref = explicit_gemm_forward(xc, wc, torch.as_tensor(im), torch.as_tensor(om), off, iden,
+                                len(bc)) + conv.bias.detach().cpu()
+    ref.square().sum().backward()
+    assert rel_err(xg.grad.cpu().numpy(), xc.grad.numpy()) <= 1e-4
+    assert rel_err(conv.weight.grad.cpu().numpy(), wc.grad.numpy()) <= 1e-4

@@ -1,0 +1,178 @@
+"""GPU parity of the integer stages (table, kernel map, strided coordinates) against the CPU
+oracle.  Bit-exact: indices and coordinates must be identical."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import canonical_pairs, sort_rows
+from warpconvnet_amd.utils import synthetic
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _dev(a):
+    return torch.as_tensor(np.ascontiguousarray(a), dtype=torch.int32, device=DEV)
+
+
+def test_table_finds_every_key_and_rejects_absent_keys(oracle):
+    """Invariant of the reference's own test (tests/coords/test_torch_hashmap.py:35-69)."""
+    from warpconvnet_amd.geometry.coords.search.torch_hashmap import HashMethod, TorchHashTable
+    rng = np.random.default_rng(0)
+    keys = np.unique(rng.integers(-1000, 1000, size=(65536, 4)).astype(np.int32), axis=0)
+    rng.shuffle(keys)
+    for method in HashMethod:
+        table = TorchHashTable.from_keys(_dev(keys), hash_method=method, device=DEV)
+        got = table.search(_dev(keys)).cpu().numpy()
+        assert np.array_equal(got, np.arange(len(keys), dtype=np.int32))
+        absent = keys + np.array([0, 5000, 0, 0], dtype=np.int32)
+        assert (table.search(_dev(absent)).cpu().numpy() == -1).all()
+    # mixed queries against the oracle's restatement of the reference table
+    q = np.concatenate([keys[:1000], absent[:1000], keys[-7:] + np.array([0, 0, 0, 1], np.int32)])
+    ref = oracle.HashTable(keys).search(q)
+    assert np.array_equal(table.search(_dev(q)).cpu().numpy(), ref)
+
+
+def test_table_duplicates_lowest_row_wins():
+    from warpconvnet_amd.geometry.coords.search.torch_hashmap import TorchHashTable
+    rng = np.random.default_rng(1)
+    base = rng.integers(0, 50, size=(5000, 4)).astype(np.int32)  # many duplicates
+    table = TorchHashTable.from_keys(_dev(base), device=DEV)
+    got = table.search(_dev(base)).cpu().numpy()
+    first = {}
+    for i, r in enumerate(map(tuple, base.tolist())):
+        first.setdefault(r, i)
+    want = np.array([first[tuple(r)] for r in base.tolist()], dtype=np.int32)
+    assert np.array_equal(got, want)
+    assert np.array_equal(table.unique_index.cpu().numpy(), np.unique(want))
+
+
+def test_table_sparse_keys_force_a_rebuild():
+    """Isolated voxels put one key in every block: the default slot count overflows on the
+    device and the host retries with more slots; results stay exact."""
+    from warpconvnet_amd.geometry.coords.search.torch_hashmap import TorchHashTable
+    rng = np.random.default_rng(2)
+    keys = np.unique(rng.integers(0, 1 << 20, size=(200000, 4)).astype(np.int32), axis=0)
+    keys[:, 0] %= 8
+    keys = np.unique(keys, axis=0)
+    table = TorchHashTable.from_keys(_dev(keys), device=DEV)
+    got = table.search(_dev(keys)).cpu().numpy()
+    assert np.array_equal(got, np.arange(len(keys), dtype=np.int32))
+
+
+def test_table_extreme_coordinates_report_range_error():
+    from warpconvnet_amd._lib import WcnError
+    from warpconvnet_amd.geometry.coords.search.torch_hashmap import TorchHashTable
+    keys = np.array([[0, -2**31, -2**31, -2**31], [2**31 - 1, 2**31 - 1, 2**31 - 1, 2**31 - 1]],
+                    dtype=np.int32)
+    with pytest.raises(WcnError):
+        TorchHashTable.from_keys(_dev(keys), device=DEV)
+    # a wide but packable range works, negative coordinates included
+    keys = np.array([[0, -2**20, 5, 7], [3, 2**20, -9, 2**15], [1, 0, 0, 0]], dtype=np.int32)
+    table = TorchHashTable.from_keys(_dev(keys), device=DEV)
+    assert table.search(_dev(keys)).cpu().tolist() == [0, 1, 2]
+
+
+CASES = [
+    # name, coords generator, kernel, stride
+    ("cloud_k3", lambda: synthetic.random_cloud(0, 20000, 40, batch_size=3), (3, 3, 3), (1, 1, 1)),
+    ("cloud_k2s2", lambda: synthetic.random_cloud(1, 20000, 40, batch_size=2), (2, 2, 2), (2, 2, 2)),
+    ("cloud_k3s2", lambda: synthetic.random_cloud(2, 20000, 40, batch_size=2), (3, 3, 3), (2, 2, 2)),
+    ("cloud_k5", lambda: synthetic.random_cloud(3, 5000, 24, batch_size=1), (5, 5, 5), (1, 1, 1)),
+    ("cloud_k323", lambda: synthetic.random_cloud(4, 5000, 24, batch_size=2), (3, 2, 3), (1, 2, 1)),
+    ("spheres_k3", lambda: synthetic.batch_indexed([synthetic.spheres_scene(0, 100_000)]),
+     (3, 3, 3), (1, 1, 1)),
+    ("indoor_k3", lambda: synthetic.batch_indexed(synthetic.indoor_batch(2, 60_000)[0]),
+     (3, 3, 3), (1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("name,gen,ksize,stride", CASES, ids=[c[0] for c in CASES])
+def test_kernel_map_bit_exact(oracle, name, gen, ksize, stride):
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    in_coords = gen()
+    batches = int(in_coords[:, 0].max()) + 1
+    if any(s != 1 for s in stride):
+        out_dev, off_dev = stride_coords(_dev(in_coords), stride)
+        out_coords = out_dev.cpu().numpy()
+        # strided coordinates: same set as the oracle, same batch offsets
+        ref_out, _, ref_off = oracle.stride_coords(in_coords, stride, batches)
+        assert np.array_equal(sort_rows(out_coords), sort_rows(ref_out))
+        assert np.array_equal(off_dev.numpy().astype(np.int64), ref_off)
+        # and in this implementation's documented order: ascending first source row
+        assert np.array_equal(out_coords, ref_out)
+    else:
+        out_coords = in_coords
+    km = generate_kernel_map(_dev(in_coords), _dev(out_coords), stride, ksize)
+    ref_in, ref_out_map, ref_off, ref_iden = oracle.kernel_map(in_coords, out_coords, ksize, stride)
+    assert km.identity_map_index == ref_iden
+    assert np.array_equal(km.offsets.numpy().astype(np.int64), ref_off)
+    # native order equals the reference's (ascending output row inside every offset) ...
+    assert np.array_equal(km.in_maps.cpu().numpy(), ref_in)
+    assert np.array_equal(km.out_maps.cpu().numpy(), ref_out_map)
+    # ... and therefore also after the canonical sort
+    assert np.array_equal(canonical_pairs(km.in_maps.cpu(), km.out_maps.cpu(), km.offsets),
+                          canonical_pairs(ref_in, ref_out_map, ref_off))
+
+
+def test_kernel_map_invariants_full_size():
+    """Size-independent properties at the benchmark's size (4 x 250k voxels, 3x3x3):
+    identity row, offset symmetry, duplicate-free rows."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    items, _ = synthetic.indoor_batch(4, 250_000)
+    coords = _dev(synthetic.batch_indexed(items))
+    n = coords.shape[0]
+    km = generate_kernel_map(coords, coords, (1, 1, 1), (3, 3, 3))
+    assert km.identity_map_index == 13
+    i13, o13 = km[13]
+    ar = torch.arange(n, dtype=torch.int32, device=DEV)
+    assert torch.equal(i13, ar) and torch.equal(o13, ar)
+    counts = torch.diff(km.offsets)
+    assert torch.equal(counts, counts.flip(0))  # |map_k| == |map_{K-1-k}|
+    for k in (0, 5, 12):
+        a_in, a_out = km[k]
+        b_in, b_out = km[26 - k]
+        assert (torch.diff(a_out) > 0).all()
+        # (i, j) in map_k  <=>  (j, i) in map_{K-1-k}
+        order = torch.argsort(b_in)
+        assert torch.equal(b_in[order], a_out) and torch.equal(b_out[order], a_in)
+
+
+def test_kernel_map_stride2_every_fine_voxel_once():
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    items, _ = synthetic.indoor_batch(2, 100_000)
+    fine = _dev(synthetic.batch_indexed(items))
+    coarse, offsets = stride_coords(fine, (2, 2, 2))
+    assert int(offsets[-1]) == coarse.shape[0] < fine.shape[0]
+    km = generate_kernel_map(fine, coarse, (2, 2, 2), (2, 2, 2))
+    assert km.identity_map_index is None
+    assert int(km.offsets[-1]) == fine.shape[0]
+    assert torch.equal(torch.sort(km.in_maps).values,
+                       torch.arange(fine.shape[0], dtype=torch.int32, device=DEV))
+
+
+def test_kernel_map_skip_symmetric_prefix():
+    """reference: tests/nn/test_sparse_conv.py:137-181."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    coords = _dev(synthetic.random_cloud(5, 10000, 30, batch_size=2))
+    full = generate_kernel_map(coords, coords, (1, 1, 1), (3, 3, 3), kernel_dilation=(1, 1, 1))
+    skip = generate_kernel_map(coords, coords, (1, 1, 1), (3, 3, 3), kernel_dilation=(1, 1, 1),
+                               skip_symmetric_kernel_map=True)
+    assert skip.identity_map_index == 13
+    n = len(skip.offsets)
+    assert torch.equal(full.offsets[:n], skip.offsets)
+    assert torch.equal(full.in_maps[: int(full.offsets[n - 1])], skip.in_maps)
+    assert torch.equal(full.out_maps[: int(full.offsets[n - 1])], skip.out_maps)
+
+
+def test_empty_and_tiny_inputs():
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    one = _dev(np.array([[0, 3, 4, 5]], dtype=np.int32))
+    km = generate_kernel_map(one, one, (1, 1, 1), (3, 3, 3))
+    assert km.offsets.tolist() == [0] * 14 + [1] * 14
+    assert km.in_maps.tolist() == [0] and km.out_maps.tolist() == [0]
+    none = torch.empty((0, 4), dtype=torch.int32, device=DEV)
+    km = generate_kernel_map(one, none, (1, 1, 1), (3, 3, 3))
+    assert int(km.offsets[-1]) == 0 and len(km) == 27

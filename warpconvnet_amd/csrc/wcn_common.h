@@ -1,0 +1,175 @@
+// Shared host/device definitions of libwcn_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/wcn_hip.h"
+
+#define WCN_WAVE 64
+#define WCN_MAX_PROBE 128  // linear-probe bound of the block table (insert and lookup)
+#define WCN_EMPTY_KEY 0xFFFFFFFFFFFFFFFFull
+#define WCN_MAX_OFFSETS 1024  // kernel volume bound of the kernel-map kernels
+
+// Device-recorded conditions (TableHeader::status, a bit set).
+#define WCN_DEV_OVERFLOW 1
+#define WCN_DEV_RANGE 2
+
+// ---- coordinate table -------------------------------------------------------------------------
+// The table does not store one slot per voxel.  Space is cut into 4x4x4-voxel blocks; a slot
+// holds the packed block coordinate, a 64-bit occupancy mask of the block and the rank of its
+// first voxel in `perm`, the list of input rows grouped by block.  A voxel's row index is
+// perm[base + popcount(mask below its bit)].  One 32-byte slot answers up to 64 probes.
+struct __attribute__((aligned(32))) WcnSlot {
+  unsigned long long key;   // packed (batch, bx, by, bz) relative to the bounding box, or EMPTY
+  unsigned long long mask;  // bit (x&3)*16 + (y&3)*4 + (z&3)
+  int32_t base;             // first position of the block's voxels in perm
+  int32_t pad[3];
+};
+
+struct WcnTableHeader {  // first 256 bytes of a table workspace
+  int32_t mn[4];         // bounding box of the keys, per column
+  int32_t mx[4];
+  int32_t num_blocks;    // occupied slots
+  int32_t status;        // WCN_DEV_* bits
+  int32_t total;         // running sum of block populations (ends at the number of distinct keys)
+  int32_t reserved[53];
+};
+static_assert(sizeof(WcnTableHeader) == 256, "header is 256 bytes");
+
+struct WcnTableView {  // host-computed addresses inside a table workspace
+  WcnTableHeader* hdr;
+  WcnSlot* slots;
+  int32_t* perm;        // n_keys
+  int32_t* slot_of;     // n_keys (slot of each key; build scratch)
+  int32_t* block_list;  // min(capacity, n_keys) occupied slot ids in claim order
+  int64_t n_keys;
+  int64_t capacity;
+};
+
+static inline size_t wcn_align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static inline size_t wcn_table_layout(void* base, int64_t n_keys, int64_t capacity,
+                                      WcnTableView* v) {
+  char* p = (char*)base;
+  size_t off = 0;
+  if (v) v->hdr = (WcnTableHeader*)(p + off);
+  off += 256;
+  if (v) v->slots = (WcnSlot*)(p + off);
+  off += wcn_align256(sizeof(WcnSlot) * (size_t)capacity);
+  if (v) v->perm = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
+  if (v) v->slot_of = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
+  if (v) v->block_list = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)(capacity < n_keys ? capacity : n_keys));
+  if (v) {
+    v->n_keys = n_keys;
+    v->capacity = capacity;
+  }
+  return off;
+}
+
+#ifdef __HIPCC__
+
+// Bit layout of the packed block key, derived from the bounding box in the header.
+struct WcnLayout {
+  uint32_t amin[4];   // batch minimum; spatial minima rounded down to a multiple of 4
+  uint32_t span[4];   // largest valid (coord - amin) per column
+  uint32_t shift[4];  // left shift of each field in the key
+  bool ok;            // all fields fit in 63 bits
+};
+
+__device__ __forceinline__ WcnLayout wcn_make_layout(const WcnTableHeader* __restrict__ h) {
+  WcnLayout L;
+  uint32_t bits[4];
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    int32_t mn = h->mn[d], mx = h->mx[d];
+    uint32_t a = d == 0 ? (uint32_t)mn : ((uint32_t)mn & ~3u);
+    L.amin[d] = a;
+    L.span[d] = (uint32_t)mx - a;
+    uint32_t cells = d == 0 ? L.span[d] : (L.span[d] >> 2);  // largest field value
+    bits[d] = cells == 0 ? 0u : 32u - (uint32_t)__builtin_clz(cells);
+  }
+  L.shift[3] = 0;
+  L.shift[2] = bits[3];
+  L.shift[1] = bits[3] + bits[2];
+  L.shift[0] = bits[3] + bits[2] + bits[1];
+  L.ok = (bits[0] + bits[1] + bits[2] + bits[3]) <= 63u;
+  return L;
+}
+
+// Relative coordinates of (b,x,y,z); false if the point lies outside the bounding box.
+__device__ __forceinline__ bool wcn_relative(const WcnLayout& L, int b, int x, int y, int z,
+                                             uint32_t r[4]) {
+  r[0] = (uint32_t)b - L.amin[0];
+  r[1] = (uint32_t)x - L.amin[1];
+  r[2] = (uint32_t)y - L.amin[2];
+  r[3] = (uint32_t)z - L.amin[3];
+  return r[0] <= L.span[0] && r[1] <= L.span[1] && r[2] <= L.span[2] && r[3] <= L.span[3];
+}
+
+__device__ __forceinline__ unsigned long long wcn_block_key(const WcnLayout& L,
+                                                            const uint32_t r[4]) {
+  return ((unsigned long long)r[0] << L.shift[0]) | ((unsigned long long)(r[1] >> 2) << L.shift[1]) |
+         ((unsigned long long)(r[2] >> 2) << L.shift[2]) | (unsigned long long)(r[3] >> 2);
+}
+
+__device__ __forceinline__ uint32_t wcn_block_bit(const uint32_t r[4]) {
+  return ((r[1] & 3u) << 4) | ((r[2] & 3u) << 2) | (r[3] & 3u);
+}
+
+// 64-bit finaliser of MurmurHash3: spreads neighbouring block keys over the table.
+__device__ __forceinline__ uint32_t wcn_mix(unsigned long long k, uint32_t cap_mask) {
+  k ^= k >> 33;
+  k *= 0xff51afd7ed558ccdull;
+  k ^= k >> 33;
+  k *= 0xc4ceb9fe1a85ec53ull;
+  k ^= k >> 33;
+  return (uint32_t)k & cap_mask;
+}
+
+// Finds the slot of a block key.  Returns its mask (0 if the block is absent) and base.
+__device__ __forceinline__ unsigned long long wcn_lookup_block(const WcnSlot* __restrict__ slots,
+                                                               uint32_t cap_mask,
+                                                               unsigned long long key,
+                                                               int32_t* base) {
+  uint32_t h = wcn_mix(key, cap_mask);
+  for (int p = 0; p < WCN_MAX_PROBE; ++p) {
+    // one 16-byte load brings key and mask; base sits in the same 32-byte slot
+    const ulonglong2 km = *reinterpret_cast<const ulonglong2*>(&slots[h]);
+    if (km.x == key) {
+      *base = slots[h].base;
+      return km.y;
+    }
+    if (km.x == WCN_EMPTY_KEY) break;
+    h = (h + 1) & cap_mask;
+  }
+  *base = 0;
+  return 0ull;
+}
+
+__device__ __forceinline__ int wcn_rank_below(unsigned long long mask, uint32_t bit) {
+  return __popcll(mask & ((1ull << bit) - 1ull));
+}
+
+__device__ __forceinline__ int wcn_lane() { return (int)(threadIdx.x & 63); }
+
+// Inclusive prefix sum over the 64 lanes of a wave.
+__device__ __forceinline__ int wcn_wave_inclusive_sum(int v) {
+  const int lane = wcn_lane();
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    int t = __shfl_up(v, d, 64);
+    if (lane >= d) v += t;
+  }
+  return v;
+}
+
+#define WCN_LAUNCH_CHECK()                      \
+  do {                                          \
+    if (hipGetLastError() != hipSuccess) return WCN_ERR_LAUNCH; \
+  } while (0)
+
+#endif  // __HIPCC__

@@ -1,0 +1,398 @@
+// Kernel-map generation and strided output coordinates on top of the block table (gfx950).
+//
+// The reference materialises a dense (K, M) table of probe results and compacts it with several
+// passes (torch_discrete.py:80-157).  Here one thread owns one output voxel and walks the K
+// offsets in registers; a wave's 64 voxels form a "group".  Pass 1 (count) stores, per offset and
+// group, how many of the 64 probes hit (a ballot popcount); a row-wise exclusive scan turns the
+// counts into start positions; pass 2 (fill) repeats the probes and each lane writes its pair at
+// start + (number of hits in lower lanes).  Because groups are 64 consecutive output rows and
+// lanes ascend within a group, pairs come out in ascending output index for each offset, exactly
+// the reference's order (discrete_kernels.cu:183-213), with no (K, M) intermediate in HBM.
+#include "wcn_common.h"
+
+int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView& v,
+                         hipStream_t s);
+int wcn_table_status_from_bits(int32_t bits);
+
+namespace {
+
+struct KmapGeom {
+  int32_t kx, ky, kz;  // kernel size
+  int32_t sx, sy, sz;  // in-to-out stride ratio applied to the output coordinates
+  int32_t cx, cy, cz;  // centre: size/2 for odd sizes, 0 for even (discrete_kernels.cu:291-294)
+  int32_t K;
+};
+
+struct KmapWorkspace {  // host-computed addresses inside a kmap workspace
+  int64_t* result;      // [K+1] offsets, [K+1] = table status bits, [K+2] = occupied slots
+  int32_t* groups;      // (K, G+1): counts after pass 1, exclusive prefix sums after the scan
+  int64_t G;            // number of 64-row groups
+};
+
+inline size_t kmap_layout(void* base, int64_t num_out, int32_t K, KmapWorkspace* w) {
+  char* p = (char*)base;
+  size_t off = 0;
+  const int64_t G = (num_out + 63) / 64;
+  if (w) w->result = (int64_t*)(p + off);
+  off += wcn_align256(sizeof(int64_t) * (size_t)(K + 3));
+  if (w) w->groups = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)K * (size_t)(G + 1));
+  if (w) w->G = G;
+  return off;
+}
+
+inline int grid_for(int64_t n, int block) {
+  int64_t g = (n + block - 1) / block;
+  return (int)(g < 1 ? 1 : g);
+}
+
+// Probe results of one output voxel are produced offset by offset; consecutive offsets differ in
+// z (the fastest digit) and mostly fall in the block of the previous probe, whose slot is kept
+// in registers, so a 3x3x3 neighbourhood costs a handful of table reads, not 27.
+template <bool FILL>
+__global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restrict__ hdr,
+                                                 const WcnSlot* __restrict__ slots,
+                                                 uint32_t cap_mask,
+                                                 const int32_t* __restrict__ perm,
+                                                 const int4* __restrict__ out_coords,
+                                                 int64_t num_out, KmapGeom g,
+                                                 int32_t* __restrict__ groups, int64_t G,
+                                                 const int64_t* __restrict__ offsets,
+                                                 int32_t* __restrict__ in_maps,
+                                                 int32_t* __restrict__ out_maps) {
+  const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t group = m >> 6;  // wave-uniform
+  if (group >= G) return;
+  const int lane = wcn_lane();
+  const bool live = m < num_out;
+  const WcnLayout L = wcn_make_layout(hdr);
+  int4 c = make_int4(0, 0, 0, 0);
+  if (live) c = out_coords[m];
+  // query origin relative to the table's box, modulo 2^32 like the reference's int arithmetic
+  const uint32_t rb = (uint32_t)c.x - L.amin[0];
+  const uint32_t rx0 = (uint32_t)c.y * (uint32_t)g.sx - (uint32_t)g.cx - L.amin[1];
+  const uint32_t ry0 = (uint32_t)c.z * (uint32_t)g.sy - (uint32_t)g.cy - L.amin[2];
+  const uint32_t rz0 = (uint32_t)c.w * (uint32_t)g.sz - (uint32_t)g.cz - L.amin[3];
+  const bool usable = live && L.ok && rb <= L.span[0];
+
+  unsigned long long cached_key = WCN_EMPTY_KEY, cached_mask = 0ull;
+  int32_t cached_base = 0;
+  int k = 0;
+  for (int i = 0; i < g.kx; ++i) {
+    for (int j = 0; j < g.ky; ++j) {
+      for (int kk = 0; kk < g.kz; ++kk, ++k) {
+        int32_t found = -1;
+        uint32_t r[4] = {rb, rx0 + (uint32_t)i, ry0 + (uint32_t)j, rz0 + (uint32_t)kk};
+        if (usable && r[1] <= L.span[1] && r[2] <= L.span[2] && r[3] <= L.span[3]) {
+          const unsigned long long key = wcn_block_key(L, r);
+          if (key != cached_key) {
+            cached_mask = wcn_lookup_block(slots, cap_mask, key, &cached_base);
+            cached_key = key;
+          }
+          const uint32_t bit = wcn_block_bit(r);
+          if ((cached_mask >> bit) & 1ull) found = perm[cached_base + wcn_rank_below(cached_mask, bit)];
+        }
+        const unsigned long long hits = __ballot(found >= 0);
+        if (!FILL) {
+          if (lane == 0) groups[(int64_t)k * (G + 1) + group] = __popcll(hits);
+        } else if (found >= 0) {
+          const int64_t pos = offsets[k] + groups[(int64_t)k * (G + 1) + group] +
+                              __popcll(hits & ((1ull << lane) - 1ull));
+          in_maps[pos] = found;
+          out_maps[pos] = (int32_t)m;
+        }
+      }
+    }
+  }
+}
+
+// In-place exclusive prefix sum of each row of `groups` (one workgroup per row, G+1 entries; the
+// last entry receives the row total).
+__global__ void __launch_bounds__(256) kmap_scan_rows(int32_t* __restrict__ groups, int64_t G,
+                                                      int64_t* __restrict__ row_total) {
+  __shared__ int s_wave[4];
+  int32_t* row = groups + (int64_t)blockIdx.x * (G + 1);
+  const int lane = wcn_lane(), wave = threadIdx.x >> 6;
+  int64_t carry = 0;
+  for (int64_t start = 0; start < G; start += 256) {
+    const int64_t idx = start + threadIdx.x;
+    const int v = idx < G ? row[idx] : 0;
+    const int incl = wcn_wave_inclusive_sum(v);
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    int before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int t = s_wave[w];
+      if (w < wave) before += t;
+      all += t;
+    }
+    if (idx < G) row[idx] = (int32_t)(carry + before + incl - v);
+    carry += all;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    // a row holds at most M < 2^31 pairs, so the int32 entries cannot overflow
+    row[G] = (int32_t)carry;
+    row_total[blockIdx.x] = carry;
+  }
+}
+
+// offsets[K+1] = exclusive prefix sum of the row totals; also copies the table's status out so
+// the host needs one read for everything.  Single workgroup, serial over K <= 1024 (tiny).
+__global__ void kmap_finish(int64_t* __restrict__ result, int32_t K,
+                            const WcnTableHeader* __restrict__ hdr) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  // result[1..K] currently hold the row totals (written at result[k+1] by the scan)
+  int64_t run = 0;
+  result[0] = 0;
+  for (int k = 0; k < K; ++k) {
+    run += result[k + 1];
+    result[k + 1] = run;
+  }
+  result[K + 1] = hdr->status;
+  result[K + 2] = hdr->num_blocks;
+}
+
+bool make_geom(const int32_t ks[3], const int32_t st[3], KmapGeom* g) {
+  if (!ks || !st) return false;
+  for (int d = 0; d < 3; ++d)
+    if (ks[d] < 1 || st[d] < 1) return false;
+  const int64_t K = (int64_t)ks[0] * ks[1] * ks[2];
+  if (K > WCN_MAX_OFFSETS) return false;
+  g->kx = ks[0]; g->ky = ks[1]; g->kz = ks[2];
+  g->sx = st[0]; g->sy = st[1]; g->sz = st[2];
+  g->cx = (ks[0] % 2) ? ks[0] / 2 : 0;
+  g->cy = (ks[1] % 2) ? ks[1] / 2 : 0;
+  g->cz = (ks[2] % 2) ? ks[2] / 2 : 0;
+  g->K = (int32_t)K;
+  return true;
+}
+
+inline bool table_args_ok(const void* table, int64_t n_keys, int64_t capacity) {
+  return table && n_keys >= 0 && capacity >= 64 && (capacity & (capacity - 1)) == 0;
+}
+
+// ---- strided output coordinates -----------------------------------------------------------------
+
+struct StrideWorkspace {
+  int64_t* result;   // [0] = M, [1] = table status bits
+  int32_t* coarse;   // (n, 4) floor-divided coordinates
+  int32_t* groups;   // (1, G+1) winners per 64-row group, then prefix sums
+  void* table;       // block table over the coarse coordinates
+  int64_t G;
+};
+
+inline size_t stride_layout(void* base, int64_t n, int64_t capacity, StrideWorkspace* w) {
+  char* p = (char*)base;
+  size_t off = 0;
+  const int64_t G = (n + 63) / 64;
+  if (w) w->result = (int64_t*)(p + off);
+  off += 256;
+  if (w) w->coarse = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * 4 * (size_t)n);
+  if (w) w->groups = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)(G + 1));
+  if (w) w->table = (void*)(p + off);
+  off += wcn_table_layout(nullptr, n, capacity, nullptr);
+  if (w) w->G = G;
+  return off;
+}
+
+__device__ __forceinline__ int32_t floor_div(int32_t a, int32_t b) {  // b > 0
+  int32_t q = a / b;
+  return (a % b != 0 && a < 0) ? q - 1 : q;
+}
+
+__global__ void __launch_bounds__(256) stride_divide(const int4* __restrict__ coords, int64_t n,
+                                                     int32_t sx, int32_t sy, int32_t sz,
+                                                     int4* __restrict__ coarse) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int4 c = coords[i];
+  coarse[i] = make_int4(c.x, floor_div(c.y, sx), floor_div(c.z, sy), floor_div(c.w, sz));
+}
+
+// A row is the representative of its coordinate if perm at its rank holds its own index (perm
+// keeps the minimum row index per distinct coordinate).
+template <bool FILL>
+__global__ void __launch_bounds__(256) stride_pick(const int4* __restrict__ coarse, int64_t n,
+                                                   const WcnTableHeader* __restrict__ hdr,
+                                                   const WcnSlot* __restrict__ slots,
+                                                   const int32_t* __restrict__ slot_of,
+                                                   const int32_t* __restrict__ perm,
+                                                   int32_t* __restrict__ groups, int64_t G,
+                                                   int4* __restrict__ out_coords,
+                                                   int32_t* __restrict__ first_index) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t group = i >> 6;
+  if (group >= G) return;
+  const int lane = wcn_lane();
+  bool winner = false;
+  int4 c = make_int4(0, 0, 0, 0);
+  if (i < n) {
+    const int32_t h = slot_of[i];
+    if (h >= 0) {
+      const WcnLayout L = wcn_make_layout(hdr);
+      c = coarse[i];
+      uint32_t r[4];
+      wcn_relative(L, c.x, c.y, c.z, c.w, r);
+      const ulonglong2 km = *reinterpret_cast<const ulonglong2*>(&slots[h]);
+      const int64_t pos = (int64_t)slots[h].base + wcn_rank_below(km.y, wcn_block_bit(r));
+      winner = pos >= 0 && pos < n && perm[pos] == (int32_t)i;
+    }
+  }
+  const unsigned long long wins = __ballot(winner);
+  if (!FILL) {
+    if (lane == 0) groups[group] = __popcll(wins);
+  } else if (winner) {
+    const int64_t pos = (int64_t)groups[group] + __popcll(wins & ((1ull << lane) - 1ull));
+    out_coords[pos] = c;
+    first_index[pos] = (int32_t)i;
+  }
+}
+
+__global__ void stride_finish(int64_t* __restrict__ result, const int32_t* __restrict__ groups,
+                              int64_t G, const WcnTableHeader* __restrict__ hdr) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  result[0] = groups[G];
+  result[1] = hdr->status;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t wcn_kmap_workspace_bytes(int64_t num_out, int32_t num_offsets) {
+  if (num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS) return 0;
+  return kmap_layout(nullptr, num_out, num_offsets, nullptr);
+}
+
+int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
+                   int64_t num_out, const int32_t host_kernel_size[3],
+                   const int32_t host_stride[3], void* workspace, void* stream) {
+  KmapGeom g;
+  if (!make_geom(host_kernel_size, host_stride, &g)) return WCN_ERR_INVALID_ARGUMENT;
+  if (!table_args_ok(table, n_keys, capacity) || !workspace || num_out < 0 ||
+      num_out >= (1ll << 31) || (num_out > 0 && !out_coords))
+    return WCN_ERR_INVALID_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  WcnTableView v;
+  wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
+  KmapWorkspace w;
+  kmap_layout(workspace, num_out, g.K, &w);
+  if (w.G > 0) {
+    hipLaunchKernelGGL(kmap_pass<false>, dim3(grid_for(num_out, 256)), dim3(256), 0, s, v.hdr,
+                       v.slots, (uint32_t)(capacity - 1), v.perm, (const int4*)out_coords, num_out,
+                       g, w.groups, w.G, (const int64_t*)nullptr, (int32_t*)nullptr,
+                       (int32_t*)nullptr);
+  }
+  hipLaunchKernelGGL(kmap_scan_rows, dim3(g.K), dim3(256), 0, s, w.groups, w.G, w.result + 1);
+  hipLaunchKernelGGL(kmap_finish, dim3(1), dim3(64), 0, s, w.result, g.K, v.hdr);
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_offsets,
+                         int64_t* host_offsets, void* stream) {
+  if (!workspace || !host_offsets || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS)
+    return WCN_ERR_INVALID_ARGUMENT;
+  KmapWorkspace w;
+  kmap_layout(const_cast<void*>(workspace), num_out, num_offsets, &w);
+  int64_t tmp[WCN_MAX_OFFSETS + 3];
+  const size_t bytes = sizeof(int64_t) * (size_t)(num_offsets + 3);
+  if (hipMemcpyAsync(tmp, w.result, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream) !=
+      hipSuccess)
+    return WCN_ERR_LAUNCH;
+  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return WCN_ERR_LAUNCH;
+  for (int k = 0; k <= num_offsets; ++k) host_offsets[k] = tmp[k];
+  const int st = wcn_table_status_from_bits((int32_t)tmp[num_offsets + 1]);
+  if (st != WCN_OK) return st;
+  if (tmp[num_offsets] > INT32_MAX) return WCN_ERR_TOO_MANY_PAIRS;
+  return WCN_OK;
+}
+
+int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
+                  int64_t num_out, const int32_t host_kernel_size[3], const int32_t host_stride[3],
+                  const void* workspace, int32_t* in_maps, int32_t* out_maps, void* stream) {
+  KmapGeom g;
+  if (!make_geom(host_kernel_size, host_stride, &g)) return WCN_ERR_INVALID_ARGUMENT;
+  if (!table_args_ok(table, n_keys, capacity) || !workspace || num_out < 0 ||
+      num_out >= (1ll << 31) || (num_out > 0 && !out_coords))
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (num_out == 0) return WCN_OK;
+  if (!in_maps || !out_maps) return WCN_ERR_INVALID_ARGUMENT;
+  WcnTableView v;
+  wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
+  KmapWorkspace w;
+  kmap_layout(const_cast<void*>(workspace), num_out, g.K, &w);
+  hipLaunchKernelGGL(kmap_pass<true>, dim3(grid_for(num_out, 256)), dim3(256), 0,
+                     (hipStream_t)stream, v.hdr, v.slots, (uint32_t)(capacity - 1), v.perm,
+                     (const int4*)out_coords, num_out, g, w.groups, w.G, (const int64_t*)w.result,
+                     in_maps, out_maps);
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+const int32_t* wcn_kmap_group_start(const void* workspace, int64_t num_out, int32_t num_offsets) {
+  if (!workspace || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS) return nullptr;
+  KmapWorkspace w;
+  kmap_layout(const_cast<void*>(workspace), num_out, num_offsets, &w);
+  return w.groups;
+}
+
+size_t wcn_stride_unique_workspace_bytes(int64_t n, int64_t capacity) {
+  if (n < 0 || capacity < 64) return 0;
+  return stride_layout(nullptr, n, capacity, nullptr);
+}
+
+int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_stride[3],
+                      void* workspace, int64_t capacity, int32_t* out_coords,
+                      int32_t* first_index, void* stream) {
+  if (!workspace || n < 0 || n >= (1ll << 31) || !host_stride) return WCN_ERR_INVALID_ARGUMENT;
+  if (capacity < 64 || (capacity & (capacity - 1)) != 0) return WCN_ERR_INVALID_ARGUMENT;
+  if (n > 0 && (!coords || !out_coords || !first_index)) return WCN_ERR_INVALID_ARGUMENT;
+  for (int d = 0; d < 3; ++d)
+    if (host_stride[d] < 1) return WCN_ERR_INVALID_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  StrideWorkspace w;
+  stride_layout(workspace, n, capacity, &w);
+  WcnTableView v;
+  wcn_table_layout(w.table, n, capacity, &v);
+  if (n > 0) {
+    hipLaunchKernelGGL(stride_divide, dim3(grid_for(n, 256)), dim3(256), 0, s, (const int4*)coords,
+                       n, host_stride[0], host_stride[1], host_stride[2], (int4*)w.coarse);
+  }
+  const int rc = wcn_table_build_impl(w.coarse, n, v, s);
+  if (rc != WCN_OK) return rc;
+  if (n > 0) {
+    hipLaunchKernelGGL(stride_pick<false>, dim3(grid_for(n, 256)), dim3(256), 0, s,
+                       (const int4*)w.coarse, n, v.hdr, v.slots, v.slot_of, v.perm, w.groups, w.G,
+                       (int4*)nullptr, (int32_t*)nullptr);
+  }
+  hipLaunchKernelGGL(kmap_scan_rows, dim3(1), dim3(256), 0, s, w.groups, w.G, w.result + 2);
+  hipLaunchKernelGGL(stride_finish, dim3(1), dim3(64), 0, s, w.result, w.groups, w.G, v.hdr);
+  if (n > 0) {
+    hipLaunchKernelGGL(stride_pick<true>, dim3(grid_for(n, 256)), dim3(256), 0, s,
+                       (const int4*)w.coarse, n, v.hdr, v.slots, v.slot_of, v.perm, w.groups, w.G,
+                       (int4*)out_coords, first_index);
+  }
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+int wcn_stride_unique_read_count(const void* workspace, int64_t n, int64_t capacity,
+                                 int64_t* host_count, void* stream) {
+  if (!workspace || !host_count) return WCN_ERR_INVALID_ARGUMENT;
+  StrideWorkspace w;
+  stride_layout(const_cast<void*>(workspace), n, capacity, &w);
+  int64_t tmp[2];
+  if (hipMemcpyAsync(tmp, w.result, sizeof(tmp), hipMemcpyDeviceToHost, (hipStream_t)stream) !=
+      hipSuccess)
+    return WCN_ERR_LAUNCH;
+  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return WCN_ERR_LAUNCH;
+  *host_count = tmp[0];
+  return wcn_table_status_from_bits((int32_t)tmp[1]);
+}
+
+}  // extern "C"

@@ -1,0 +1,294 @@
+// Coordinate table of 4x4x4-voxel blocks: build and point queries (gfx950).
+//
+// Build pipeline (all on the caller's stream, no host round trip):
+//   table_clear   header, slots and perm to their empty values
+//   table_bbox    bounding box of the keys (LDS reduction, one atomic min/max per workgroup)
+//   table_insert  per key: claim / find the block slot with a 64-bit CAS, OR the voxel bit in
+//   table_base    per occupied slot: base = running sum of block populations (one atomic per wave)
+//   table_perm    per key: perm[base + rank of its bit] = min(row index)
+//
+// HBM traffic per key: 16 B read (bbox) + 16 B read (insert) + 4 B slot_of write + 4 B read +
+// 4 B perm write, plus 32 B per table slot to clear and one 32 B slot touched per key.
+#include "wcn_common.h"
+
+namespace {
+
+__global__ void __launch_bounds__(256) table_clear(WcnTableHeader* __restrict__ hdr,
+                                                   WcnSlot* __restrict__ slots, int64_t capacity,
+                                                   int32_t* __restrict__ perm, int64_t n_keys) {
+  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  if (tid == 0) {
+    for (int d = 0; d < 4; ++d) {
+      hdr->mn[d] = INT32_MAX;
+      hdr->mx[d] = INT32_MIN;
+    }
+    hdr->num_blocks = 0;
+    hdr->status = 0;
+    hdr->total = 0;
+  }
+  // each slot is two 16-byte stores: {EMPTY, 0} and {0, 0, 0, 0}
+  uint4* raw = reinterpret_cast<uint4*>(slots);
+  for (int64_t i = tid; i < 2 * capacity; i += nthreads) {
+    uint4 v = (i & 1) ? make_uint4(0u, 0u, 0u, 0u) : make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0u, 0u);
+    raw[i] = v;
+  }
+  for (int64_t i = tid; i < n_keys; i += nthreads) perm[i] = INT32_MAX;
+}
+
+__global__ void __launch_bounds__(256) table_bbox(const int4* __restrict__ keys, int64_t n_keys,
+                                                  WcnTableHeader* __restrict__ hdr) {
+  __shared__ int s_mn[4][4];
+  __shared__ int s_mx[4][4];
+  int mn[4] = {INT32_MAX, INT32_MAX, INT32_MAX, INT32_MAX};
+  int mx[4] = {INT32_MIN, INT32_MIN, INT32_MIN, INT32_MIN};
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_keys; i += nthreads) {
+    const int4 c = keys[i];
+    mn[0] = min(mn[0], c.x); mx[0] = max(mx[0], c.x);
+    mn[1] = min(mn[1], c.y); mx[1] = max(mx[1], c.y);
+    mn[2] = min(mn[2], c.z); mx[2] = max(mx[2], c.z);
+    mn[3] = min(mn[3], c.w); mx[3] = max(mx[3], c.w);
+  }
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+      mn[d] = min(mn[d], __shfl_xor(mn[d], s, 64));
+      mx[d] = max(mx[d], __shfl_xor(mx[d], s, 64));
+    }
+  }
+  const int wave = threadIdx.x >> 6;
+  if (wcn_lane() == 0) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      s_mn[wave][d] = mn[d];
+      s_mx[wave][d] = mx[d];
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 4) {
+    const int d = threadIdx.x;
+    int a = s_mn[0][d], b = s_mx[0][d];
+    for (int w = 1; w < 4; ++w) {
+      a = min(a, s_mn[w][d]);
+      b = max(b, s_mx[w][d]);
+    }
+    atomicMin(&hdr->mn[d], a);
+    atomicMax(&hdr->mx[d], b);
+  }
+}
+
+__global__ void __launch_bounds__(256) table_insert(const int4* __restrict__ keys, int64_t n_keys,
+                                                    WcnTableHeader* __restrict__ hdr,
+                                                    WcnSlot* __restrict__ slots, uint32_t cap_mask,
+                                                    int32_t* __restrict__ slot_of,
+                                                    int32_t* __restrict__ block_list,
+                                                    int64_t block_list_len) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_keys) return;
+  const WcnLayout L = wcn_make_layout(hdr);
+  if (!L.ok) {
+    if (i == 0) atomicOr(&hdr->status, WCN_DEV_RANGE);
+    slot_of[i] = -1;
+    return;
+  }
+  const int4 c = keys[i];
+  uint32_t r[4];
+  wcn_relative(L, c.x, c.y, c.z, c.w, r);  // always inside: the box was built from these keys
+  const unsigned long long key = wcn_block_key(L, r);
+  const unsigned long long bit = 1ull << wcn_block_bit(r);
+  uint32_t h = wcn_mix(key, cap_mask);
+  int32_t placed = -1;
+  for (int p = 0; p < WCN_MAX_PROBE; ++p) {
+    // cheap pre-read: most keys find their block already present
+    unsigned long long seen = __atomic_load_n(&slots[h].key, __ATOMIC_RELAXED);
+    if (seen == WCN_EMPTY_KEY) {
+      seen = atomicCAS(&slots[h].key, WCN_EMPTY_KEY, key);
+      if (seen == WCN_EMPTY_KEY) {
+        const int32_t at = atomicAdd(&hdr->num_blocks, 1);
+        if (at < block_list_len) block_list[at] = (int32_t)h;
+        seen = key;
+      }
+    }
+    if (seen == key) {
+      atomicOr(&slots[h].mask, bit);
+      placed = (int32_t)h;
+      break;
+    }
+    h = (h + 1) & cap_mask;
+  }
+  if (placed < 0) atomicOr(&hdr->status, WCN_DEV_OVERFLOW);
+  slot_of[i] = placed;
+}
+
+__global__ void __launch_bounds__(256) table_base(WcnTableHeader* __restrict__ hdr,
+                                                  WcnSlot* __restrict__ slots,
+                                                  const int32_t* __restrict__ block_list,
+                                                  int64_t block_list_len) {
+  const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t nb = hdr->num_blocks;
+  if (nb > block_list_len) nb = block_list_len;
+  // whole waves leave together: the prefix sum below needs every lane of a live wave
+  if ((j & ~(int64_t)63) >= nb) return;
+  int32_t h = -1, cnt = 0;
+  if (j < nb) {
+    h = block_list[j];
+    cnt = __popcll(slots[h].mask);
+  }
+  const int incl = wcn_wave_inclusive_sum(cnt);
+  int wave_base = 0;
+  if (wcn_lane() == 63) wave_base = atomicAdd(&hdr->total, incl);
+  wave_base = __shfl(wave_base, 63, 64);
+  if (h >= 0) slots[h].base = wave_base + incl - cnt;
+}
+
+__global__ void __launch_bounds__(256) table_perm(const int4* __restrict__ keys, int64_t n_keys,
+                                                  const WcnTableHeader* __restrict__ hdr,
+                                                  const WcnSlot* __restrict__ slots,
+                                                  const int32_t* __restrict__ slot_of,
+                                                  int32_t* __restrict__ perm) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_keys) return;
+  const int32_t h = slot_of[i];
+  if (h < 0) return;
+  const WcnLayout L = wcn_make_layout(hdr);
+  const int4 c = keys[i];
+  uint32_t r[4];
+  wcn_relative(L, c.x, c.y, c.z, c.w, r);
+  const ulonglong2 km = *reinterpret_cast<const ulonglong2*>(&slots[h]);
+  const int32_t pos = slots[h].base + wcn_rank_below(km.y, wcn_block_bit(r));
+  if (pos >= 0 && pos < n_keys) atomicMin(&perm[pos], (int32_t)i);
+}
+
+__global__ void __launch_bounds__(256) table_query(const WcnTableHeader* __restrict__ hdr,
+                                                   const WcnSlot* __restrict__ slots,
+                                                   uint32_t cap_mask,
+                                                   const int32_t* __restrict__ perm,
+                                                   const int4* __restrict__ queries,
+                                                   int64_t num_queries,
+                                                   int32_t* __restrict__ results) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= num_queries) return;
+  const WcnLayout L = wcn_make_layout(hdr);
+  const int4 c = queries[i];
+  uint32_t r[4];
+  int32_t res = -1;
+  if (L.ok && wcn_relative(L, c.x, c.y, c.z, c.w, r)) {
+    int32_t base;
+    const unsigned long long mask = wcn_lookup_block(slots, cap_mask, wcn_block_key(L, r), &base);
+    const uint32_t bit = wcn_block_bit(r);
+    if ((mask >> bit) & 1ull) res = perm[base + wcn_rank_below(mask, bit)];
+  }
+  results[i] = res;
+}
+
+inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
+
+inline int grid_for(int64_t n, int block, int cap = 1 << 20) {
+  int64_t g = (n + block - 1) / block;
+  if (g < 1) g = 1;
+  if (g > cap) g = cap;
+  return (int)g;
+}
+
+}  // namespace
+
+// Enqueue the five build kernels.  Shared with the strided-coordinate path.
+int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView& v,
+                         hipStream_t s) {
+  const uint32_t cap_mask = (uint32_t)(v.capacity - 1);
+  const int64_t list_len = v.capacity < n_keys ? v.capacity : n_keys;
+  const int64_t clear_items = 2 * v.capacity > n_keys ? 2 * v.capacity : n_keys;
+  hipLaunchKernelGGL(table_clear, dim3(grid_for(clear_items, 256, 4096)), dim3(256), 0, s, v.hdr,
+                     v.slots, v.capacity, v.perm, n_keys);
+  if (n_keys > 0) {
+    hipLaunchKernelGGL(table_bbox, dim3(grid_for(n_keys, 256 * 8, 2048)), dim3(256), 0, s,
+                       (const int4*)keys, n_keys, v.hdr);
+    hipLaunchKernelGGL(table_insert, dim3(grid_for(n_keys, 256)), dim3(256), 0, s,
+                       (const int4*)keys, n_keys, v.hdr, v.slots, cap_mask, v.slot_of,
+                       v.block_list, list_len);
+    hipLaunchKernelGGL(table_base, dim3(grid_for(list_len, 256)), dim3(256), 0, s, v.hdr, v.slots,
+                       v.block_list, list_len);
+    hipLaunchKernelGGL(table_perm, dim3(grid_for(n_keys, 256)), dim3(256), 0, s,
+                       (const int4*)keys, n_keys, v.hdr, v.slots, v.slot_of, v.perm);
+  }
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+int wcn_table_status_from_bits(int32_t bits) {
+  if (bits & WCN_DEV_RANGE) return WCN_ERR_COORD_RANGE;
+  if (bits & WCN_DEV_OVERFLOW) return WCN_ERR_TABLE_OVERFLOW;
+  return WCN_OK;
+}
+
+extern "C" {
+
+int wcn_version(void) { return 100; }
+
+const char* wcn_status_string(int status) {
+  switch (status) {
+    case WCN_OK: return "success";
+    case WCN_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case WCN_ERR_LAUNCH: return "HIP launch or copy failed";
+    case WCN_ERR_TABLE_OVERFLOW: return "coordinate table probe limit exceeded (capacity too small)";
+    case WCN_ERR_COORD_RANGE: return "coordinate bounding box does not fit the 63-bit block key";
+    case WCN_ERR_TOO_MANY_PAIRS: return "kernel map exceeds 2^31-1 pairs";
+    case WCN_ERR_WORKSPACE: return "workspace too small";
+    default: return "unknown status";
+  }
+}
+
+int64_t wcn_table_default_capacity(int64_t n_keys) {
+  // Blocks hold up to 64 voxels; surface-like data fills ~10 per block.  One slot per two keys
+  // keeps the load factor under 0.5 unless almost every voxel is alone in its block, in which
+  // case the build reports WCN_ERR_TABLE_OVERFLOW and the caller retries with 4x the slots.
+  int64_t want = n_keys / 2 + 1;
+  int64_t cap = 1024;
+  while (cap < want) cap <<= 1;
+  return cap;
+}
+
+size_t wcn_table_bytes(int64_t n_keys, int64_t capacity) {
+  if (n_keys < 0 || capacity <= 0) return 0;
+  return wcn_table_layout(nullptr, n_keys, capacity, nullptr);
+}
+
+int wcn_table_build(const int32_t* keys, int64_t n_keys, void* table, int64_t capacity,
+                    void* stream) {
+  if (!table || n_keys < 0 || (n_keys > 0 && !keys)) return WCN_ERR_INVALID_ARGUMENT;
+  if (!is_pow2(capacity) || capacity < 64 || capacity > (1ll << 31)) return WCN_ERR_INVALID_ARGUMENT;
+  if (n_keys >= (1ll << 31)) return WCN_ERR_INVALID_ARGUMENT;
+  WcnTableView v;
+  wcn_table_layout(table, n_keys, capacity, &v);
+  return wcn_table_build_impl(keys, n_keys, v, (hipStream_t)stream);
+}
+
+int wcn_table_query(const void* table, int64_t n_keys, int64_t capacity, const int32_t* queries,
+                    int64_t num_queries, int32_t* results, void* stream) {
+  if (!table || num_queries < 0 || (num_queries > 0 && (!queries || !results)))
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (!is_pow2(capacity) || capacity < 64 || n_keys < 0) return WCN_ERR_INVALID_ARGUMENT;
+  if (num_queries == 0) return WCN_OK;
+  WcnTableView v;
+  wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
+  hipLaunchKernelGGL(table_query, dim3(grid_for(num_queries, 256)), dim3(256), 0,
+                     (hipStream_t)stream, v.hdr, v.slots, (uint32_t)(capacity - 1), v.perm,
+                     (const int4*)queries, num_queries, results);
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+int wcn_table_read_status(const void* table, int32_t* host_num_blocks, void* stream) {
+  if (!table) return WCN_ERR_INVALID_ARGUMENT;
+  WcnTableHeader h;
+  if (hipMemcpyAsync(&h, table, sizeof(h), hipMemcpyDeviceToHost, (hipStream_t)stream) !=
+      hipSuccess)
+    return WCN_ERR_LAUNCH;
+  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return WCN_ERR_LAUNCH;
+  if (host_num_blocks) *host_num_blocks = h.num_blocks;
+  return wcn_table_status_from_bits(h.status);
+}
+
+}  // extern "C"

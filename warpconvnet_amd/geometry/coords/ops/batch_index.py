@@ -1,0 +1,26 @@
+"""Batch index / offsets conversions (reference: warpconvnet/geometry/coords/ops/batch_index.py)."""
+import torch
+from torch import Tensor
+
+
+@torch.no_grad()
+def batch_index_from_offset(offsets: Tensor) -> Tensor:
+    """[0,2,5] -> [0,0,1,1,1] (reference: batch_index.py:22-36)."""
+    assert len(offsets) > 1, "offsets must have at least two elements. [0, N] for batch size 1"
+    counts = torch.diff(offsets)
+    return torch.arange(len(counts), device=offsets.device, dtype=torch.long).repeat_interleave(counts)
+
+
+@torch.no_grad()
+def batch_indexed_coordinates(batched_coords: Tensor, offsets: Tensor) -> Tensor:
+    """(N, D) coordinates -> (N, D+1) rows [batch, ...] in the coordinate dtype and device
+    (reference: batch_index.py:110-117)."""
+    batch_index = batch_index_from_offset(offsets).to(batched_coords)
+    return torch.cat([batch_index.unsqueeze(1), batched_coords], dim=1)
+
+
+@torch.no_grad()
+def offsets_from_batch_index(batch_index: Tensor) -> Tensor:
+    """[0,0,1,1,2,2,2,3,3] -> [0,2,4,7,9] on the CPU (reference: batch_index.py:143-161)."""
+    counts = torch.bincount(batch_index).cpu()
+    return torch.cat([torch.zeros(1, dtype=torch.int32), counts.cumsum(dim=0)], dim=0)

@@ -1,0 +1,59 @@
+"""Strided (down-sampled) output coordinates (reference:
+warpconvnet/geometry/coords/ops/stride.py:17-54 and warpconvnet/utils/unique.py:125-144)."""
+import ctypes
+from typing import Tuple
+
+import torch
+from torch import Tensor
+
+from ...._lib import ERR_TABLE_OVERFLOW, check, int3, lib, ptr, stream_ptr, workspace
+from ....utils.ntuple import ntuple
+from .batch_index import offsets_from_batch_index
+from ..search.torch_hashmap import _four_columns
+
+
+@torch.no_grad()
+def stride_coords(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
+                  order="random") -> Tuple[Tensor, Tensor]:
+    """Unique rows of floor(coords / [1, *stride]) and their batch offsets.
+
+    One call into the HIP library (floor division, table build over the coarse rows, selection of
+    the lowest source row per coarse voxel, order-preserving compaction) and one host read for the
+    row count.  Output rows ascend in their representative's source row, so a batch-sorted input
+    yields a batch-sorted output (the reference sorts by batch afterwards, stride.py:44-48, with an
+    order inside a batch that depends on a thread race; as sets the results are identical).
+    Only the reference's default ordering is built.
+    """
+    num_spatial_dims = batch_indexed_coords.shape[1] - 1
+    assert len(stride) == num_spatial_dims, \
+        (f"Stride must match the number of spatial dimensions. Got {len(stride)} spatial "
+         f"dimensions for but coordinates with {num_spatial_dims} spatial dimensions.")
+    if str(getattr(order, "value", order)).lower() != "random":
+        raise NotImplementedError("only the default (unordered) output ordering is built")
+    if all(s == 1 for s in stride):
+        return batch_indexed_coords, offsets_from_batch_index(batch_indexed_coords[:, 0])
+    assert batch_indexed_coords.dtype == torch.int32
+    device = batch_indexed_coords.device
+    coords = _four_columns(batch_indexed_coords)
+    n = coords.shape[0]
+    L = lib()
+    st = int3(list(ntuple(stride, ndim=num_spatial_dims)) + [1] * (3 - num_spatial_dims))
+    out = torch.empty((n, 4), dtype=torch.int32, device=device)
+    first = torch.empty(n, dtype=torch.int32, device=device)
+    slots = L.wcn_table_default_capacity(n)
+    count = ctypes.c_int64(0)
+    while True:
+        ws = workspace(L.wcn_stride_unique_workspace_bytes(n, slots), device)
+        check(L.wcn_stride_unique(ptr(coords), n, st, ptr(ws), slots, ptr(out), ptr(first),
+                                  stream_ptr(device)), "wcn_stride_unique")
+        status = L.wcn_stride_unique_read_count(ptr(ws), n, slots, ctypes.byref(count),
+                                                stream_ptr(device))
+        if status == ERR_TABLE_OVERFLOW and slots < (1 << 30):
+            slots *= 4
+            continue
+        check(status, "wcn_stride_unique")
+        break
+    unique_coords = out[: count.value, : num_spatial_dims + 1]
+    if num_spatial_dims != 3:
+        unique_coords = unique_coords.contiguous()
+    return unique_coords, offsets_from_batch_index(unique_coords[:, 0])

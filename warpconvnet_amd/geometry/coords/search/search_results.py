@@ -1,0 +1,86 @@
+"""Kernel-map container (reference: warpconvnet/geometry/coords/search/search_results.py:54-174).
+
+Pairs of all kernel offsets are stored flat: offset k owns in_maps[offsets[k]:offsets[k+1]] and
+the matching out_maps slice; offsets live on the CPU.
+"""
+from typing import List, Literal, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+
+class IntSearchResult:
+    in_maps: Tensor
+    out_maps: Tensor
+    offsets: Tensor
+    identity_map_index: Optional[int]
+
+    def __init__(self, in_maps: Tensor, out_maps: Tensor, offsets: Tensor,
+                 identity_map_index: Optional[int] = None):
+        offsets = offsets.cpu()
+        assert len(in_maps) == len(out_maps) == int(offsets[-1])
+        self.in_maps = in_maps
+        self.out_maps = out_maps
+        self.offsets = offsets
+        self.identity_map_index = identity_map_index
+        # Device-side helpers of the HIP contraction (not part of the reference interface):
+        # whether out_maps ascends inside every offset, and the per-64-row group starts the map
+        # builder produced as a by-product (None: the contraction derives them itself).
+        self._out_sorted: Optional[bool] = None
+        self._group_start: Optional[Tensor] = None
+        self._sorted_view: Optional["IntSearchResult"] = None
+
+    @torch.no_grad()
+    def __getitem__(self, idx: int) -> Tuple[Tensor, Tensor]:
+        start, end = int(self.offsets[idx]), int(self.offsets[idx + 1])
+        return self.in_maps[start:end], self.out_maps[start:end]
+
+    def __len__(self) -> int:
+        return len(self.offsets) - 1
+
+    def __iter__(self):
+        for i in range(len(self)):
+            yield self[i]
+
+    def numel(self, i: int) -> int:
+        return int(self.offsets[i + 1] - self.offsets[i])
+
+    @torch.no_grad()
+    def get_batch(self, start_idx: int, end_idx: int,
+                  out_format: Literal["list", "tensor"] = "list"):
+        ins: List[Tensor] = []
+        outs: List[Tensor] = []
+        for i in range(start_idx, end_idx):
+            a, b = self[i]
+            ins.append(a)
+            outs.append(b)
+        if out_format == "list":
+            return ins, outs
+        if out_format != "tensor":
+            raise ValueError(f"Invalid output format: {out_format}")
+        width = max(len(a) for a in ins)
+        in_t = torch.full((len(ins), width), -1, dtype=torch.int64, device=self.in_maps.device)
+        out_t = torch.full((len(outs), width), -1, dtype=torch.int64, device=self.out_maps.device)
+        for i, (a, b) in enumerate(zip(ins, outs)):
+            in_t[i, :len(a)] = a
+            out_t[i, :len(b)] = b
+        return in_t, out_t
+
+    @torch.no_grad()
+    def to_csr(self) -> Tuple[Tensor, Tensor, Tensor]:
+        """(in indices sorted by out index, unique out indices, CPU row offsets)."""
+        out_sorted, order = torch.sort(self.out_maps)
+        unique_out, counts = torch.unique(out_sorted, return_counts=True, sorted=True)
+        offsets = torch.cat([torch.zeros(1, dtype=torch.int32), torch.cumsum(counts.cpu(), dim=0)])
+        return self.in_maps[order], unique_out, offsets
+
+    def clone(self) -> "IntSearchResult":
+        return IntSearchResult(self.in_maps.clone(), self.out_maps.clone(), self.offsets.clone(),
+                               self.identity_map_index)
+
+    @property
+    def device(self):
+        return self.in_maps.device
+
+    def __repr__(self) -> str:
+        return f"{self.__class__.__name__}(len={len(self)}, iden_map={self.identity_map_index})"

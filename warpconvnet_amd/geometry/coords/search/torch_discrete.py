@@ -1,0 +1,154 @@
+"""Kernel-map generation (reference: warpconvnet/geometry/coords/search/torch_discrete.py).
+
+`generate_kernel_map` keeps the reference signature and result type.  The device work is two
+calls into the HIP library with a single host read between them:
+
+    wcn_table_build (enqueued, not awaited)
+    wcn_kmap_count  (probes + per-offset counts + prefix sums, enqueued)
+    wcn_kmap_read_result  <- the only wait: offsets[K+1] and the table status
+    wcn_kmap_fill   (writes in_maps / out_maps in the reference's order)
+
+where the reference waits five times and round-trips a dense (K, M) table through HBM
+(torch_discrete.py:80-157,301-337).
+"""
+import ctypes
+from typing import Literal, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+from torch import Tensor
+
+from ...._lib import ERR_TABLE_OVERFLOW, check, int3, lib, ptr, stream_ptr, workspace
+from ....utils.ntuple import ntuple
+from .search_results import IntSearchResult
+from .torch_hashmap import HashMethod, TorchHashTable, _four_columns
+
+
+@torch.no_grad()
+def kernel_offsets_from_size(kernel_size: Tuple[int, ...], kernel_dilation: Tuple[int, ...],
+                             center_offset: Optional[Tuple[int, ...]] = None,
+                             device="cpu") -> Tensor:
+    """(K, D+1) int32 offsets, batch column 0, last spatial dimension fastest, centre (s-1)//2
+    for odd sizes and 0 for even ones, scaled by the dilation (reference: torch_discrete.py:44-77)."""
+    assert len(kernel_size) == len(kernel_dilation)
+    axes = []
+    for d, (size, dil) in enumerate(zip(kernel_size, kernel_dilation)):
+        centre = (size - 1) // 2 if size % 2 == 1 else 0
+        if center_offset is not None:
+            centre = centre + center_offset[d]
+        axes.append((torch.arange(size, dtype=torch.int32) - centre) * dil)
+    grid = torch.meshgrid(*axes, indexing="ij")
+    spatial = torch.stack([g.reshape(-1) for g in grid], dim=1)
+    batch = torch.zeros(spatial.shape[0], 1, dtype=torch.int32)
+    return torch.cat([batch, spatial], dim=1).to(device)
+
+
+def _pad_kernel_args(values: Sequence[int], fill: int):
+    """The device kernels are written for three spatial dimensions; lower-dimensional problems
+    run with size-1 / stride-1 trailing dimensions."""
+    values = [int(v) for v in values]
+    return values + [fill] * (3 - len(values))
+
+
+@torch.no_grad()
+def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_size, stride,
+                           identity_map_index: Optional[int]) -> IntSearchResult:
+    """Count, read the offsets, fill.  Handles the device-reported table overflow by rebuilding
+    the table with more slots and starting over."""
+    device = out_coords.device
+    L = lib()
+    ks, st = int3(_pad_kernel_args(kernel_size, 1)), int3(_pad_kernel_args(stride, 1))
+    K = int(np.prod([int(k) for k in kernel_size]))
+    out4 = _four_columns(out_coords)
+    M = out4.shape[0]
+    ws = workspace(L.wcn_kmap_workspace_bytes(M, K), device)
+    host_offsets = (ctypes.c_int64 * (K + 1))()
+    while True:
+        raw, n_keys, slots = table._raw()
+        check(L.wcn_kmap_count(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws),
+                               stream_ptr(device)), "wcn_kmap_count")
+        status = L.wcn_kmap_read_result(ptr(ws), M, K, host_offsets, stream_ptr(device))
+        if status == ERR_TABLE_OVERFLOW:
+            table._grow()
+            continue
+        check(status, "wcn_kmap_count")
+        table._checked = True
+        break
+    total = int(host_offsets[K])
+    in_maps = torch.empty(total, dtype=torch.int32, device=device)
+    out_maps = torch.empty(total, dtype=torch.int32, device=device)
+    check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), ptr(in_maps),
+                          ptr(out_maps), stream_ptr(device)), "wcn_kmap_fill")
+    offsets = torch.tensor(list(host_offsets), dtype=torch.int32)
+    result = IntSearchResult(in_maps, out_maps, offsets, identity_map_index=identity_map_index)
+    # by-products the contraction can reuse: pairs ascend in out index inside every offset, and
+    # the workspace holds the per-64-row group starts (kept alive by the reference below)
+    result._out_sorted = True
+    result._group_start = ws
+    result._group_start_ptr = L.wcn_kmap_group_start(ptr(ws), M, K)
+    result._group_start_shape = (K, M)
+    return result
+
+
+@torch.no_grad()
+def generate_kernel_map(
+    batch_indexed_in_coords: Tensor,
+    batch_indexed_out_coords: Tensor,
+    in_to_out_stride_ratio: Tuple[int, ...],
+    kernel_size: Tuple[int, ...],
+    kernel_dilation: Optional[Tuple[int, ...]] = None,
+    kernel_center_offset: Optional[Tuple[int, ...]] = None,
+    method: Literal["offset", "size"] = "size",
+    hash_method: HashMethod = HashMethod.CITY,
+    skip_symmetric_kernel_map: bool = False,
+) -> IntSearchResult:
+    """Kernel map between input and output coordinates (reference: torch_discrete.py:365-466).
+
+    For every kernel offset k (enumerated with the last spatial dimension fastest) and output
+    row m, the query out[m] * [1, stride] + offset_k is looked up among the inputs; hits become
+    pairs (in index, m) stored per offset in ascending m.  `identity_map_index` is K // 2 iff all
+    kernel sizes are odd and the input and output row counts agree.
+    """
+    device = batch_indexed_in_coords.device
+    assert device == batch_indexed_out_coords.device
+    assert batch_indexed_in_coords.dtype == torch.int32
+    assert batch_indexed_out_coords.dtype == torch.int32
+    if skip_symmetric_kernel_map:
+        assert len(batch_indexed_in_coords) == len(batch_indexed_out_coords), \
+            "You can only skip symmetric kernel map if the input and output coordinates are the same."
+        assert all(k % 2 == 1 for k in kernel_size), "Kernel size must be odd for symmetric skipping."
+    num_spatial_dims = batch_indexed_out_coords.shape[1] - 1
+    assert len(in_to_out_stride_ratio) == num_spatial_dims
+    assert len(kernel_size) == num_spatial_dims
+    if method not in ("size", "offset"):
+        raise ValueError(f"Invalid method: {method}. Choose 'query', 'offset', or 'size'.")
+    if method == "size":
+        assert kernel_dilation is None or all(s == 1 for s in kernel_dilation), \
+            "Kernel dilation is not supported with method='size'. Use method='offset' instead."
+        assert kernel_center_offset is None, \
+            "Custom kernel_center_offset is not supported with method='size'. Use method='offset' instead."
+    elif (kernel_dilation is not None and any(s != 1 for s in kernel_dilation)) \
+            or kernel_center_offset is not None:
+        raise NotImplementedError("dilated or re-centred kernels are not built on this path")
+    if num_spatial_dims > 3:
+        raise NotImplementedError("more than 3 spatial dimensions are not supported")
+
+    table = TorchHashTable.from_keys(batch_indexed_in_coords, hash_method=hash_method,
+                                     device=device, _defer_check=True)
+
+    is_odd = all(k % 2 == 1 for k in kernel_size)
+    same_count = batch_indexed_in_coords.shape[0] == batch_indexed_out_coords.shape[0]
+    identity_map_index = int(np.prod(kernel_size)) // 2 if (is_odd and same_count) else None
+
+    stride = ntuple(in_to_out_stride_ratio, ndim=num_spatial_dims)
+    result = _kernel_map_from_table(table, batch_indexed_out_coords, kernel_size, stride,
+                                    identity_map_index)
+    if skip_symmetric_kernel_map and is_odd:
+        # only the offsets before the centre are kept (torch_discrete.py:286-296)
+        half = int(np.prod(kernel_size)) // 2
+        end = int(result.offsets[half])
+        result = IntSearchResult(result.in_maps[:end], result.out_maps[:end],
+                                 result.offsets[: half + 1].clone(),
+                                 identity_map_index=identity_map_index)
+        result._out_sorted = True
+    return result

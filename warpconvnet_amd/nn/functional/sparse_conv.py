@@ -1,0 +1,354 @@
+"""Functional sparse convolution (reference: warpconvnet/nn/functional/sparse_conv.py).
+
+`spatially_sparse_conv` keeps the reference signature and bookkeeping (1x1 shortcut, tensor
+stride arithmetic, kernel-map cache with the transposed in/out swap, bias, output Voxels) and
+sends the three device stages to the HIP library: output coordinates (`stride_coords`), kernel
+map (`generate_kernel_map`) and the feature contraction (`wcn_sparse_conv_fwd`, one launch
+sequence for all kernel offsets, fp32 accumulation, one rounding).
+
+There is a single contraction algorithm; the `fwd_algo` / `bwd_algo` / block-size arguments of
+the reference are accepted for call compatibility and do not select anything.  The backward pass
+of the autograd Function is expressed with torch operations over the same kernel map
+(reference: sparse_conv.py:314-355).
+"""
+import ctypes
+import enum
+import os
+from typing import List, Optional, Tuple, Union
+
+import numpy as np
+import torch
+from torch import Tensor
+from torch.autograd import Function
+
+from ..._lib import DTYPE_CODE, check, lib, ptr, require_device, stream_ptr, workspace
+from ...geometry.coords.integer import IntCoords
+from ...geometry.coords.ops.stride import stride_coords
+from ...geometry.coords.search.cache import IntSearchCache, IntSearchCacheKey
+from ...geometry.coords.search.search_results import IntSearchResult
+from ...geometry.coords.search.torch_discrete import generate_kernel_map
+from ...geometry.types.voxels import Voxels
+from ...utils.ntuple import ntuple
+
+
+class STRIDED_CONV_MODE(enum.Enum):
+    REDUCE_AND_STRIDE = "reduce_and_stride"  # pooling before the convolution: not built
+    STRIDE_ONLY = "stride_only"
+
+
+class SPARSE_CONV_FWD_ALGO_MODE(enum.Enum):
+    EXPLICIT_GEMM = "explicit_gemm"
+    IMPLICIT_GEMM = "implicit_gemm"
+    CUTLASS_IMPLICIT_GEMM = "cutlass_implicit_gemm"
+    AUTO = "auto"
+
+
+class SPARSE_CONV_BWD_ALGO_MODE(enum.Enum):
+    EXPLICIT_GEMM = "explicit_gemm"
+    IMPLICIT_GEMM = "implicit_gemm"
+    CUTLASS_IMPLICIT_GEMM = "cutlass_implicit_gemm"
+    AUTO = "auto"
+
+
+class POINT_ORDERING(enum.Enum):
+    RANDOM = "random"
+    MORTON_XYZ = "morton_xyz"
+
+
+def _is_random_order(order) -> bool:
+    return str(getattr(order, "value", order)).lower() == "random"
+
+
+# ------------------------------------------------------------------------------------------------
+# Feature contraction
+# ------------------------------------------------------------------------------------------------
+
+@torch.no_grad()
+def _sorted_by_out(kernel_map: IntSearchResult) -> IntSearchResult:
+    """A view of the map whose pairs ascend in out index inside every offset (what the device
+    contraction needs).  Maps from `generate_kernel_map` already do; the in/out-swapped map of a
+    transposed convolution does not and is reordered once, then cached on the map."""
+    if kernel_map._out_sorted:
+        return kernel_map
+    if kernel_map._sorted_view is not None:
+        return kernel_map._sorted_view
+    K = len(kernel_map)
+    offs = kernel_map.offsets.to(torch.int64)
+    counts = (offs[1:] - offs[:-1]).to(kernel_map.out_maps.device)
+    which = torch.repeat_interleave(torch.arange(K, device=counts.device), counts)
+    bound = int(kernel_map.out_maps.max().item()) + 1 if kernel_map.out_maps.numel() else 1
+    order = torch.argsort(which * bound + kernel_map.out_maps.long())
+    view = IntSearchResult(kernel_map.in_maps[order].contiguous(),
+                           kernel_map.out_maps[order].contiguous(), kernel_map.offsets,
+                           kernel_map.identity_map_index)
+    view._out_sorted = True
+    kernel_map._sorted_view = view
+    return view
+
+
+@torch.no_grad()
+def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSearchResult,
+                        num_out_coords: int, bias: Optional[Tensor] = None,
+                        compute_dtype: Optional[torch.dtype] = None) -> Tensor:
+    """out = bias + sum_k scatter(X[in_k] @ W[k]) on the GPU (replaces the per-offset loops of
+    sparse_conv.py:281-311 / :358-415 / :495-544 and the native GEMMs they call)."""
+    require_device(in_features, "in_features")
+    if in_features.ndim != 2 or weight.ndim != 3 or weight.shape[1] != in_features.shape[1]:
+        raise ValueError(f"shape mismatch: features {tuple(in_features.shape)}, "
+                         f"weight {tuple(weight.shape)}")
+    if len(kernel_map) != weight.shape[0]:
+        raise ValueError(f"kernel map has {len(kernel_map)} offsets, weight has {weight.shape[0]}")
+    x = in_features if compute_dtype is None else in_features.to(compute_dtype)
+    if x.dtype not in DTYPE_CODE:
+        raise TypeError(f"unsupported feature dtype {x.dtype}")
+    x = x.contiguous()
+    w = weight.detach()
+    if w.dtype != x.dtype and w.dtype != torch.float32:
+        w = w.to(x.dtype)
+    w = w.contiguous()
+    b = None if bias is None else bias.detach().to(x.dtype).contiguous()
+    km = _sorted_by_out(kernel_map)
+    K, c_in, c_out = w.shape
+    device = x.device
+    out = torch.empty((num_out_coords, c_out), dtype=x.dtype, device=device)
+    L = lib()
+    nbytes = L.wcn_conv_workspace_bytes(num_out_coords, K, c_in, c_out, DTYPE_CODE[x.dtype])
+    ws = workspace(nbytes, device)
+    host_offsets = (ctypes.c_int64 * (K + 1))(*[int(v) for v in km.offsets.tolist()])
+    group_start = None
+    if getattr(km, "_group_start", None) is not None and \
+            getattr(km, "_group_start_shape", None) == (K, num_out_coords):
+        group_start = ctypes.c_void_p(km._group_start_ptr)
+    iden = -1 if km.identity_map_index is None else int(km.identity_map_index)
+    check(L.wcn_sparse_conv_fwd(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(w),
+                                DTYPE_CODE[w.dtype], K, c_out, ptr(b), ptr(km.in_maps),
+                                ptr(km.out_maps), host_offsets, iden, group_start, ptr(out),
+                                num_out_coords, ptr(ws), ws.numel(), stream_ptr(device)),
+          "wcn_sparse_conv_fwd")
+    return out if out.dtype == in_features.dtype else out.to(in_features.dtype)
+
+
+def _explicit_gemm_backward_logic(grad_output: Tensor, in_features: Tensor, weight: Tensor,
+                                  kernel_map: IntSearchResult,
+                                  compute_dtype: Optional[torch.dtype]):
+    """Gradients with torch operations over the kernel map (reference: sparse_conv.py:314-355):
+    dX[in_k] += dY[out_k] @ W[k]^T ;  dW[k] = X[in_k]^T @ dY[out_k]."""
+    dtype = compute_dtype or in_features.dtype
+    x = in_features.to(dtype)
+    w = weight.to(dtype)
+    gy = grad_output.to(dtype)
+    grad_x = torch.zeros_like(x)
+    grad_w = torch.zeros_like(w)
+    iden = kernel_map.identity_map_index
+    if iden is not None:
+        grad_x += gy @ w[iden].T
+        grad_w[iden] = x.T @ gy
+    for k in range(len(kernel_map)):
+        if k == iden:
+            continue
+        in_map, out_map = kernel_map[k]
+        if in_map.numel() == 0:
+            continue
+        in_map, out_map = in_map.long(), out_map.long()
+        g = gy[out_map]
+        grad_x.index_add_(0, in_map, g @ w[k].T)
+        grad_w[k] = x[in_map].T @ g
+    return grad_x.to(in_features.dtype), grad_w.to(weight.dtype)
+
+
+class UnifiedSpatiallySparseConvFunction(Function):
+    """autograd wrapper with the reference's argument list (sparse_conv.py:1321-1482).  The
+    algorithm and block-size arguments are accepted and ignored."""
+
+    @staticmethod
+    def forward(ctx, in_features, weight, kernel_map, num_out_coords, fwd_algo=None, bwd_algo=None,
+                compute_dtype=None, fwd_block_size=None, bwd_block_size=None):
+        if num_out_coords == 0 or in_features.shape[0] == 0:
+            out = torch.zeros((num_out_coords, weight.shape[-1]), dtype=in_features.dtype,
+                              device=in_features.device)
+        else:
+            out = sparse_conv_forward(in_features, weight, kernel_map, num_out_coords,
+                                      compute_dtype=compute_dtype)
+        ctx.save_for_backward(in_features, weight)
+        ctx.kernel_map = kernel_map
+        ctx.compute_dtype = compute_dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        in_features, weight = ctx.saved_tensors
+        grad_x, grad_w = _explicit_gemm_backward_logic(grad_output, in_features, weight,
+                                                       ctx.kernel_map, ctx.compute_dtype)
+        if not ctx.needs_input_grad[0]:
+            grad_x = None
+        if not ctx.needs_input_grad[1]:
+            grad_w = None
+        return grad_x, grad_w, None, None, None, None, None, None, None
+
+
+SpatiallySparseConvExplicitGEMMFunction = UnifiedSpatiallySparseConvFunction
+
+
+# ------------------------------------------------------------------------------------------------
+# Output coordinates and kernel map
+# ------------------------------------------------------------------------------------------------
+
+def generate_output_coords_and_kernel_map(
+    input_sparse_tensor: Voxels,
+    kernel_size: Tuple[int, ...],
+    kernel_dilation: Tuple[int, ...],
+    stride: Tuple[int, ...],
+    generative: bool,
+    transposed: bool,
+    output_spatially_sparse_tensor: Optional[Voxels],
+    stride_mode: STRIDED_CONV_MODE = STRIDED_CONV_MODE.STRIDE_ONLY,
+    order=POINT_ORDERING.RANDOM,
+) -> Tuple[Tensor, Tensor, IntSearchResult]:
+    """Output coordinates (given / strided / same as input), then the kernel map, through the
+    cache on the input tensor (reference: sparse_conv.py:1808-1996).  A transposed convolution
+    reuses the cached forward map of the matching strided convolution with in/out exchanged."""
+    if generative:
+        raise NotImplementedError("generative convolutions (coordinate expansion) are not built")
+    if stride_mode != STRIDED_CONV_MODE.STRIDE_ONLY:
+        raise NotImplementedError("only STRIDED_CONV_MODE.STRIDE_ONLY is built")
+    if not _is_random_order(order):
+        raise NotImplementedError("only the default (unordered) output ordering is built")
+    in_coords = input_sparse_tensor.batch_indexed_coordinates
+
+    if output_spatially_sparse_tensor is not None:
+        out_coords = output_spatially_sparse_tensor.batch_indexed_coordinates
+        out_offsets = output_spatially_sparse_tensor.offsets
+    elif any(s != 1 for s in stride):
+        out_coords, out_offsets = stride_coords(in_coords, stride)
+    else:
+        out_coords, out_offsets = in_coords, input_sparse_tensor.offsets
+
+    def make_key(is_transposed, in_off, out_off):
+        return IntSearchCacheKey(kernel_size=kernel_size, kernel_dilation=kernel_dilation,
+                                 transposed=is_transposed, generative=generative,
+                                 stride_mode=str(stride_mode), skip_symmetric_kernel_map=False,
+                                 in_offsets=in_off, out_offsets=out_off)
+
+    key = make_key(transposed, input_sparse_tensor.offsets, out_offsets)
+    cache = input_sparse_tensor.cache
+    if cache is not None:
+        kernel_map = cache.get(key)
+        if kernel_map is not None:
+            return out_coords, out_offsets, kernel_map
+
+    if transposed:
+        forward_map = None
+        if cache is not None:
+            forward_map = cache.get(make_key(False, out_offsets, input_sparse_tensor.offsets))
+        if forward_map is None:
+            forward_map = generate_kernel_map(out_coords, in_coords, stride, kernel_size,
+                                              kernel_dilation, skip_symmetric_kernel_map=False)
+        kernel_map = IntSearchResult(in_maps=forward_map.out_maps, out_maps=forward_map.in_maps,
+                                     offsets=forward_map.offsets)
+    else:
+        kernel_map = generate_kernel_map(in_coords, out_coords, stride, kernel_size,
+                                         kernel_dilation, skip_symmetric_kernel_map=False)
+
+    if input_sparse_tensor.cache is None:
+        input_sparse_tensor._extra_attributes["_cache"] = IntSearchCache()
+    input_sparse_tensor.cache.put(key, kernel_map)
+    return out_coords, out_offsets, kernel_map
+
+
+# ------------------------------------------------------------------------------------------------
+# Public entry point
+# ------------------------------------------------------------------------------------------------
+
+def spatially_sparse_conv(
+    input_sparse_tensor: Voxels,
+    weight: Tensor,
+    kernel_size: Union[int, List[int], Tuple[int, ...]],
+    stride: Union[int, List[int], Tuple[int, ...]] = 1,
+    kernel_dilation: Union[int, List[int], Tuple[int, ...]] = 1,
+    bias: Optional[Tensor] = None,
+    kernel_matmul_batch_size: int = 2,
+    generative: bool = False,
+    output_spatially_sparse_tensor: Optional[Voxels] = None,
+    transposed: bool = False,
+    fwd_algo=SPARSE_CONV_FWD_ALGO_MODE.EXPLICIT_GEMM,
+    bwd_algo=SPARSE_CONV_BWD_ALGO_MODE.EXPLICIT_GEMM,
+    stride_mode: STRIDED_CONV_MODE = STRIDED_CONV_MODE.STRIDE_ONLY,
+    stride_reduce: str = "max",
+    order=POINT_ORDERING.RANDOM,
+    compute_dtype: Optional[torch.dtype] = None,
+    implicit_matmul_fwd_block_size: Optional[int] = 16,
+    implicit_matmul_bwd_block_size: Optional[int] = 16,
+) -> Voxels:
+    """Sparse convolution of a Voxels tensor with weight (K, C_in, C_out)
+    (reference: sparse_conv.py:1662-1805)."""
+    if not isinstance(input_sparse_tensor, Voxels):
+        raise TypeError("Native spatially_sparse_conv expects input_sparse_tensor of type Voxels, "
+                        f"got {type(input_sparse_tensor)}")
+    if output_spatially_sparse_tensor is not None and \
+            not isinstance(output_spatially_sparse_tensor, Voxels):
+        raise TypeError("Native spatially_sparse_conv expects output_spatially_sparse_tensor of "
+                        f"type Voxels or None, got {type(output_spatially_sparse_tensor)}")
+
+    ndim = input_sparse_tensor.num_spatial_dims
+    _kernel_size = ntuple(kernel_size, ndim=ndim)
+    _kernel_dilation = ntuple(kernel_dilation, ndim=ndim)
+    _stride = ntuple(stride, ndim=ndim)
+
+    if int(np.prod(_kernel_size)) == 1 and int(np.prod(_stride)) == 1:
+        out_features = input_sparse_tensor.feature_tensor @ weight[0]
+        if bias is not None:
+            out_features = out_features + bias
+        return input_sparse_tensor.replace(batched_features=out_features)
+
+    in_tensor_stride = input_sparse_tensor.tensor_stride
+    if in_tensor_stride is None:
+        in_tensor_stride = ntuple(1, ndim=ndim)
+
+    if transposed and not generative:
+        assert output_spatially_sparse_tensor is not None, \
+            "Output spatially sparse tensor is required for transposed convolution"
+
+    if not transposed:
+        out_tensor_stride = tuple(o * s for o, s in zip(_stride, in_tensor_stride))
+    else:
+        if output_spatially_sparse_tensor is not None and \
+                output_spatially_sparse_tensor.tensor_stride is not None:
+            out_tensor_stride = output_spatially_sparse_tensor.tensor_stride
+        else:
+            out_tensor_stride = ntuple(1, ndim=ndim)
+        assert any(o < i for o, i in zip(out_tensor_stride, in_tensor_stride)), \
+            "Output stride is larger than input stride"
+
+    features = input_sparse_tensor.feature_tensor
+    effective_compute_dtype = compute_dtype if compute_dtype is not None else features.dtype
+
+    out_coords, out_offsets, kernel_map = generate_output_coords_and_kernel_map(
+        input_sparse_tensor=input_sparse_tensor, kernel_size=_kernel_size,
+        kernel_dilation=_kernel_dilation, stride=_stride, generative=generative,
+        transposed=transposed, output_spatially_sparse_tensor=output_spatially_sparse_tensor,
+        stride_mode=stride_mode, order=order)
+    num_out_coords = out_coords.shape[0]
+
+    needs_grad = torch.is_grad_enabled() and (features.requires_grad or weight.requires_grad)
+    if needs_grad:
+        out_features = UnifiedSpatiallySparseConvFunction.apply(
+            features, weight, kernel_map, num_out_coords, fwd_algo, bwd_algo,
+            effective_compute_dtype, implicit_matmul_fwd_block_size,
+            implicit_matmul_bwd_block_size)
+        if bias is not None:
+            out_features = out_features + bias
+    elif num_out_coords == 0 or features.shape[0] == 0:
+        out_features = torch.zeros((num_out_coords, weight.shape[-1]), dtype=features.dtype,
+                                   device=features.device)
+        if bias is not None:
+            out_features = out_features + bias.to(features.dtype)
+    else:
+        # inference: the bias add is fused into the contraction's epilogue
+        out_features = sparse_conv_forward(features, weight, kernel_map, num_out_coords, bias=bias,
+                                           compute_dtype=effective_compute_dtype)
+
+    return input_sparse_tensor.replace(
+        batched_coordinates=IntCoords(out_coords[:, 1:], offsets=out_offsets.cpu().int()),
+        batched_features=out_features,
+        tensor_stride=out_tensor_stride,
+    )
