@@ -18,7 +18,7 @@ def _autocast_view(t: Tensor) -> Tensor:
     """Under torch.autocast the features are presented in the autocast dtype
     (reference: geometry.py:17-34)."""
     if torch.is_autocast_enabled():
-        amp_dtype = torch.get_autocast_gpu_dtype()
+        amp_dtype = torch.get_autocast_dtype("cuda")
         if amp_dtype is not None:
             return t.to(dtype=amp_dtype)
     return t

@@ -297,7 +297,7 @@ def spatially_sparse_conv(
     if int(np.prod(_kernel_size)) == 1 and int(np.prod(_stride)) == 1:
         out_features = input_sparse_tensor.feature_tensor @ weight[0]
         if bias is not None:
-            out_features = out_features + bias
+            out_features = out_features + bias.to(out_features.dtype)
         return input_sparse_tensor.replace(batched_features=out_features)
 
     in_tensor_stride = input_sparse_tensor.tensor_stride
@@ -336,7 +336,7 @@ def spatially_sparse_conv(
             effective_compute_dtype, implicit_matmul_fwd_block_size,
             implicit_matmul_bwd_block_size)
         if bias is not None:
-            out_features = out_features + bias
+            out_features = out_features + bias.to(out_features.dtype)
     elif num_out_coords == 0 or features.shape[0] == 0:
         out_features = torch.zeros((num_out_coords, weight.shape[-1]), dtype=features.dtype,
                                    device=features.device)
