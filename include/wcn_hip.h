@@ -156,6 +156,13 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
                         int32_t identity_offset, const int32_t* group_start_or_null, void* out,
                         int64_t num_out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Measurement hook (no counterpart in the reference, which times whole calls with CUDA events:
+ * warpconvnet/utils/timer.py:41-60).  The two hipEvent_t handles are recorded on the call's
+ * stream immediately before and after the contraction kernel of the NEXT wcn_sparse_conv_fwd
+ * call made by this host thread, so that hipEventElapsedTime gives that kernel's duration
+ * alone; the hook then disarms itself.  Pass NULLs to disarm. */
+int wcn_conv_set_timing_events(void* start_event, void* stop_event);
+
 #ifdef __cplusplus
 }
 #endif

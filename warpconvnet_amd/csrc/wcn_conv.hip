@@ -304,6 +304,11 @@ inline size_t conv_layout(void* base, int64_t num_out, int K, int c_in, int c_ou
   return off;
 }
 
+// Optional timing hook: events armed by wcn_conv_set_timing_events bracket the next conv_fwd
+// launch of this thread (and only that kernel), then disarm.
+thread_local hipEvent_t g_time_start = nullptr;
+thread_local hipEvent_t g_time_stop = nullptr;
+
 template <typename T>
 int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dtype,
                 hipStream_t s) {
@@ -318,7 +323,10 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
                        (T*)a.Wt);
   }
   const dim3 grid((unsigned)((a.num_out + TM - 1) / TM), (unsigned)(a.c_out_pad / TN));
+  if (g_time_start) (void)hipEventRecord(g_time_start, s);
   hipLaunchKernelGGL(conv_fwd<T>, grid, dim3(256), 0, s, a);
+  if (g_time_stop) (void)hipEventRecord(g_time_stop, s);
+  g_time_start = g_time_stop = nullptr;
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }
@@ -326,6 +334,12 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
 }  // namespace
 
 extern "C" {
+
+int wcn_conv_set_timing_events(void* start_event, void* stop_event) {
+  g_time_start = (hipEvent_t)start_event;
+  g_time_stop = (hipEvent_t)stop_event;
+  return WCN_OK;
+}
 
 size_t wcn_conv_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_in, int32_t c_out,
                                 int32_t dtype) {
