@@ -176,3 +176,33 @@ def test_empty_and_tiny_inputs():
     none = torch.empty((0, 4), dtype=torch.int32, device=DEV)
     km = generate_kernel_map(one, none, (1, 1, 1), (3, 3, 3))
     assert int(km.offsets[-1]) == 0 and len(km) == 27
+
+
+def test_golden_fixtures_on_gpu():
+    """Committed fixtures: strided coordinates, kernel map (bit-exact) and fp32 features."""
+    import glob
+    import os
+    from helpers import rel_err
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    paths = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
+    assert len(paths) >= 4
+    for path in paths:
+        g = np.load(path)
+        ksize, stride = tuple(int(v) for v in g["kernel_size"]), tuple(int(v) for v in g["stride"])
+        in_dev = _dev(g["in_coords"])
+        if any(s != 1 for s in stride):
+            out_dev, offsets = stride_coords(in_dev, stride)
+            assert np.array_equal(out_dev.cpu().numpy(), g["out_coords"])
+            assert np.array_equal(offsets.numpy().astype(np.int64), g["out_offsets"])
+        else:
+            out_dev = in_dev
+        km = generate_kernel_map(in_dev, out_dev, stride, ksize)
+        assert np.array_equal(km.in_maps.cpu().numpy(), g["in_maps"]), path
+        assert np.array_equal(km.out_maps.cpu().numpy(), g["out_maps"]), path
+        assert np.array_equal(km.offsets.numpy().astype(np.int64), g["offsets"]), path
+        assert (-1 if km.identity_map_index is None else km.identity_map_index) == int(g["identity"])
+        out = sparse_conv_forward(torch.as_tensor(g["features"], device=DEV),
+                                  torch.as_tensor(g["weight"], device=DEV), km, len(g["out_coords"]))
+        assert rel_err(out.cpu().numpy(), g["out_features_f64"]) <= 1e-5, path

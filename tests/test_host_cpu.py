@@ -1,0 +1,248 @@
+"""Host-side logic and the C-ABI surface, without a GPU: containers, cache keys, argument
+checks, and that libwcn_hip.so loads and exports every symbol include/wcn_hip.h declares."""
+import ctypes
+import math
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- C ABI -----------------------------------------------------------------------------------
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "wcn_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(wcn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from warpconvnet_amd._lib import SIGNATURES, lib
+    handle = lib()
+    declared = _declared_symbols()
+    assert len(declared) >= 18
+    for name in declared:
+        assert hasattr(handle, name), f"{name} declared in include/wcn_hip.h but not exported"
+    assert sorted(SIGNATURES) == declared, "ctypes binding and header disagree"
+
+
+def test_size_queries_and_status_strings():
+    from warpconvnet_amd._lib import lib
+    L = lib()
+    assert L.wcn_version() >= 100
+    for code in range(0, -7, -1):
+        assert L.wcn_status_string(code).decode() not in ("", "unknown status")
+    assert L.wcn_status_string(-99).decode() == "unknown status"
+    for n in (0, 1, 1000, 10**6, 10**8):
+        cap = L.wcn_table_default_capacity(n)
+        assert cap >= 1024 and cap & (cap - 1) == 0 and cap >= n // 2
+        assert L.wcn_table_bytes(n, cap) >= 256 + 32 * cap + 8 * n
+    assert L.wcn_kmap_workspace_bytes(10**6, 27) >= 27 * (10**6 // 64 + 1) * 4
+    assert L.wcn_kmap_workspace_bytes(10, 0) == 0 and L.wcn_kmap_workspace_bytes(10, 5000) == 0
+    assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 1) >= 27 * 64 * 64 * 2
+    assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 7) == 0
+    assert L.wcn_stride_unique_workspace_bytes(1000, 1024) > 16 * 1000
+
+
+def test_entry_points_reject_bad_arguments_before_touching_the_device():
+    from warpconvnet_amd._lib import lib
+    L = lib()
+    null = ctypes.c_void_p(0)
+    fake = ctypes.c_void_p(4096)  # never dereferenced: validation fails first
+    three = (ctypes.c_int32 * 3)(3, 3, 3)
+    bad = (ctypes.c_int32 * 3)(3, 0, 3)
+    assert L.wcn_table_build(fake, 10, null, 1024, null) == -1
+    assert L.wcn_table_build(fake, 10, fake, 1000, null) == -1      # capacity not a power of two
+    assert L.wcn_table_build(fake, -1, fake, 1024, null) == -1
+    assert L.wcn_table_query(fake, 10, 1000, fake, 5, fake, null) == -1
+    assert L.wcn_kmap_count(fake, 10, 1024, fake, 5, bad, three, fake, null) == -1
+    assert L.wcn_kmap_count(fake, 10, 1024, fake, 5, three, three, null, null) == -1
+    big = (ctypes.c_int32 * 3)(11, 11, 11)                             # 1331 offsets > 1024
+    assert L.wcn_kmap_count(fake, 10, 1024, fake, 5, big, three, fake, null) == -1
+    assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, three, three, fake, null, null, null) == -1
+    assert L.wcn_stride_unique(fake, 10, bad, fake, 1024, fake, fake, null) == -1
+    offs = (ctypes.c_int64 * 28)(*([0] * 28))
+    assert L.wcn_sparse_conv_fwd(fake, 10, 64, 9, fake, 1, 27, 64, null, fake, fake, offs, -1, null,
+                                 fake, 10, fake, 1 << 30, null) == -1  # dtype 9
+    assert L.wcn_sparse_conv_fwd(fake, 10, 64, 1, fake, 2, 27, 64, null, fake, fake, offs, -1, null,
+                                 fake, 10, fake, 1 << 30, null) == -1  # f16 features, bf16 weights
+    assert L.wcn_sparse_conv_fwd(fake, 10, 64, 1, fake, 1, 27, 64, null, fake, fake, offs, -1, null,
+                                 fake, 10, fake, 16, null) == -6       # workspace too small
+    offs[3] = 5
+    assert L.wcn_sparse_conv_fwd(fake, 10, 64, 1, fake, 1, 27, 64, null, fake, fake, offs, -1, null,
+                                 fake, 10, fake, 1 << 30, null) == -1  # offsets not monotone
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from warpconvnet_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "absent.so"))
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.lib()
+
+
+# ---- containers ------------------------------------------------------------------------------
+
+def _voxels(**kw):
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    g = torch.Generator().manual_seed(0)
+    coords = [torch.randint(0, 50, (n, 3), generator=g, dtype=torch.int32) for n in (11, 7, 5)]
+    feats = [torch.randn(len(c), 6, generator=g) for c in coords]
+    return Voxels(coords, feats, **kw), coords, feats
+
+
+def test_voxels_construction_offsets_and_batch_index():
+    """reference: tests/types/test_voxels.py:30-46."""
+    vox, coords, feats = _voxels(voxel_size=0.02)
+    assert vox.batch_size == 3 and len(vox) == 23 and vox.num_channels == 6
+    assert vox.offsets.tolist() == [0, 11, 18, 23] and not vox.offsets.is_cuda
+    assert vox.num_spatial_dims == 3 and vox.voxel_size == 0.02 and vox.tensor_stride is None
+    bc = vox.batch_indexed_coordinates
+    assert bc.shape == (23, 4) and bc.dtype == torch.int32
+    assert bc[:, 0].tolist() == [0] * 11 + [1] * 7 + [2] * 5
+    assert torch.equal(bc[:, 1:], torch.cat(coords))
+    assert torch.equal(vox.feature_tensor, torch.cat(feats))
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    again = Voxels(torch.cat(coords), torch.cat(feats), offsets=vox.offsets)
+    assert torch.equal(again.coordinate_tensor, vox.coordinate_tensor)
+    with pytest.raises(AssertionError):
+        Voxels(torch.cat(coords), torch.cat(feats))  # tensor input needs offsets
+    with pytest.raises(AssertionError):
+        Voxels(torch.cat(coords).float(), torch.cat(feats), offsets=vox.offsets)
+
+
+def test_voxels_replace_keeps_extra_attributes_and_cache():
+    """reference: tests/types/test_voxels.py:189-239 and geometry.py:313-347."""
+    from warpconvnet_amd.geometry.coords.search.cache import IntSearchCache
+    vox, _, _ = _voxels(voxel_size=0.05, custom="x", tensor_stride=2)
+    assert vox.tensor_stride == (2, 2, 2) and vox.stride == (2, 2, 2)
+    vox._extra_attributes["_cache"] = IntSearchCache()
+    new = vox.replace(batched_features=vox.feature_tensor * 2)
+    assert new.extra_attributes["custom"] == "x" and new.voxel_size == 0.05
+    assert new.cache is vox.cache
+    assert new.tensor_stride == (2, 2, 2)
+    assert torch.equal(new.feature_tensor, vox.feature_tensor * 2)
+    newer = new.replace(tensor_stride=(4, 4, 4), voxel_size=0.1)
+    assert newer.tensor_stride == (4, 4, 4) and newer.voxel_size == 0.1
+    half = vox.half()
+    assert half.feature_tensor.dtype == torch.float16 and half.extra_attributes["custom"] == "x"
+    assert vox.to(dtype=torch.float64).dtype == torch.float64
+
+
+def test_int_search_result_and_cache_key():
+    from warpconvnet_amd.geometry.coords.search.cache import IntSearchCache, IntSearchCacheKey
+    from warpconvnet_amd.geometry.coords.search.search_results import IntSearchResult
+    km = IntSearchResult(torch.tensor([5, 6, 7, 8], dtype=torch.int32),
+                         torch.tensor([0, 1, 0, 2], dtype=torch.int32),
+                         torch.tensor([0, 2, 2, 4], dtype=torch.int32), identity_map_index=1)
+    assert len(km) == 3 and km.numel(0) == 2 and km.numel(1) == 0
+    assert km[2][0].tolist() == [7, 8] and km[2][1].tolist() == [0, 2]
+    assert [a.tolist() for a, _ in km] == [[5, 6], [], [7, 8]]
+    ins, outs = km.get_batch(0, 3, out_format="tensor")
+    assert ins.tolist() == [[5, 6], [-1, -1], [7, 8]]
+    with pytest.raises(AssertionError):
+        IntSearchResult(km.in_maps, km.out_maps, torch.tensor([0, 2, 3]))
+    clone = km.clone()
+    assert clone.identity_map_index == 1 and torch.equal(clone.in_maps, km.in_maps)
+
+    def key(**kw):
+        base = dict(kernel_size=(3, 3, 3), kernel_dilation=(1, 1, 1), transposed=False,
+                    generative=False, stride_mode="stride_only", skip_symmetric_kernel_map=False,
+                    in_offsets=torch.tensor([0, 4, 9]), out_offsets=torch.tensor([0, 4, 9]))
+        base.update(kw)
+        return IntSearchCacheKey(**base)
+
+    cache = IntSearchCache()
+    cache.put(key(), km)
+    assert cache.get(key()) is km and hash(key()) == hash(key())
+    assert cache.get(key(transposed=True)) is None
+    assert cache.get(key(kernel_size=(2, 2, 2))) is None
+    assert cache.get(key(out_offsets=torch.tensor([0, 3, 9]))) is None
+
+
+def test_ntuple_and_offsets_helpers():
+    from warpconvnet_amd.geometry.coords.ops.batch_index import batch_index_from_offset, \
+        batch_indexed_coordinates, offsets_from_batch_index
+    from warpconvnet_amd.utils.ntuple import ntuple
+    assert ntuple(3, 3) == (3, 3, 3) and ntuple([1, 2, 3], 3) == (1, 2, 3)
+    assert ntuple(torch.tensor([2, 2]), 2) == (2, 2)
+    with pytest.raises(AssertionError):
+        ntuple((1, 2), 3)
+    off = torch.tensor([0, 2, 2, 5])
+    assert batch_index_from_offset(off).tolist() == [0, 0, 2, 2, 2]
+    assert offsets_from_batch_index(torch.tensor([0, 0, 1, 1, 2, 2, 2, 3, 3])).tolist() == [0, 2, 4, 7, 9]
+    bc = batch_indexed_coordinates(torch.arange(15, dtype=torch.int32).reshape(5, 3), off)
+    assert bc.dtype == torch.int32 and bc[:, 0].tolist() == [0, 0, 2, 2, 2]
+
+
+def test_kernel_offsets_from_size_matches_oracle(oracle):
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import kernel_offsets_from_size
+    for ks, dil in (((3, 3, 3), (1, 1, 1)), ((2, 2, 2), (1, 1, 1)), ((3, 2, 5), (1, 2, 3))):
+        assert np.array_equal(kernel_offsets_from_size(ks, dil).numpy(), oracle.kernel_offsets(ks, dil))
+
+
+# ---- module / functional argument handling -----------------------------------------------------
+
+def test_module_parameters_and_init_bound():
+    """weight (K, C_in, C_out) uniform within sqrt(3) * sqrt(2 / (1 + 5)) / sqrt(C_in * K)
+    (reference: nn/modules/sparse_conv.py:136,159-191)."""
+    from warpconvnet_amd.nn.modules.sparse_conv import SparseConv2d, SparseConv3d, SpatiallySparseConv
+    torch.manual_seed(0)
+    m = SparseConv3d(16, 32, 3)
+    assert tuple(m.weight.shape) == (27, 16, 32) and tuple(m.bias.shape) == (32,)
+    bound = math.sqrt(3) * math.sqrt(2.0 / 6.0) / math.sqrt(16 * 27)
+    assert m.weight.abs().max().item() <= bound and m.weight.abs().max().item() > 0.9 * bound
+    assert m.bias.abs().max().item() <= 1 / math.sqrt(16 * 27)
+    assert list(m.state_dict()) == ["weight", "bias"]
+    t = SparseConv3d(16, 32, 2, stride=2, transposed=True, bias=False)
+    assert t.bias is None and tuple(t.weight.shape) == (8, 16, 32) and t.stride == (2, 2, 2)
+    assert t.weight.abs().max().item() <= math.sqrt(3) * math.sqrt(2.0 / 6.0) / math.sqrt(32 * 8)
+    assert SparseConv2d(4, 4, 3).kernel_size == (3, 3)
+    assert SpatiallySparseConv(4, 4, (3, 1, 3), fwd_algo="explicit_gemm").kernel_size == (3, 1, 3)
+    assert "kernel_size=(3, 3, 3)" in repr(m)
+
+
+def test_functional_type_errors_and_cpu_guard():
+    from warpconvnet_amd.geometry.coords.search.torch_hashmap import HashMethod, TorchHashTable
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    vox, _, _ = _voxels()
+    w = torch.randn(27, 6, 4)
+    with pytest.raises(TypeError):
+        spatially_sparse_conv(vox.feature_tensor, w, 3)
+    with pytest.raises(TypeError):
+        spatially_sparse_conv(vox, w, 3, output_spatially_sparse_tensor=vox.feature_tensor)
+    # 1x1 shortcut is plain torch and works anywhere
+    out = spatially_sparse_conv(vox, torch.randn(1, 6, 4), 1, bias=torch.ones(4))
+    assert out.feature_tensor.shape == (23, 4)
+    table = TorchHashTable(64)
+    with pytest.raises(ValueError):
+        table.insert(torch.zeros(4, 4, dtype=torch.int32))           # CPU tensor
+    with pytest.raises(TypeError):
+        table.insert(np.zeros((4, 4), dtype=np.int32))
+    with pytest.raises(TypeError):
+        TorchHashTable(64, hash_method="city")
+    with pytest.raises(RuntimeError):
+        table.search(torch.zeros(1, 4, dtype=torch.int32))
+    assert HashMethod.CITY.kernel_suffix() == "city"
+    with pytest.raises(ValueError):                                   # no silent CPU fallback
+        from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+        from warpconvnet_amd.geometry.coords.search.search_results import IntSearchResult
+        km = IntSearchResult(torch.zeros(0, dtype=torch.int32), torch.zeros(0, dtype=torch.int32),
+                             torch.zeros(28, dtype=torch.int32))
+        sparse_conv_forward(vox.feature_tensor, w, km, 23)
+
+
+def test_synthetic_scenes_are_seeded_and_unique():
+    from warpconvnet_amd.utils import synthetic
+    a = synthetic.indoor_scene(3, 5000)
+    b = synthetic.indoor_scene(3, 5000)
+    assert np.array_equal(a, b) and a.dtype == np.int32 and a.shape == (5000, 3)
+    assert len(np.unique(a, axis=0)) == 5000
+    s = synthetic.spheres_scene(1, 3000)
+    assert len(np.unique(s, axis=0)) == 3000
+    bc = synthetic.batch_indexed([a, s])
+    assert bc.shape == (8000, 4) and (np.diff(bc[:, 0]) >= 0).all()

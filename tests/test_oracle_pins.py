@@ -1,0 +1,250 @@
+"""Pins of the CPU oracle: every oracle function is checked here against something that does
+not share its code - a library routine, a published known answer, a brute-force restatement with
+Python dicts, or an invariant the mathematics fixes.  No GPU needed."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import canonical_pairs, sort_rows
+from warpconvnet_amd.utils import synthetic
+
+
+# ---- hash functions --------------------------------------------------------------------------
+
+def test_murmur_matches_library_murmur3_32(oracle):
+    """The reference's Murmur variant (seed 0x9747B28C, 4-byte blocks, length finaliser) is the
+    standard MurmurHash3_x86_32 of the little-endian bytes: published vector and sklearn."""
+    from sklearn.utils import murmurhash3_32
+    assert oracle.hash32([0x74736574], oracle.HASH_MURMUR) == 0x704B81DC  # "test"
+    rng = np.random.default_rng(0)
+    for dim in (1, 2, 4, 7):
+        for _ in range(20):
+            key = rng.integers(-2**31, 2**31, size=dim).astype(np.int32)
+            want = murmurhash3_32(key.astype("<i4").tobytes(), seed=0x9747B28C, positive=True)
+            assert oracle.hash32(key, oracle.HASH_MURMUR) == want
+
+
+def test_city_mix_is_fmix32_chain(oracle):
+    """City variant: h <- fmix32(h + k * 0x9E3779B9).  fmix32(s) is what murmur3_32 returns for
+    the empty string with seed s, so the chain is rebuilt from the library routine."""
+    from sklearn.utils import murmurhash3_32
+    assert oracle.hash32([0, 0, 0, 0], oracle.HASH_CITY) == 0
+    rng = np.random.default_rng(1)
+    for _ in range(50):
+        key = rng.integers(-2**31, 2**31, size=4).astype(np.int32)
+        h = 0
+        for k in key.astype(np.int64):
+            h = murmurhash3_32(b"", seed=int((h + (int(k) % 2**32) * 0x9E3779B9) % 2**32),
+                               positive=True)
+        assert oracle.hash32(key, oracle.HASH_CITY) == h
+
+
+def test_fnv1a_published_vectors(oracle):
+    """With every word below 256 the word-wise FNV-1a equals the byte-wise FNV-1a-32 whose
+    published test vectors are used here."""
+    assert oracle.hash32(list(b"a"), oracle.HASH_FNV1A) == 0xE40C292C
+    assert oracle.hash32(list(b"foobar"), oracle.HASH_FNV1A) == 0xBF9CF968
+
+
+def test_slot_is_nonnegative_signed_modulo(oracle):
+    lib = oracle.lib()
+    import ctypes
+    rng = np.random.default_rng(2)
+    for _ in range(200):
+        key = rng.integers(-2**31, 2**31, size=4).astype(np.int32)
+        cap = int(rng.integers(1, 100000))
+        h = oracle.hash32(key, oracle.HASH_CITY)
+        signed = h - 2**32 if h >= 2**31 else h
+        got = lib.wcn_oracle_hash_slot(key.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), 4, cap, 1)
+        assert got == signed % cap  # Python's % is the mathematical modulo
+
+
+# ---- table -----------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("method", [0, 1, 2])
+def test_table_search_invariants(oracle, method):
+    """tests/coords/test_torch_hashmap.py:35-69 of the reference: all inserted keys are found at
+    their own row, keys from a disjoint range are absent."""
+    rng = np.random.default_rng(3)
+    keys = np.unique(rng.integers(-500, 500, size=(20000, 4)).astype(np.int32), axis=0)
+    rng.shuffle(keys)
+    table = oracle.HashTable(keys, method=method)
+    assert table.dropped == 0
+    assert np.array_equal(table.search(keys), np.arange(len(keys), dtype=np.int32))
+    assert (table.search(keys + np.array([0, 2000, 0, 0], np.int32)) == -1).all()
+    lookup = {tuple(r): i for i, r in enumerate(keys.tolist())}
+    q = rng.integers(-500, 500, size=(5000, 4)).astype(np.int32)
+    want = np.array([lookup.get(tuple(r), -1) for r in q.tolist()], dtype=np.int32)
+    assert np.array_equal(table.search(q), want)
+
+
+# ---- kernel map ------------------------------------------------------------------------------
+
+def brute_force_kernel_map(in_coords, out_coords, ksize, stride):
+    """Independent restatement: a Python dict of coordinate tuples, offsets from itertools."""
+    lookup = {}
+    for i, r in enumerate(map(tuple, in_coords.tolist())):
+        lookup.setdefault(r, i)
+    centre = [s // 2 if s % 2 == 1 else 0 for s in ksize]
+    ins, outs, offsets = [], [], [0]
+    for i, j, k in itertools.product(range(ksize[0]), range(ksize[1]), range(ksize[2])):
+        for m, (b, x, y, z) in enumerate(out_coords.tolist()):
+            q = (b, x * stride[0] + i - centre[0], y * stride[1] + j - centre[1],
+                 z * stride[2] + k - centre[2])
+            hit = lookup.get(q)
+            if hit is not None:
+                ins.append(hit)
+                outs.append(m)
+        offsets.append(len(ins))
+    return np.array(ins, np.int32), np.array(outs, np.int32), np.array(offsets, np.int64)
+
+
+KMAP_CASES = [((3, 3, 3), (1, 1, 1)), ((2, 2, 2), (2, 2, 2)), ((3, 3, 3), (2, 2, 2)),
+              ((5, 5, 5), (1, 1, 1)), ((3, 2, 1), (1, 2, 1)), ((4, 4, 4), (1, 1, 1))]
+
+
+@pytest.mark.parametrize("ksize,stride", KMAP_CASES)
+def test_kernel_map_equals_brute_force(oracle, ksize, stride):
+    in_coords = synthetic.random_cloud(7, 1500, 14, batch_size=2)
+    if any(s != 1 for s in stride):
+        out_coords = np.unique(np.concatenate(
+            [in_coords[:, :1], np.floor_divide(in_coords[:, 1:], np.array(stride))], axis=1), axis=0)
+    else:
+        out_coords = in_coords
+    got = oracle.kernel_map(in_coords, out_coords, ksize, stride)
+    want = brute_force_kernel_map(in_coords, out_coords, ksize, stride)
+    for g, w in zip(got[:3], want):
+        assert np.array_equal(g, w)
+    odd = all(k % 2 == 1 for k in ksize)
+    assert got[3] == (int(np.prod(ksize)) // 2 if odd and len(in_coords) == len(out_coords) else None)
+
+
+@pytest.mark.parametrize("method", [0, 1, 2])
+def test_kernel_map_does_not_depend_on_hash(oracle, method):
+    coords = synthetic.random_cloud(8, 3000, 18)
+    a = oracle.kernel_map(coords, coords, (3, 3, 3), method=method)
+    b = oracle.kernel_map(coords, coords, (3, 3, 3), method=1)
+    for x, y in zip(a[:3], b[:3]):
+        assert np.array_equal(x, y)
+
+
+def test_kernel_map_invariants(oracle):
+    coords = synthetic.batch_indexed([synthetic.spheres_scene(1, 20000)])
+    im, om, off, iden = oracle.kernel_map(coords, coords, (3, 3, 3))
+    n = len(coords)
+    assert iden == 13
+    assert np.array_equal(im[off[13]:off[14]], np.arange(n)) and np.array_equal(om[off[13]:off[14]], np.arange(n))
+    counts = np.diff(off)
+    assert np.array_equal(counts, counts[::-1])
+    for k in range(13):
+        a = np.stack([im[off[k]:off[k + 1]], om[off[k]:off[k + 1]]], 1)
+        b = np.stack([om[off[26 - k]:off[27 - k]], im[off[26 - k]:off[27 - k]]], 1)
+        assert np.array_equal(sort_rows(a), sort_rows(b))
+        assert (np.diff(om[off[k]:off[k + 1]]) > 0).all()
+        assert len(np.unique(im[off[k]:off[k + 1]])) == counts[k]
+
+
+def test_kernel_map_dense_cube_closed_form(oracle):
+    """A full S^3 cube in raster order: the neighbour of voxel (x,y,z) at offset (dx,dy,dz) is
+    row ((x+dx)*S + y+dy)*S + z+dz when inside the cube."""
+    S = 7
+    g = np.stack(np.meshgrid(np.arange(S), np.arange(S), np.arange(S), indexing="ij"), -1).reshape(-1, 3)
+    coords = np.concatenate([np.zeros((S**3, 1), np.int32), g.astype(np.int32)], 1)
+    im, om, off, _ = oracle.kernel_map(coords, coords, (3, 3, 3))
+    k = 0
+    for dx, dy, dz in itertools.product((-1, 0, 1), repeat=3):
+        nb = g + np.array([dx, dy, dz])
+        ok = ((nb >= 0) & (nb < S)).all(1)
+        rows = np.nonzero(ok)[0]
+        want_in = (nb[ok, 0] * S + nb[ok, 1]) * S + nb[ok, 2]
+        assert np.array_equal(om[off[k]:off[k + 1]], rows)
+        assert np.array_equal(im[off[k]:off[k + 1]], want_in)
+        k += 1
+
+
+def test_stride2_kernel2_partitions_the_fine_voxels(oracle):
+    fine = synthetic.random_cloud(9, 4000, 20, batch_size=2)
+    coarse, first, offsets = oracle.stride_coords(fine, (2, 2, 2), 2)
+    im, om, off, iden = oracle.kernel_map(fine, coarse, (2, 2, 2), (2, 2, 2))
+    assert iden is None and off[-1] == len(fine)
+    assert np.array_equal(np.sort(im), np.arange(len(fine)))
+    # every pair links a fine voxel to the coarse voxel that contains it
+    assert np.array_equal(np.floor_divide(fine[im][:, 1:], 2), coarse[om][:, 1:])
+
+
+def test_kernel_offsets_table(oracle):
+    """torch_discrete.py:44-77: last dimension fastest, centre (s-1)//2 odd / 0 even, dilation."""
+    got = oracle.kernel_offsets((3, 2, 3), (1, 1, 2))
+    want = [(0, i - 1, j, (k - 1) * 2) for i, j, k in itertools.product(range(3), range(2), range(3))]
+    assert got.tolist() == [list(w) for w in want]
+
+
+# ---- strided coordinates ---------------------------------------------------------------------
+
+@pytest.mark.parametrize("stride", [(2, 2, 2), (2, 1, 4), (3, 3, 3)])
+def test_stride_coords_equals_numpy_unique(oracle, stride):
+    coords = synthetic.random_cloud(10, 5000, 40, batch_size=3)
+    coords[:, 1:] -= 17  # negative coordinates exercise floor (not truncation)
+    out, first, offsets = oracle.stride_coords(coords, stride, 3)
+    disc = np.concatenate([coords[:, :1], np.floor_divide(coords[:, 1:], np.array(stride))], 1)
+    uniq, first_idx = np.unique(disc, axis=0, return_index=True)
+    assert np.array_equal(sort_rows(out), uniq)                    # same set as the library routine
+    assert np.array_equal(np.sort(first), np.sort(first_idx))      # lowest row represents a voxel
+    assert np.array_equal(out, disc[first])
+    assert np.array_equal(offsets, np.concatenate([[0], np.cumsum(np.bincount(out[:, 0], minlength=3))]))
+    assert (np.diff(out[:, 0]) >= 0).all()
+
+
+# ---- explicit gather-GEMM-scatter ------------------------------------------------------------
+
+def test_conv_f64_dense_cube_equals_conv3d(oracle):
+    S, c_in, c_out = 6, 5, 4
+    g = torch.Generator().manual_seed(0)
+    dense = torch.randn(1, c_in, S, S, S, generator=g, dtype=torch.float64)
+    w = torch.randn(27, c_in, c_out, generator=g, dtype=torch.float64)
+    grid = torch.stack(torch.meshgrid(torch.arange(S), torch.arange(S), torch.arange(S), indexing="ij"), -1)
+    xyz = grid.reshape(-1, 3)[torch.randperm(S**3, generator=g)]
+    coords = np.concatenate([np.zeros((S**3, 1), np.int32), xyz.numpy().astype(np.int32)], 1)
+    feats = dense[0, :, xyz[:, 0], xyz[:, 1], xyz[:, 2]].T.contiguous()
+    im, om, off, iden = oracle.kernel_map(coords, coords, (3, 3, 3))
+    got = oracle.explicit_conv_f64(feats.numpy(), w.numpy(), im, om, off, iden, len(coords))
+    w5 = w.reshape(3, 3, 3, c_in, c_out).permute(4, 3, 0, 1, 2).contiguous()
+    want = torch.nn.functional.conv3d(dense, w5, padding=1)[0][:, xyz[:, 0], xyz[:, 1], xyz[:, 2]].T
+    assert np.abs(got - want.numpy()).max() < 1e-12
+
+
+def test_conv_f64_equals_pairwise_brute_force(oracle):
+    rng = np.random.default_rng(5)
+    coords = synthetic.random_cloud(11, 60, 6)
+    n = len(coords)
+    x = rng.normal(size=(n, 3))
+    w = rng.normal(size=(27, 3, 2))
+    im, om, off, iden = oracle.kernel_map(coords, coords, (3, 3, 3))
+    want = np.zeros((n, 2))
+    for k in range(27):
+        for p in range(off[k], off[k + 1]):
+            want[om[p]] += x[im[p]] @ w[k]
+    assert np.abs(oracle.explicit_conv_f64(x, w, im, om, off, iden, n) - want).max() < 1e-12
+    # without the identity shortcut the result is the same, because map row 13 is the identity
+    assert np.abs(oracle.explicit_conv_f64(x, w, im, om, off, None, n) - want).max() < 1e-12
+
+
+def test_torch_restatement_agrees_with_c_oracle(oracle):
+    from oracle.explicit_conv import explicit_gemm_forward
+    coords = synthetic.random_cloud(12, 3000, 18, batch_size=2)
+    n = len(coords)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(n, 16, generator=g, dtype=torch.float64)
+    w = torch.randn(27, 16, 24, generator=g, dtype=torch.float64)
+    im, om, off, iden = oracle.kernel_map(coords, coords, (3, 3, 3))
+    a = explicit_gemm_forward(x, w, torch.as_tensor(im), torch.as_tensor(om), off, iden, n).numpy()
+    b = oracle.explicit_conv_f64(x.numpy(), w.numpy(), im, om, off, iden, n)
+    assert np.abs(a - b).max() < 1e-11
+    # low-precision run: rounded after every offset, still within the stated feature tolerance
+    h = explicit_gemm_forward(x.to(torch.bfloat16), w.to(torch.bfloat16), torch.as_tensor(im),
+                              torch.as_tensor(om), off, iden, n, compute_dtype=torch.float32)
+    assert h.dtype == torch.bfloat16
+    ref = oracle.explicit_conv_f64(x.to(torch.bfloat16).double().numpy(), w.to(torch.bfloat16).double().numpy(), im, om, off, iden, n)
+    assert np.abs(h.double().numpy() - ref).max() / np.abs(ref).max() < 1e-2
