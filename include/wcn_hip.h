@@ -106,8 +106,8 @@ int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int
                   const void* workspace, int32_t* in_maps, int32_t* out_maps, void* stream);
 
 /* Device address, inside a kmap workspace, of the (K, ceil(num_out/64)+1) int32 table
- * group_start[k][g] = number of pairs of offset k whose output index is below 64*g.  The
- * contraction accepts it as `host_or_null_group_start` to skip its own search. */
+ * group_start[k][g] = number of pairs of offset k whose output row is below 64*g (valid after
+ * wcn_kmap_count).  The contraction accepts it to skip its own search. */
 const int32_t* wcn_kmap_group_start(const void* workspace, int64_t num_out, int32_t num_offsets);
 
 /* ---------------------------------------------------------------------------------------------
@@ -142,19 +142,24 @@ int wcn_stride_unique_read_count(const void* workspace, int64_t n, int64_t capac
  * If identity_offset >= 0 that offset is applied as out[m] += X[m] @ W[identity_offset] for
  * every m < min(N, M) and its pairs in the map are ignored, as the reference does
  * (sparse_conv.py:292-302).
- * Within every offset out_maps must be strictly ascending (true for every map the reference
- * builds except the in/out-swapped map of a transposed convolution, which the caller sorts).
+ * The map is the reference's: in_maps, out_maps, host_offsets[K+1]; the pairs of one offset must
+ * name distinct output rows.  out_maps_ascend = 1 promises that out_maps ascends inside every
+ * offset (true for every map wcn_kmap_fill or the reference's generate_kernel_map builds);
+ * with 0 (the in/out-swapped map of a transposed convolution) the pairs are re-ordered inside
+ * the workspace first.  group_start_or_null: the table wcn_kmap_group_start returns for this
+ * map, or NULL to have it derived here (only meaningful with out_maps_ascend = 1).
  * ------------------------------------------------------------------------------------------- */
 
 size_t wcn_conv_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_in, int32_t c_out,
-                                int32_t dtype);
+                                int32_t dtype, int64_t num_pairs, int32_t out_maps_ascend);
 
 int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
                         const void* weight, int32_t weight_dtype, int32_t num_offsets,
                         int32_t c_out, const void* bias_or_null, const int32_t* in_maps,
                         const int32_t* out_maps, const int64_t* host_offsets,
-                        int32_t identity_offset, const int32_t* group_start_or_null, void* out,
-                        int64_t num_out, void* workspace, size_t workspace_bytes, void* stream);
+                        int32_t identity_offset, int32_t out_maps_ascend,
+                        const int32_t* group_start_or_null, void* out, int64_t num_out,
+                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* Measurement hook (no counterpart in the reference, which times whole calls with CUDA events:
  * warpconvnet/utils/timer.py:41-60).  The two hipEvent_t handles are recorded on the call's

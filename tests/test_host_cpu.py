@@ -43,8 +43,9 @@ def test_size_queries_and_status_strings():
         assert L.wcn_table_bytes(n, cap) >= 256 + 32 * cap + 8 * n
     assert L.wcn_kmap_workspace_bytes(10**6, 27) >= 27 * (10**6 // 64 + 1) * 4
     assert L.wcn_kmap_workspace_bytes(10, 0) == 0 and L.wcn_kmap_workspace_bytes(10, 5000) == 0
-    assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 1) >= 27 * 64 * 64 * 2
-    assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 7) == 0
+    assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 1, 5000, 1) >= 27 * 64 * 64 * 2
+    assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 1, 5000, 0) >= 27 * 64 * 64 * 2 + 12 * 5000 + 8 * 1000
+    assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 7, 0, 1) == 0
     assert L.wcn_stride_unique_workspace_bytes(1000, 1024) > 16 * 1000
 
 
@@ -63,18 +64,22 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert L.wcn_kmap_count(fake, 10, 1024, fake, 5, three, three, null, null) == -1
     big = (ctypes.c_int32 * 3)(11, 11, 11)                             # 1331 offsets > 1024
     assert L.wcn_kmap_count(fake, 10, 1024, fake, 5, big, three, fake, null) == -1
+    assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, bad, three, fake, fake, fake, null) == -1
     assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, three, three, fake, null, null, null) == -1
     assert L.wcn_stride_unique(fake, 10, bad, fake, 1024, fake, fake, null) == -1
     offs = (ctypes.c_int64 * 28)(*([0] * 28))
-    assert L.wcn_sparse_conv_fwd(fake, 10, 64, 9, fake, 1, 27, 64, null, fake, fake, offs, -1, null,
-                                 fake, 10, fake, 1 << 30, null) == -1  # dtype 9
-    assert L.wcn_sparse_conv_fwd(fake, 10, 64, 1, fake, 2, 27, 64, null, fake, fake, offs, -1, null,
-                                 fake, 10, fake, 1 << 30, null) == -1  # f16 features, bf16 weights
-    assert L.wcn_sparse_conv_fwd(fake, 10, 64, 1, fake, 1, 27, 64, null, fake, fake, offs, -1, null,
-                                 fake, 10, fake, 16, null) == -6       # workspace too small
+
+    def conv(dtype=1, wdtype=1, ws_bytes=1 << 30, ascend=1, gs=null, offsets=offs):
+        return L.wcn_sparse_conv_fwd(fake, 10, 64, dtype, fake, wdtype, 27, 64, null, fake, fake,
+                                     offsets, -1, ascend, gs, fake, 10, fake, ws_bytes, null)
+
+    assert conv(dtype=9) == -1
+    assert conv(wdtype=2) == -1                      # f16 features with bf16 weights
+    assert conv(ws_bytes=16) == -6                   # workspace too small
+    assert conv(ascend=0, gs=fake) == -1             # group starts need ascending pairs
+    assert conv(offsets=None) == -1
     offs[3] = 5
-    assert L.wcn_sparse_conv_fwd(fake, 10, 64, 1, fake, 1, 27, 64, null, fake, fake, offs, -1, null,
-                                 fake, 10, fake, 1 << 30, null) == -1  # offsets not monotone
+    assert conv() == -1                              # offsets not monotone
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

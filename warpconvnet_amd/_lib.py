@@ -32,10 +32,10 @@ SIGNATURES = {
     "wcn_stride_unique_workspace_bytes": (_sz, [_i64, _i64]),
     "wcn_stride_unique": (ctypes.c_int, [_vp, _i64, _i32p, _vp, _i64, _vp, _vp, _vp]),
     "wcn_stride_unique_read_count": (ctypes.c_int, [_vp, _i64, _i64, _i64p, _vp]),
-    "wcn_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i32]),
+    "wcn_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i32, _i64, _i32]),
     "wcn_conv_set_timing_events": (ctypes.c_int, [_vp, _vp]),
     "wcn_sparse_conv_fwd": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
-                                           _vp, _i64p, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
+                                           _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
 }
 
 _lib = None

@@ -42,7 +42,6 @@ struct WcnTableView {  // host-computed addresses inside a table workspace
   WcnSlot* slots;
   int32_t* perm;        // n_keys
   int32_t* slot_of;     // n_keys (slot of each key; build scratch)
-  int32_t* block_list;  // min(capacity, n_keys) occupied slot ids in claim order
   int64_t n_keys;
   int64_t capacity;
 };
@@ -61,8 +60,6 @@ static inline size_t wcn_table_layout(void* base, int64_t n_keys, int64_t capaci
   off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
   if (v) v->slot_of = (int32_t*)(p + off);
   off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
-  if (v) v->block_list = (int32_t*)(p + off);
-  off += wcn_align256(sizeof(int32_t) * (size_t)(capacity < n_keys ? capacity : n_keys));
   if (v) {
     v->n_keys = n_keys;
     v->capacity = capacity;
@@ -130,24 +127,32 @@ __device__ __forceinline__ uint32_t wcn_mix(unsigned long long k, uint32_t cap_m
   return (uint32_t)k & cap_mask;
 }
 
-// Finds the slot of a block key.  Returns its mask (0 if the block is absent) and base.
-__device__ __forceinline__ unsigned long long wcn_lookup_block(const WcnSlot* __restrict__ slots,
-                                                               uint32_t cap_mask,
-                                                               unsigned long long key,
-                                                               int32_t* base) {
-  uint32_t h = wcn_mix(key, cap_mask);
-  for (int p = 0; p < WCN_MAX_PROBE; ++p) {
-    // one 16-byte load brings key and mask; base sits in the same 32-byte slot
-    const ulonglong2 km = *reinterpret_cast<const ulonglong2*>(&slots[h]);
-    if (km.x == key) {
-      *base = slots[h].base;
-      return km.y;
+// Finds the slot of a block key.  Returns its mask (0 if the block is absent) and base.  Both
+// 16-byte halves of the 32-byte slot are requested together, so a hit costs one memory round trip.
+__device__ __forceinline__ unsigned long long wcn_lookup_block_from(
+    const WcnSlot* __restrict__ slots, uint32_t cap_mask, unsigned long long key, uint32_t h,
+    int first_probe, int32_t* base) {
+  for (int p = first_probe; p < WCN_MAX_PROBE; ++p) {
+    const uint4* raw = reinterpret_cast<const uint4*>(&slots[h]);
+    const uint4 lo = raw[0];
+    const uint4 hi = raw[1];
+    const unsigned long long k = ((unsigned long long)lo.y << 32) | lo.x;
+    if (k == key) {
+      *base = (int32_t)hi.x;
+      return ((unsigned long long)lo.w << 32) | lo.z;
     }
-    if (km.x == WCN_EMPTY_KEY) break;
+    if (k == WCN_EMPTY_KEY) break;
     h = (h + 1) & cap_mask;
   }
   *base = 0;
   return 0ull;
+}
+
+__device__ __forceinline__ unsigned long long wcn_lookup_block(const WcnSlot* __restrict__ slots,
+                                                               uint32_t cap_mask,
+                                                               unsigned long long key,
+                                                               int32_t* base) {
+  return wcn_lookup_block_from(slots, cap_mask, key, wcn_mix(key, cap_mask), 0, base);
 }
 
 __device__ __forceinline__ int wcn_rank_below(unsigned long long mask, uint32_t bit) {

@@ -2,51 +2,45 @@
 //
 //   out[m, :] = bias + sum_k sum_{p in offset k, out_maps[p] == m} X[in_maps[p], :] @ W[k]
 //
-// Output-stationary and atomic-free: a workgroup owns TM consecutive output rows and TN output
-// channels and keeps their fp32 accumulators in LDS for the whole kernel.  Because the pairs of
-// every offset ascend in output index, the pairs that touch the workgroup's rows are one
-// contiguous run per offset, located with the group_start table (number of pairs of offset k
-// below output row 64*g).  For each offset the run is processed in chunks of RB pairs: the RB
-// input rows are gathered into LDS, multiplied with W[k] (kept transposed so that both MFMA
-// operands are 16-byte LDS reads) by v_mfma_f32_16x16x32_{f16,bf16} / v_mfma_f32_16x16x4_f32,
-// and the fp32 products are added to the accumulator rows the pairs name.  Rows are rounded to
-// the feature dtype once, when the tile is written.
+// Output-stationary, atomic-free, accumulators in registers.  A workgroup of four waves owns 256
+// consecutive output rows x 64 output channels; each wave keeps the fp32 accumulators of its 64
+// rows in MFMA result layout for the whole kernel.  The map is consumed in output-row form (per
+// row: bit mask of the offsets that hit, row pointer, hit input rows).
 //
-// Compulsory HBM bytes: every input row once per offset that uses it (L * C_in * s, served by the
-// L2 / Infinity Cache when rows are revisited), the maps once (8 L), the output once
-// (M * C_out * s); the weights (K * C_in * C_out * s) stay cache resident.
+// The loop over offsets is cut into batches.  For a batch (up to 8 offsets, up to 256 hits) the
+// workgroup lists the hits of its rows, assigns each hit a slot, and gathers all hit input rows
+// into LDS with every load issued back to back (this is what keeps tens of KB in flight per CU;
+// a gather per offset would leave the kernel latency bound).  Then, offset by offset, W[k]^T is
+// staged in LDS (double buffered, fetched one offset ahead) and each wave multiplies its 64 rows:
+// lane l of a 16-row block reads the gathered row of output row (l & 15) through its slot, or
+// zeros if that output row has no hit for this offset, so the product lands in the accumulator
+// rows directly (v_mfma_f32_16x16x32_{f16,bf16}, v_mfma_f32_16x16x4_f32).  16-row blocks without
+// any hit are skipped.  One rounding to the feature dtype when the tile is written.
+//
+// Compulsory HBM bytes: every hit input row once (L * C_in * s; revisits are served by the L2 /
+// Infinity Cache), the map once (8 M + 4 L), the output once (M * C_out * s); the weights
+// (K * C_in * C_out * s) stay cache resident.
 #include <algorithm>
+#include <type_traits>
 
 #include "wcn_common.h"
+
+void wcn_scan_rows_launch(int32_t* groups, int64_t G, int rows, int64_t* row_total, hipStream_t s);
 
 namespace {
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte piece
 
-constexpr int TM = 128;  // output rows per workgroup (two 64-row groups of the kernel map)
-constexpr int TN = 64;   // output channels per workgroup
-constexpr int RB = 64;   // pairs per chunk (4 waves x 16 MFMA rows)
-constexpr int ACC_LD = TN + 4;
-
-template <typename T>
-struct Cfg;
-template <>
-struct Cfg<_Float16> {
-  static constexpr int CK = 64;     // input channels staged per chunk
-  static constexpr int LD = CK + 8; // LDS row pitch in elements (144 B: spreads rows over banks)
-};
-template <>
-struct Cfg<__bf16> {
-  static constexpr int CK = 64;
-  static constexpr int LD = CK + 8;
-};
-template <>
-struct Cfg<float> {
-  static constexpr int CK = 32;
-  static constexpr int LD = CK + 4;
-};
+constexpr int ROWS = 256;    // output rows per workgroup
+constexpr int TN = 64;       // output channels per workgroup
+constexpr int THREADS = 256; // wave w owns rows 64 * (w & 3) .. +63 and channel blocks of column group (w >> 2)
+constexpr int NBW = TN / 16 / (THREADS / 256);  // 16-channel blocks per wave
+constexpr int BPT = TN * 8 / THREADS;           // 16-byte parts of a weight tile per thread
+constexpr int A_ROWS = 256;  // gathered input rows resident in LDS
+constexpr int BATCH = 7;     // offsets per gather batch, at most
 
 __device__ __forceinline__ float to_float(_Float16 v) { return (float)v; }
 __device__ __forceinline__ float to_float(__bf16 v) { return (float)v; }
@@ -56,40 +50,50 @@ __device__ __forceinline__ T from_float(float v) {
   return (T)v;
 }
 
-// One 16x16 output block: acc += A(16 x CK, rows of As) * B(CK x 16, rows of Bs are columns).
-// Operand layout of the 16x16x32 MFMAs: lane l holds row (l & 15), k = 8 * (l >> 4) .. +7 of A
-// and column (l & 15), same k of B; the result holds column (l & 15), rows 4 * (l >> 4) .. +3.
-__device__ __forceinline__ f32x4 mma_block(const _Float16* a_row, const _Float16* b_row, int lane,
-                                           f32x4 acc) {
-#pragma unroll
-  for (int ks = 0; ks < Cfg<_Float16>::CK / 32; ++ks) {
-    const f16x8 a = *reinterpret_cast<const f16x8*>(a_row + ks * 32 + (lane >> 4) * 8);
-    const f16x8 b = *reinterpret_cast<const f16x8*>(b_row + ks * 32 + (lane >> 4) * 8);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+// MFMA operand handling per element type.  16x16x32 (f16/bf16): lane l holds row (l & 15),
+// k = 8 * (l >> 4) .. +7 of A and column (l & 15), same k of B; 16x16x4 (f32): lane l holds
+// A[row l & 15][k = l >> 4], B[k = l >> 4][col l & 15].  The result holds column (l & 15), rows
+// 4 * (l >> 4) .. +3.  Both operands are read from rows of CK contiguous k values.
+template <typename T>
+struct Mma;
+template <>
+struct Mma<_Float16> {
+  typedef f16x8 V;
+  static constexpr int CK = 64, KS = 2;
+  // 8 consecutive k of row `r`: logical part ks * 4 + kgrp, stored at its swizzled position
+  static __device__ __forceinline__ V load(const _Float16* row, int r, int ks, int kgrp) {
+    return *reinterpret_cast<const V*>(row + ((ks * 4 + kgrp) ^ ((r >> 1) & 7)) * 8);
   }
-  return acc;
-}
-__device__ __forceinline__ f32x4 mma_block(const __bf16* a_row, const __bf16* b_row, int lane,
-                                           f32x4 acc) {
-#pragma unroll
-  for (int ks = 0; ks < Cfg<__bf16>::CK / 32; ++ks) {
-    const bf16x8 a = *reinterpret_cast<const bf16x8*>(a_row + ks * 32 + (lane >> 4) * 8);
-    const bf16x8 b = *reinterpret_cast<const bf16x8*>(b_row + ks * 32 + (lane >> 4) * 8);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+  static __device__ __forceinline__ V zero() { return (V){0, 0, 0, 0, 0, 0, 0, 0}; }
+  static __device__ __forceinline__ f32x4 mma(V a, V b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
-  return acc;
-}
-// fp32: v_mfma_f32_16x16x4_f32, lane l holds A[row l & 15][k = l >> 4] and B[k = l >> 4][col l & 15].
-__device__ __forceinline__ f32x4 mma_block(const float* a_row, const float* b_row, int lane,
-                                           f32x4 acc) {
-#pragma unroll
-  for (int ks = 0; ks < Cfg<float>::CK / 4; ++ks) {
-    const float a = a_row[ks * 4 + (lane >> 4)];
-    const float b = b_row[ks * 4 + (lane >> 4)];
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc, 0, 0, 0);
+};
+template <>
+struct Mma<__bf16> {
+  typedef bf16x8 V;
+  static constexpr int CK = 64, KS = 2;
+  static __device__ __forceinline__ V load(const __bf16* row, int r, int ks, int kgrp) {
+    return *reinterpret_cast<const V*>(row + ((ks * 4 + kgrp) ^ ((r >> 1) & 7)) * 8);
   }
-  return acc;
-}
+  static __device__ __forceinline__ V zero() { return (V){0, 0, 0, 0, 0, 0, 0, 0}; }
+  static __device__ __forceinline__ f32x4 mma(V a, V b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<float> {
+  typedef float V;
+  static constexpr int CK = 32, KS = 8;
+  // element ks * 4 + kgrp of row `r`: part ks (four floats), swizzled, then the float inside it
+  static __device__ __forceinline__ V load(const float* row, int r, int ks, int kgrp) {
+    return row[(ks ^ ((r >> 1) & 7)) * 4 + kgrp];
+  }
+  static __device__ __forceinline__ V zero() { return 0.f; }
+  static __device__ __forceinline__ f32x4 mma(V a, V b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+};
 
 // Wt[k][n][c] = W[k][c][n] converted to T, zero padded to (c_out_pad, c_in_pad).
 template <typename T, typename WT>
@@ -108,7 +112,275 @@ __global__ void __launch_bounds__(256) conv_prep_weight(const WT* __restrict__ W
   }
 }
 
-// group_start[k][g] = number of pairs of offset k with out_maps < 64 * g (binary search).
+struct ConvArgs {
+  const void* X;
+  const void* Wt;
+  const void* bias;            // same dtype as X, or null
+  const int32_t* in_maps;      // pair lists; inside every offset out_maps ascends
+  const int32_t* out_maps;
+  const int64_t* offsets;      // (K + 1), device
+  const int32_t* group_start;  // (K, G + 1): pairs of offset k below output row 64 * g
+  void* out;
+  int64_t num_in, num_out, G;
+  int32_t K, c_in, c_out, c_in_pad, c_out_pad, identity;
+  int32_t vec_in;   // feature rows are 16-byte aligned and a whole number of 16-byte vectors
+  int32_t vec_out;  // same for output rows
+};
+
+struct WTile {
+  u32x4 p[BPT];
+};
+
+// LDS rows are 128 bytes (eight 16-byte parts) with no padding; part p of row r is stored at
+// part p ^ ((r >> 1) & 7), which makes the 16-byte operand reads of 16 consecutive rows (and of
+// most scattered row sets) hit distinct banks.
+__device__ __forceinline__ int lds_part(int row, int part) { return part ^ ((row >> 1) & 7); }
+
+template <typename T>
+__global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
+  typedef Mma<T> M;
+  typedef typename M::V V;
+  constexpr int CK = M::CK, KS = M::KS;
+  constexpr int VEC = 16 / sizeof(T);  // elements per 16-byte part; a row is CK = 8 * VEC elements
+  static_assert(CK == 8 * VEC, "a staged row is eight 16-byte parts");
+  __shared__ __attribute__((aligned(16))) T As[A_ROWS * CK + VEC];  // + one all-zero 16-byte part
+  __shared__ __attribute__((aligned(16))) T Bs[2][TN * CK];
+  __shared__ uint16_t s_slot[BATCH][ROWS];  // gathered row of (offset, output row); A_ROWS = none
+  __shared__ int32_t s_gidx[A_ROWS];
+  __shared__ int32_t s_cnt[32];
+  __shared__ int32_t s_start[32];
+
+  const T* __restrict__ X = (const T*)a.X;
+  const T* __restrict__ Wt = (const T*)a.Wt;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wrow = (wave & 3) * 64, wcol = (wave >> 2) * (NBW * 16);
+  const int64_t m0 = (int64_t)blockIdx.x * ROWS;
+  const int n0 = blockIdx.y * TN;
+  const int tile_rows = (int)(a.num_out - m0 < ROWS ? a.num_out - m0 : ROWS);
+  const int64_t g0 = m0 >> 6;
+  const int64_t g1 = g0 + ROWS / 64 < a.G ? g0 + ROWS / 64 : a.G;
+
+  if (tid < VEC) As[A_ROWS * CK + tid] = from_float<T>(0.f);
+
+  f32x4 acc[4][NBW];
+#pragma unroll
+  for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+    for (int nb = 0; nb < NBW; ++nb) acc[rb][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  // this thread's 16-byte parts of a (TN x CK) weight tile (rows b_n + h * THREADS / 8)
+  const int b_n = tid >> 3, b_part = tid & 7;
+  // MFMA operand addressing: lane l reads row (l & 15) of a 16-row block, k-group (l >> 4)
+  const int kgrp = lane >> 4;
+
+  for (int c0 = 0; c0 < a.c_in_pad; c0 += CK) {
+    for (int kbase = 0; kbase < a.K; kbase += 32) {
+      const int nk = a.K - kbase < 32 ? a.K - kbase : 32;
+      __syncthreads();  // the previous chunk's readers of s_cnt / s_start are done
+      if (tid < 32) {
+        int cnt = 0;
+        int32_t start = 0;
+        const int k = kbase + tid;
+        if (tid < nk) {
+          if (k == a.identity) {  // every row reads its own input row; the map's pairs are ignored
+            const int64_t left = a.num_in - m0;
+            cnt = (int)(left < 0 ? 0 : (left < tile_rows ? left : tile_rows));
+          } else {
+            const int32_t* gs = a.group_start + (int64_t)k * (a.G + 1);
+            start = (int32_t)(a.offsets[k] + gs[g0]);
+            cnt = gs[g1] - gs[g0];
+            if (cnt < 0 || cnt > ROWS) cnt = 0;  // inconsistent table: contribute nothing
+          }
+        }
+        s_cnt[tid] = cnt;
+        s_start[tid] = start;
+      }
+      __syncthreads();
+
+      int b0 = 0;
+      while (b0 < nk) {
+        // batch [b0, b1): as many offsets as fit the LDS row budget (one offset always fits)
+        int b1 = b0, total = 0;
+        while (b1 < nk && b1 - b0 < BATCH && total + s_cnt[b1] <= A_ROWS) total += s_cnt[b1++];
+        if (total == 0) {
+          b0 = b1;
+          continue;
+        }
+        // the pair that becomes gathered row `tid` of this batch
+        int my_j = -1, my_in = -1, my_out = -1;
+        if (tid < ROWS) {
+          int before = 0;
+#pragma unroll
+          for (int j = 0; j < BATCH; ++j) {
+            const int c = b0 + j < b1 ? s_cnt[b0 + j] : 0;
+            if (my_j < 0 && tid >= before && tid < before + c) {
+              my_j = j;
+              const int i = tid - before;
+              if (kbase + b0 + j == a.identity) {
+                my_in = (int)(m0 + i);
+                my_out = i;
+              } else {
+                const int64_t p = (int64_t)s_start[b0 + j] + i;
+                my_in = a.in_maps[p];
+                my_out = (int)(a.out_maps[p] - m0);
+              }
+            }
+            before += c;
+          }
+        }
+        // weight tiles travel through two register slots: the first two offsets of the batch are
+        // requested together with the gather, offset j + 2 as soon as offset j left its slot
+        WTile wa, wb;
+        auto fetch_b = [&](int j, WTile& r) {
+          if (j < BATCH && b0 + j < b1 && s_cnt[b0 + j] > 0) {
+#pragma unroll
+            for (int h = 0; h < BPT; ++h)
+              r.p[h] = *reinterpret_cast<const u32x4*>(
+                  Wt + ((int64_t)(kbase + b0 + j) * a.c_out_pad + n0 + b_n + h * (THREADS / 8)) * a.c_in_pad +
+                  c0 + b_part * VEC);
+          }
+        };
+        fetch_b(0, wa);
+        fetch_b(1, wb);
+        // slot table of the batch: "no hit" everywhere, then one entry per pair
+        if (tid < BATCH * ROWS / 8)
+          *reinterpret_cast<u32x4*>(&s_slot[0][0] + tid * 8) =
+              (u32x4){A_ROWS * 0x10001u, A_ROWS * 0x10001u, A_ROWS * 0x10001u, A_ROWS * 0x10001u};
+        __syncthreads();
+        if (my_j >= 0) {
+          if ((uint32_t)my_in >= (uint64_t)a.num_in) my_in = -1;  // malformed map: zeros
+          s_gidx[tid] = my_in;
+          if ((uint32_t)my_out < (uint32_t)tile_rows) s_slot[my_j][my_out] = (uint16_t)tid;
+        }
+        __syncthreads();
+
+        // gather every hit row of the batch: loads first, all independent, then the LDS stores
+        if (a.vec_in) {
+          u32x4 piece[A_ROWS * 8 / THREADS];
+#pragma unroll
+          for (int i = 0; i < A_ROWS * 8 / THREADS; ++i) {
+            const int seg = tid + i * THREADS, sl = seg >> 3, part = seg & 7;
+            piece[i] = (u32x4){0u, 0u, 0u, 0u};
+            if (seg < total * 8) {
+              const int32_t g = s_gidx[sl];
+              if (g >= 0 && c0 + part * VEC < a.c_in)
+                piece[i] = *reinterpret_cast<const u32x4*>(X + (int64_t)g * a.c_in + c0 + part * VEC);
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < A_ROWS * 8 / THREADS; ++i) {
+            const int seg = tid + i * THREADS, sl = seg >> 3, part = seg & 7;
+            if (seg < total * 8)
+              *reinterpret_cast<u32x4*>(&As[sl * CK + lds_part(sl, part) * VEC]) = piece[i];
+          }
+        } else {
+          for (int e = tid; e < total * CK; e += THREADS) {
+            const int sl = e / CK, c = e % CK;
+            const int32_t g = s_gidx[sl];
+            T val = from_float<T>(0.f);
+            if (g >= 0 && c0 + c < a.c_in) val = X[(int64_t)g * a.c_in + c0 + c];
+            As[sl * CK + lds_part(sl, c / VEC) * VEC + c % VEC] = val;
+          }
+        }
+
+        // One barrier per offset: W[k]^T goes to the buffer the previous offset did not use, the
+        // barrier publishes it (and, the first time, the gathered rows), then every wave multiplies.
+        // A wave can only overwrite a buffer after all waves passed the barrier that follows its
+        // last use.
+        int buf = 0;
+        auto multiply = [&](int j, WTile& r) {
+          if (b0 + j >= b1) return;  // uniform
+          if (s_cnt[b0 + j] == 0) {
+            fetch_b(j + 2, r);  // keep the ring moving
+            return;
+          }
+#pragma unroll
+          for (int h = 0; h < BPT; ++h) {
+            const int n = b_n + h * (THREADS / 8);
+            *reinterpret_cast<u32x4*>(&Bs[buf][n * CK + lds_part(n, b_part) * VEC]) = r.p[h];
+          }
+          fetch_b(j + 2, r);
+          // gathered rows of this wave's four 16-row blocks
+          int sl[4];
+#pragma unroll
+          for (int rb = 0; rb < 4; ++rb) sl[rb] = s_slot[j][wrow + rb * 16 + (lane & 15)];
+          __syncthreads();
+          V bfr[NBW][KS];
+#pragma unroll
+          for (int nb = 0; nb < NBW; ++nb) {
+            const int n = wcol + nb * 16 + (lane & 15);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) bfr[nb][ks] = M::load(&Bs[buf][n * CK], n, ks, kgrp);
+          }
+#pragma unroll
+          for (int rb = 0; rb < 4; ++rb) {
+            if (__ballot(sl[rb] != A_ROWS) == 0ull) continue;  // no hit in these 16 rows
+            V av[KS];  // rows without a hit read zeros
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+              av[ks] = sl[rb] != A_ROWS ? M::load(&As[sl[rb] * CK], sl[rb], ks, kgrp) : M::zero();
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+              for (int nb = 0; nb < NBW; ++nb) acc[rb][nb] = M::mma(av[ks], bfr[nb][ks], acc[rb][nb]);
+          }
+          buf ^= 1;
+        };
+#pragma nounroll
+        for (int j = 0; j < BATCH; j += 2) {
+          multiply(j, wa);
+          multiply(j + 1, wb);
+        }
+        __syncthreads();  // every wave is done with the gathered rows and the slot table
+        b0 = b1;
+      }
+    }
+  }
+
+  // epilogue: bias add, one rounding to T
+  T* __restrict__ out = (T*)a.out;
+  const T* __restrict__ bias = (const T*)a.bias;
+  if (sizeof(T) == 2 && a.vec_out) {
+    // stage the tile in LDS (As is free: the last batch ended with a barrier) for 16-byte stores
+    __syncthreads();
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+      for (int nb = 0; nb < NBW; ++nb) {
+        const int col = wcol + nb * 16 + (lane & 15);
+        const float bv = (bias && n0 + col < a.c_out) ? to_float(bias[n0 + col]) : 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int lr = wrow + rb * 16 + kgrp * 4 + r;
+          As[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC] = from_float<T>(acc[rb][nb][r] + bv);
+        }
+      }
+    __syncthreads();
+    for (int v = tid; v < ROWS * 8; v += THREADS) {
+      const int r = v >> 3, part = v & 7;
+      if (m0 + r < a.num_out && n0 + part * VEC < a.c_out)
+        *reinterpret_cast<u32x4*>(out + (m0 + r) * a.c_out + n0 + part * VEC) =
+            *reinterpret_cast<const u32x4*>(&As[r * CK + lds_part(r, part) * VEC]);
+    }
+  } else {
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+      for (int nb = 0; nb < NBW; ++nb) {
+        const int col = n0 + wcol + nb * 16 + (lane & 15);
+        if (col >= a.c_out) continue;
+        const float bv = bias ? to_float(bias[col]) : 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int64_t orow = m0 + wrow + rb * 16 + kgrp * 4 + r;
+          if (orow < a.num_out) out[orow * a.c_out + col] = from_float<T>(acc[rb][nb][r] + bv);
+        }
+      }
+  }
+}
+
+// group_start[k][g] = number of pairs of offset k with out_maps < 64 * g (binary search; needs
+// out_maps ascending inside every offset).
 __global__ void __launch_bounds__(256) conv_group_start(const int32_t* __restrict__ out_maps,
                                                         const int64_t* __restrict__ offsets, int K,
                                                         int64_t G, int32_t* __restrict__ gs) {
@@ -116,8 +388,8 @@ __global__ void __launch_bounds__(256) conv_group_start(const int32_t* __restric
   if (i >= (int64_t)K * (G + 1)) return;
   const int k = (int)(i / (G + 1));
   const int64_t g = i % (G + 1);
-  const int64_t lo0 = offsets[k], hi0 = offsets[k + 1];
-  int64_t lo = lo0, hi = hi0;
+  const int64_t lo0 = offsets[k];
+  int64_t lo = lo0, hi = offsets[k + 1];
   const int64_t target = g * 64;
   while (lo < hi) {
     const int64_t mid = (lo + hi) >> 1;
@@ -126,180 +398,162 @@ __global__ void __launch_bounds__(256) conv_group_start(const int32_t* __restric
   gs[i] = (int32_t)(lo - lo0);
 }
 
-struct ConvArgs {
-  const void* X;
-  const void* Wt;
-  const void* bias;         // same dtype as X, or null
-  const int32_t* in_maps;
-  const int32_t* out_maps;
-  const int64_t* offsets;   // device copy, K+1
-  const int32_t* group_start;  // (K, G+1)
-  void* out;
-  int64_t num_in, num_out, G;
-  int32_t K, c_in, c_out, c_in_pad, c_out_pad, identity;
-  int32_t vec_rows;  // feature rows are 16-byte aligned and a whole number of 16-byte vectors
-};
+// ---- pair lists -> output-row form (for maps that were not built by wcn_kmap_fill) ---------------
 
-__device__ __forceinline__ int64_t imin(int64_t x, int64_t y) { return x < y ? x : y; }
-__device__ __forceinline__ int64_t imax(int64_t x, int64_t y) { return x > y ? x : y; }
-
-template <typename T>
-__global__ void __launch_bounds__(256) conv_fwd(ConvArgs a) {
-  constexpr int CK = Cfg<T>::CK;
-  constexpr int LD = Cfg<T>::LD;
-  constexpr int VEC = 16 / sizeof(T);  // elements per 16-byte vector
-  __shared__ float accs[TM * ACC_LD];
-  __shared__ __attribute__((aligned(16))) T As[RB * LD];
-  __shared__ __attribute__((aligned(16))) T Bs[TN * LD];
-  __shared__ int32_t s_in[RB];
-  __shared__ int32_t s_out[RB];
-
-  const T* __restrict__ X = (const T*)a.X;
-  const T* __restrict__ Wt = (const T*)a.Wt;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t m0 = (int64_t)blockIdx.x * TM;
-  const int n0 = blockIdx.y * TN;
-  const int tile_rows = (int)imin(TM, a.num_out - m0);
-  const int64_t g0 = m0 >> 6;
-  const int64_t g1 = imin(g0 + TM / 64, a.G);
-  const bool vec_rows = a.vec_rows != 0;
-  const int64_t num_pairs = a.offsets[a.K];
-
-  for (int i = tid; i < TM * ACC_LD; i += 256) accs[i] = 0.f;
-  __syncthreads();
-
-  for (int k = 0; k < a.K; ++k) {
-    int64_t p0, cnt;
-    const bool iden = (k == a.identity);
-    if (iden) {
-      p0 = 0;
-      cnt = imax(0, imin(tile_rows, a.num_in - m0));
-    } else {
-      const int32_t* gs = a.group_start + (int64_t)k * (a.G + 1);
-      p0 = a.offsets[k] + gs[g0];
-      cnt = imin(gs[g1] - gs[g0], num_pairs - p0);  // never read past the maps
-    }
-    for (int64_t r0 = 0; r0 < cnt; r0 += RB) {
-      const int rows = (int)imin(RB, cnt - r0);
-      __syncthreads();  // previous chunk's readers of s_in / s_out are done
-      if (tid < RB) {
-        int32_t ii = 0, oo = 0;
-        if (tid < rows) {
-          if (iden) {
-            ii = (int32_t)(m0 + r0 + tid);
-            oo = (int32_t)(r0 + tid);
-          } else {
-            ii = a.in_maps[p0 + r0 + tid];
-            oo = (int32_t)(a.out_maps[p0 + r0 + tid] - m0);
-          }
-          // a malformed map must not turn into a wild access: such a pair contributes nothing
-          if ((uint32_t)ii >= (uint64_t)a.num_in || (uint32_t)oo >= (uint32_t)tile_rows) {
-            ii = -1;
-            oo = -1;
-          }
-        }
-        s_in[tid] = ii;
-        s_out[tid] = oo;
-      }
-      f32x4 acc[TN / 16];
-#pragma unroll
-      for (int nb = 0; nb < TN / 16; ++nb) acc[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-      for (int c0 = 0; c0 < a.c_in_pad; c0 += CK) {
-        __syncthreads();  // s_in visible; previous channel chunk's MFMA reads are done
-        // stage the gathered input rows: RB rows x CK channels
-        if (vec_rows) {
-          for (int v = tid; v < RB * (CK / VEC); v += 256) {
-            const int r = v / (CK / VEC), cv = (v % (CK / VEC)) * VEC;
-            uint4 val = make_uint4(0u, 0u, 0u, 0u);
-            if (r < rows && c0 + cv < a.c_in && s_in[r] >= 0)
-              val = *reinterpret_cast<const uint4*>(X + (int64_t)s_in[r] * a.c_in + c0 + cv);
-            *reinterpret_cast<uint4*>(&As[r * LD + cv]) = val;
-          }
-        } else {
-          for (int e = tid; e < RB * CK; e += 256) {
-            const int r = e / CK, c = e % CK;
-            T val = from_float<T>(0.f);
-            if (r < rows && c0 + c < a.c_in && s_in[r] >= 0)
-              val = X[(int64_t)s_in[r] * a.c_in + c0 + c];
-            As[r * LD + c] = val;
-          }
-        }
-        // stage W[k]^T: TN output channels x CK input channels (already padded, always aligned)
-        for (int v = tid; v < TN * (CK / VEC); v += 256) {
-          const int n = v / (CK / VEC), cv = (v % (CK / VEC)) * VEC;
-          const uint4 val = *reinterpret_cast<const uint4*>(
-              Wt + ((int64_t)k * a.c_out_pad + n0 + n) * a.c_in_pad + c0 + cv);
-          *reinterpret_cast<uint4*>(&Bs[n * LD + cv]) = val;
-        }
-        __syncthreads();
-        if (wave * 16 < rows) {
-          const T* a_row = &As[(wave * 16 + (lane & 15)) * LD];
-#pragma unroll
-          for (int nb = 0; nb < TN / 16; ++nb)
-            acc[nb] = mma_block(a_row, &Bs[(nb * 16 + (lane & 15)) * LD], lane, acc[nb]);
-        }
-      }
-      // add the chunk's products to the accumulator rows its pairs name (rows of one offset
-      // are distinct, so plain read-modify-write is race free)
-      if (wave * 16 < rows) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int row = wave * 16 + (lane >> 4) * 4 + r;
-          if (row < rows && s_out[row] >= 0) {
-            float* dst = &accs[s_out[row] * ACC_LD + (lane & 15)];
-#pragma unroll
-            for (int nb = 0; nb < TN / 16; ++nb) dst[nb * 16] += acc[nb][r];
-          }
-        }
-      }
-    }
+__device__ __forceinline__ int offset_of_pair(const int64_t* __restrict__ offsets, int K, int64_t p) {
+  int lo = 0, hi = K;  // largest k with offsets[k] <= p
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (offsets[mid] <= p) lo = mid; else hi = mid;
   }
-  __syncthreads();
+  return lo;
+}
 
-  // write the tile: bias add, one rounding to T
-  T* __restrict__ out = (T*)a.out;
-  const T* __restrict__ bias = (const T*)a.bias;
-  for (int e = tid; e < TM * TN; e += 256) {
-    const int r = e / TN, c = e % TN;
-    if (r < tile_rows && n0 + c < a.c_out) {
-      float v = accs[r * ACC_LD + c];
-      if (bias) v += to_float(bias[n0 + c]);
-      out[(m0 + r) * a.c_out + n0 + c] = from_float<T>(v);
+__global__ void __launch_bounds__(256) rows_clear(uint32_t* __restrict__ row_mask, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x)
+    row_mask[i] = 0u;
+}
+
+__global__ void __launch_bounds__(256) rows_mark(const int32_t* __restrict__ out_maps,
+                                                 const int64_t* __restrict__ offsets, int K,
+                                                 int words, int64_t num_out,
+                                                 uint32_t* __restrict__ row_mask) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= offsets[K]) return;
+  const int k = offset_of_pair(offsets, K, p);
+  const int32_t o = out_maps[p];
+  if ((uint32_t)o < (uint64_t)num_out) atomicOr(&row_mask[(int64_t)o * words + (k >> 5)], 1u << (k & 31));
+}
+
+template <bool WRITE_PTR>
+__global__ void __launch_bounds__(256) rows_count(const uint32_t* __restrict__ row_mask, int words,
+                                                  int64_t num_out, int32_t* __restrict__ groups,
+                                                  int32_t* __restrict__ row_ptr) {
+  const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t group = m >> 6;
+  if (group >= (num_out + 63) / 64) return;
+  int cnt = 0;
+  if (m < num_out)
+    for (int w = 0; w < words; ++w) cnt += __popc(row_mask[m * words + w]);
+  const int incl = wcn_wave_inclusive_sum(cnt);
+  if (!WRITE_PTR) {
+    if (wcn_lane() == 63) groups[group] = incl;
+  } else if (m < num_out) {
+    row_ptr[m] = groups[group] + incl - cnt;
+    if (m == num_out - 1) row_ptr[num_out] = groups[group] + incl;
+  }
+}
+
+__global__ void __launch_bounds__(256) rows_fill(const int32_t* __restrict__ in_maps,
+                                                 const int32_t* __restrict__ out_maps,
+                                                 const int64_t* __restrict__ offsets, int K,
+                                                 int words, int64_t num_out,
+                                                 const uint32_t* __restrict__ row_mask,
+                                                 const int32_t* __restrict__ row_ptr,
+                                                 int32_t* __restrict__ row_in) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= offsets[K]) return;
+  const int k = offset_of_pair(offsets, K, p);
+  const int32_t o = out_maps[p];
+  if ((uint32_t)o >= (uint64_t)num_out) return;
+  const uint32_t* mw = row_mask + (int64_t)o * words;
+  int rank = 0;
+  for (int w = 0; w < (k >> 5); ++w) rank += __popc(mw[w]);
+  rank += __popc(mw[k >> 5] & ((1u << (k & 31)) - 1u));
+  row_in[row_ptr[o] + rank] = in_maps[p];
+}
+
+// Output-row form -> pair lists that ascend in output row inside every offset, plus their
+// group_start table.  Same two-pass scheme as the map builder: per (offset, 64-row group) hit
+// counts by ballot, row-wise scan, then every hit lane writes its pair at start + prefix.
+template <bool FILL>
+__global__ void __launch_bounds__(256) rows_to_pairs(const uint32_t* __restrict__ row_mask,
+                                                     const int32_t* __restrict__ row_ptr,
+                                                     const int32_t* __restrict__ row_in, int K,
+                                                     int words, int64_t num_out,
+                                                     const int64_t* __restrict__ offsets,
+                                                     int32_t* __restrict__ gs, int64_t G,
+                                                     int32_t* __restrict__ in_sorted,
+                                                     int32_t* __restrict__ out_sorted) {
+  const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t group = m >> 6;
+  if (group >= G) return;
+  const int lane = wcn_lane();
+  const bool live = m < num_out;
+  int rank = live ? row_ptr[m] : 0;
+  for (int w = 0; w < words; ++w) {
+    const uint32_t word = live ? row_mask[m * words + w] : 0u;
+    const int nbits = K - w * 32 < 32 ? K - w * 32 : 32;
+    for (int b = 0; b < nbits; ++b) {
+      const int k = w * 32 + b;
+      const bool hit = (word >> b) & 1u;
+      const unsigned long long hits = __ballot(hit);
+      if (!FILL) {
+        if (lane == 0) gs[(int64_t)k * (G + 1) + group] = __popcll(hits);
+      } else if (hit) {
+        const int64_t p = offsets[k] + gs[(int64_t)k * (G + 1) + group] +
+                          __popcll(hits & ((1ull << lane) - 1ull));
+        in_sorted[p] = row_in[rank++];
+        out_sorted[p] = (int32_t)m;
+      }
     }
   }
 }
 
 inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
+inline size_t elem_size(int dtype) { return dtype == WCN_DTYPE_F32 ? 4 : 2; }
+inline int ck_of(int dtype) { return dtype == WCN_DTYPE_F32 ? Mma<float>::CK : Mma<_Float16>::CK; }
 
 struct ConvWorkspace {
-  int64_t* offsets;      // K+1
-  int32_t* group_start;  // (K, G+1)
+  int64_t* offsets;      // K+1 (device copy of the host offsets)
   void* Wt;              // K * c_out_pad * c_in_pad elements
+  int32_t* group_start;  // (K, G+1), when not supplied by the caller
+  int64_t* row_total;    // K+1 scratch of the scans
+  uint32_t* row_mask;    // the rest only when the pair lists have to be re-ordered here
+  int32_t* row_ptr;
+  int32_t* row_in;
+  int32_t* groups;
+  int32_t* in_sorted;
+  int32_t* out_sorted;
+  int c_in_pad, c_out_pad, words;
   int64_t G;
-  int c_in_pad, c_out_pad;
 };
 
-inline size_t elem_size(int dtype) { return dtype == WCN_DTYPE_F32 ? 4 : 2; }
-
-inline int ck_of(int dtype) { return dtype == WCN_DTYPE_F32 ? Cfg<float>::CK : Cfg<_Float16>::CK; }
-
 inline size_t conv_layout(void* base, int64_t num_out, int K, int c_in, int c_out, int dtype,
-                          ConvWorkspace* w) {
+                          int64_t resort_pairs, ConvWorkspace* w) {
   char* p = (char*)base;
   size_t off = 0;
   const int64_t G = (num_out + 63) / 64;
+  const int words = (K + 31) / 32;
   const int cip = round_up(c_in, ck_of(dtype)), cop = round_up(c_out, TN);
   if (w) w->offsets = (int64_t*)(p + off);
   off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
-  if (w) w->group_start = (int32_t*)(p + off);
-  off += wcn_align256(sizeof(int32_t) * (size_t)K * (size_t)(G + 1));
   if (w) w->Wt = (void*)(p + off);
   off += wcn_align256(elem_size(dtype) * (size_t)K * cop * cip);
+  if (w) w->group_start = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)K * (size_t)(G + 1));
+  if (w) w->row_total = (int64_t*)(p + off);
+  off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
+  if (resort_pairs >= 0) {
+    if (w) w->row_mask = (uint32_t*)(p + off);
+    off += wcn_align256(sizeof(uint32_t) * (size_t)num_out * words);
+    if (w) w->row_ptr = (int32_t*)(p + off);
+    off += wcn_align256(sizeof(int32_t) * (size_t)(num_out + 1));
+    if (w) w->row_in = (int32_t*)(p + off);
+    off += wcn_align256(sizeof(int32_t) * (size_t)resort_pairs);
+    if (w) w->groups = (int32_t*)(p + off);
+    off += wcn_align256(sizeof(int32_t) * (size_t)(G + 1));
+    if (w) w->in_sorted = (int32_t*)(p + off);
+    off += wcn_align256(sizeof(int32_t) * (size_t)resort_pairs);
+    if (w) w->out_sorted = (int32_t*)(p + off);
+    off += wcn_align256(sizeof(int32_t) * (size_t)resort_pairs);
+  }
   if (w) {
     w->G = G;
     w->c_in_pad = cip;
     w->c_out_pad = cop;
+    w->words = words;
   }
   return off;
 }
@@ -322,9 +576,9 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
                        (const float*)weight, a.K, a.c_in, a.c_out, a.c_in_pad, a.c_out_pad,
                        (T*)a.Wt);
   }
-  const dim3 grid((unsigned)((a.num_out + TM - 1) / TM), (unsigned)(a.c_out_pad / TN));
+  const dim3 grid((unsigned)((a.num_out + ROWS - 1) / ROWS), (unsigned)(a.c_out_pad / TN));
   if (g_time_start) (void)hipEventRecord(g_time_start, s);
-  hipLaunchKernelGGL(conv_fwd<T>, grid, dim3(256), 0, s, a);
+  hipLaunchKernelGGL(conv_fwd<T>, grid, dim3(THREADS), 0, s, a);
   if (g_time_stop) (void)hipEventRecord(g_time_stop, s);
   g_time_start = g_time_stop = nullptr;
   WCN_LAUNCH_CHECK();
@@ -342,54 +596,90 @@ int wcn_conv_set_timing_events(void* start_event, void* stop_event) {
 }
 
 size_t wcn_conv_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_in, int32_t c_out,
-                                int32_t dtype) {
-  if (num_out < 0 || num_offsets < 1 || c_in < 1 || c_out < 1 || dtype < 0 || dtype > 2) return 0;
-  return conv_layout(nullptr, num_out, num_offsets, c_in, c_out, dtype, nullptr);
+                                int32_t dtype, int64_t num_pairs, int32_t out_maps_ascend) {
+  if (num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || c_in < 1 || c_out < 1 ||
+      dtype < 0 || dtype > 2 || num_pairs < 0)
+    return 0;
+  return conv_layout(nullptr, num_out, num_offsets, c_in, c_out, dtype,
+                     out_maps_ascend ? -1 : num_pairs, nullptr);
 }
 
 int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
                         const void* weight, int32_t weight_dtype, int32_t num_offsets,
                         int32_t c_out, const void* bias_or_null, const int32_t* in_maps,
                         const int32_t* out_maps, const int64_t* host_offsets,
-                        int32_t identity_offset, const int32_t* group_start_or_null, void* out,
-                        int64_t num_out, void* workspace, size_t workspace_bytes, void* stream) {
+                        int32_t identity_offset, int32_t out_maps_ascend,
+                        const int32_t* group_start_or_null, void* out, int64_t num_out,
+                        void* workspace, size_t workspace_bytes, void* stream) {
   if (dtype < 0 || dtype > 2 || (weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32))
     return WCN_ERR_INVALID_ARGUMENT;
-  if (num_in < 0 || num_out < 0 || num_offsets < 1 || c_in < 1 || c_out < 1 || !weight ||
-      !host_offsets || !workspace)
+  if (num_in < 0 || num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || c_in < 1 ||
+      c_out < 1 || !weight || !workspace || !host_offsets)
     return WCN_ERR_INVALID_ARGUMENT;
   if (num_in >= (1ll << 31) || num_out >= (1ll << 31)) return WCN_ERR_INVALID_ARGUMENT;
   if (identity_offset >= num_offsets) return WCN_ERR_INVALID_ARGUMENT;
-  if (num_out == 0) return WCN_OK;
-  if (!out || (num_in > 0 && !features)) return WCN_ERR_INVALID_ARGUMENT;
+  if (group_start_or_null && !out_maps_ascend) return WCN_ERR_INVALID_ARGUMENT;
   const int64_t L = host_offsets[num_offsets];
-  if (host_offsets[0] != 0 || L < 0) return WCN_ERR_INVALID_ARGUMENT;
+  if (host_offsets[0] != 0 || L < 0 || L > INT32_MAX) return WCN_ERR_INVALID_ARGUMENT;
   for (int k = 0; k < num_offsets; ++k)
     if (host_offsets[k + 1] < host_offsets[k]) return WCN_ERR_INVALID_ARGUMENT;
   if (L > 0 && (!in_maps || !out_maps)) return WCN_ERR_INVALID_ARGUMENT;
-  if (workspace_bytes < wcn_conv_workspace_bytes(num_out, num_offsets, c_in, c_out, dtype))
+  if (num_out == 0) return WCN_OK;
+  if (!out || (num_in > 0 && !features)) return WCN_ERR_INVALID_ARGUMENT;
+  if (workspace_bytes <
+      wcn_conv_workspace_bytes(num_out, num_offsets, c_in, c_out, dtype, L, out_maps_ascend))
     return WCN_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   ConvWorkspace w;
-  conv_layout(workspace, num_out, num_offsets, c_in, c_out, dtype, &w);
+  conv_layout(workspace, num_out, num_offsets, c_in, c_out, dtype, out_maps_ascend ? -1 : L, &w);
   if (hipMemcpyAsync(w.offsets, host_offsets, sizeof(int64_t) * (size_t)(num_offsets + 1),
                      hipMemcpyHostToDevice, s) != hipSuccess)
     return WCN_ERR_LAUNCH;
-  const int32_t* gs = group_start_or_null;
-  if (!gs) {
+
+  ConvArgs a;
+  a.in_maps = in_maps;
+  a.out_maps = out_maps;
+  a.group_start = group_start_or_null;
+  const unsigned rows_grid = (unsigned)((num_out + 255) / 256);
+  if (!out_maps_ascend) {
+    // pair lists -> output-row form -> pair lists ascending in output row, with group_start
+    const int64_t mask_words = num_out * w.words;
+    hipLaunchKernelGGL(rows_clear, dim3((unsigned)std::min<int64_t>(4096, (mask_words + 255) / 256)),
+                       dim3(256), 0, s, w.row_mask, mask_words);
+    if (L > 0)
+      hipLaunchKernelGGL(rows_mark, dim3((unsigned)((L + 255) / 256)), dim3(256), 0, s, out_maps,
+                         (const int64_t*)w.offsets, num_offsets, w.words, num_out, w.row_mask);
+    hipLaunchKernelGGL(rows_count<false>, dim3(rows_grid), dim3(256), 0, s,
+                       (const uint32_t*)w.row_mask, w.words, num_out, w.groups, w.row_ptr);
+    wcn_scan_rows_launch(w.groups, w.G, 1, w.row_total, s);
+    hipLaunchKernelGGL(rows_count<true>, dim3(rows_grid), dim3(256), 0, s,
+                       (const uint32_t*)w.row_mask, w.words, num_out, w.groups, w.row_ptr);
+    if (L > 0)
+      hipLaunchKernelGGL(rows_fill, dim3((unsigned)((L + 255) / 256)), dim3(256), 0, s, in_maps,
+                         out_maps, (const int64_t*)w.offsets, num_offsets, w.words, num_out,
+                         (const uint32_t*)w.row_mask, (const int32_t*)w.row_ptr, w.row_in);
+    hipLaunchKernelGGL(rows_to_pairs<false>, dim3(rows_grid), dim3(256), 0, s,
+                       (const uint32_t*)w.row_mask, (const int32_t*)w.row_ptr,
+                       (const int32_t*)w.row_in, num_offsets, w.words, num_out,
+                       (const int64_t*)w.offsets, w.group_start, w.G, w.in_sorted, w.out_sorted);
+    wcn_scan_rows_launch(w.group_start, w.G, num_offsets, w.row_total, s);
+    hipLaunchKernelGGL(rows_to_pairs<true>, dim3(rows_grid), dim3(256), 0, s,
+                       (const uint32_t*)w.row_mask, (const int32_t*)w.row_ptr,
+                       (const int32_t*)w.row_in, num_offsets, w.words, num_out,
+                       (const int64_t*)w.offsets, w.group_start, w.G, w.in_sorted, w.out_sorted);
+    a.in_maps = w.in_sorted;
+    a.out_maps = w.out_sorted;
+    a.group_start = w.group_start;
+  } else if (!a.group_start) {
     const int64_t items = (int64_t)num_offsets * (w.G + 1);
     hipLaunchKernelGGL(conv_group_start, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
                        out_maps, (const int64_t*)w.offsets, num_offsets, w.G, w.group_start);
-    gs = w.group_start;
+    a.group_start = w.group_start;
   }
-  ConvArgs a;
+  a.offsets = w.offsets;
   a.X = features;
   a.Wt = w.Wt;
   a.bias = bias_or_null;
-  a.in_maps = in_maps;
-  a.out_maps = out_maps;
-  a.offsets = w.offsets;
-  a.group_start = gs;
   a.out = out;
   a.num_in = num_in;
   a.num_out = num_out;
@@ -400,7 +690,9 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
   a.c_in_pad = w.c_in_pad;
   a.c_out_pad = w.c_out_pad;
   a.identity = identity_offset;
-  a.vec_rows = (((size_t)c_in * elem_size(dtype)) % 16 == 0 && ((uintptr_t)features % 16) == 0) ? 1 : 0;
+  const size_t es = elem_size(dtype);
+  a.vec_in = (((size_t)c_in * es) % 16 == 0 && ((uintptr_t)features % 16) == 0) ? 1 : 0;
+  a.vec_out = (((size_t)c_out * es) % 16 == 0 && ((uintptr_t)out % 16) == 0) ? 1 : 0;
   switch (dtype) {
     case WCN_DTYPE_F32: return launch_conv<float>(a, weight, weight_dtype, dtype, s);
     case WCN_DTYPE_F16: return launch_conv<_Float16>(a, weight, weight_dtype, dtype, s);

@@ -1,7 +1,7 @@
 // Kernel-map generation and strided output coordinates on top of the block table (gfx950).
 //
 // The reference materialises a dense (K, M) table of probe results and compacts it with several
-// passes (torch_discrete.py:80-157).  Here one thread owns one output voxel and walks the K
+// passes (torch_discrete.py:80-157).  Here one thread owns one output voxel and resolves its K
 // offsets in registers; a wave's 64 voxels form a "group".  Pass 1 (count) stores, per offset and
 // group, how many of the 64 probes hit (a ballot popcount); a row-wise exclusive scan turns the
 // counts into start positions; pass 2 (fill) repeats the probes and each lane writes its pair at
@@ -24,8 +24,10 @@ struct KmapGeom {
 };
 
 struct KmapWorkspace {  // host-computed addresses inside a kmap workspace
-  int64_t* result;      // [K+1] offsets, [K+1] = table status bits, [K+2] = occupied slots
-  int32_t* groups;      // (K, G+1): counts after pass 1, exclusive prefix sums after the scan
+  int64_t* result;      // [0..K] offsets, [K+1] = table status bits, [K+2] = occupied slots
+  int64_t* row_total;   // [K+1] totals of the rows of `groups`
+  int32_t* groups;      // (K+1, G+1): rows 0..K-1 per-offset hit counts of each 64-row group, row K
+                        // all hits of the group; after the scan, exclusive prefix sums
   int64_t G;            // number of 64-row groups
 };
 
@@ -35,8 +37,10 @@ inline size_t kmap_layout(void* base, int64_t num_out, int32_t K, KmapWorkspace*
   const int64_t G = (num_out + 63) / 64;
   if (w) w->result = (int64_t*)(p + off);
   off += wcn_align256(sizeof(int64_t) * (size_t)(K + 3));
+  if (w) w->row_total = (int64_t*)(p + off);
+  off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
   if (w) w->groups = (int32_t*)(p + off);
-  off += wcn_align256(sizeof(int32_t) * (size_t)K * (size_t)(G + 1));
+  off += wcn_align256(sizeof(int32_t) * (size_t)(K + 1) * (size_t)(G + 1));
   if (w) w->G = G;
   return off;
 }
@@ -46,9 +50,14 @@ inline int grid_for(int64_t n, int block) {
   return (int)(g < 1 ? 1 : g);
 }
 
-// Probe results of one output voxel are produced offset by offset; consecutive offsets differ in
-// z (the fastest digit) and mostly fall in the block of the previous probe, whose slot is kept
-// in registers, so a 3x3x3 neighbourhood costs a handful of table reads, not 27.
+struct KmapOut {        // outputs of the fill pass (all may be null in the count pass)
+  int32_t* in_maps;
+  int32_t* out_maps;
+};
+
+// ---- generic kernel: any kernel size up to WCN_MAX_OFFSETS offsets -----------------------------
+// Probe results are produced offset by offset; consecutive offsets differ in z (the fastest
+// digit) and mostly fall in the block of the previous probe, whose slot is kept in registers.
 template <bool FILL>
 __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restrict__ hdr,
                                                  const WcnSlot* __restrict__ slots,
@@ -57,9 +66,7 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
                                                  const int4* __restrict__ out_coords,
                                                  int64_t num_out, KmapGeom g,
                                                  int32_t* __restrict__ groups, int64_t G,
-                                                 const int64_t* __restrict__ offsets,
-                                                 int32_t* __restrict__ in_maps,
-                                                 int32_t* __restrict__ out_maps) {
+                                                 const int64_t* __restrict__ offsets, KmapOut o) {
   const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t group = m >> 6;  // wave-uniform
   if (group >= G) return;
@@ -77,7 +84,7 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
 
   unsigned long long cached_key = WCN_EMPTY_KEY, cached_mask = 0ull;
   int32_t cached_base = 0;
-  int k = 0;
+  int k = 0, group_hits = 0;
   for (int i = 0; i < g.kx; ++i) {
     for (int j = 0; j < g.ky; ++j) {
       for (int kk = 0; kk < g.kz; ++kk, ++k) {
@@ -94,60 +101,212 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
         }
         const unsigned long long hits = __ballot(found >= 0);
         if (!FILL) {
-          if (lane == 0) groups[(int64_t)k * (G + 1) + group] = __popcll(hits);
+          const int cnt = __popcll(hits);
+          group_hits += cnt;
+          if (lane == 0) groups[(int64_t)k * (G + 1) + group] = cnt;
         } else if (found >= 0) {
           const int64_t pos = offsets[k] + groups[(int64_t)k * (G + 1) + group] +
                               __popcll(hits & ((1ull << lane) - 1ull));
-          in_maps[pos] = found;
-          out_maps[pos] = (int32_t)m;
+          o.in_maps[pos] = found;
+          o.out_maps[pos] = (int32_t)m;
         }
       }
+    }
+  }
+  if (!FILL && lane == 0) groups[(int64_t)g.K * (G + 1) + group] = group_hits;
+}
+
+// ---- fixed-size kernel: compile-time kernel size, every dimension spans at most 2 blocks -------
+// Phase 1 requests the (up to) 8 block slots the neighbourhood can touch, all at once, so their
+// memory latencies overlap; phase 2 derives the hit bit of each of the K offsets from the cached
+// masks (no memory traffic); phase 3 (fill only) reads the hit rows from `perm`, again as
+// independent loads, and writes both forms of the map.
+template <int KX, int KY, int KZ, bool FILL>
+__global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __restrict__ hdr,
+                                                       const WcnSlot* __restrict__ slots,
+                                                       uint32_t cap_mask,
+                                                       const int32_t* __restrict__ perm,
+                                                       const int4* __restrict__ out_coords,
+                                                       int64_t num_out, KmapGeom g,
+                                                       int32_t* __restrict__ groups, int64_t G,
+                                                       const int64_t* __restrict__ offsets,
+                                                       KmapOut o) {
+  constexpr int K = KX * KY * KZ;
+  static_assert(K <= 32 && KX <= 5 && KY <= 5 && KZ <= 5, "fixed kernel covers small kernels");
+  __shared__ unsigned long long s_mask[8][256];
+  __shared__ int32_t s_base[8][256];
+  const int tid = threadIdx.x;
+  const int64_t m = (int64_t)blockIdx.x * blockDim.x + tid;
+  const int64_t group = m >> 6;  // wave-uniform
+  if (group >= G) return;
+  const int lane = wcn_lane();
+  const bool live = m < num_out;
+  const WcnLayout L = wcn_make_layout(hdr);
+  int4 c = make_int4(0, 0, 0, 0);
+  if (live) c = out_coords[m];
+  const uint32_t rb = (uint32_t)c.x - L.amin[0];
+  const uint32_t r0[3] = {(uint32_t)c.y * (uint32_t)g.sx - (uint32_t)g.cx - L.amin[1],
+                          (uint32_t)c.z * (uint32_t)g.sy - (uint32_t)g.cy - L.amin[2],
+                          (uint32_t)c.w * (uint32_t)g.sz - (uint32_t)g.cz - L.amin[3]};
+  const bool usable = live && L.ok && rb <= L.span[0];
+  constexpr int KD[3] = {KX, KY, KZ};
+
+  // candidate block coordinates per dimension: the block of the first neighbour and the next one
+  uint32_t cand[3][2];
+  bool cok[3][2];
+#pragma unroll
+  for (int d = 0; d < 3; ++d) {
+    const uint32_t lim = L.span[d + 1] >> 2;
+    cand[d][0] = r0[d] >> 2;
+    cand[d][1] = (r0[d] + 4u) >> 2;
+    cok[d][0] = cand[d][0] <= lim;
+    cok[d][1] = cand[d][1] <= lim && ((r0[d] & 3u) + (uint32_t)(KD[d] - 1)) >= 4u;
+  }
+  unsigned long long key[8];
+  uint32_t hh[8];
+  bool need[8];
+  uint4 lo[8], hi[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int dx = e >> 2, dy = (e >> 1) & 1, dz = e & 1;
+    need[e] = usable && cok[0][dx] && cok[1][dy] && cok[2][dz];
+    key[e] = ((unsigned long long)rb << L.shift[0]) |
+             ((unsigned long long)cand[0][dx] << L.shift[1]) |
+             ((unsigned long long)cand[1][dy] << L.shift[2]) | (unsigned long long)cand[2][dz];
+    hh[e] = wcn_mix(key[e], cap_mask);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    lo[e] = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0u, 0u);
+    hi[e] = make_uint4(0u, 0u, 0u, 0u);
+    if (need[e]) {
+      const uint4* raw = reinterpret_cast<const uint4*>(&slots[hh[e]]);
+      lo[e] = raw[0];
+      hi[e] = raw[1];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    unsigned long long mask = 0ull;
+    int32_t base = 0;
+    if (need[e]) {
+      const unsigned long long k0 = ((unsigned long long)lo[e].y << 32) | lo[e].x;
+      if (k0 == key[e]) {
+        mask = ((unsigned long long)lo[e].w << 32) | lo[e].z;
+        base = (int32_t)hi[e].x;
+      } else if (k0 != WCN_EMPTY_KEY) {  // collision on the first probe: walk on
+        mask = wcn_lookup_block_from(slots, cap_mask, key[e], (hh[e] + 1) & cap_mask, 1, &base);
+      }
+    }
+    s_mask[e][tid] = mask;
+    s_base[e][tid] = base;
+  }
+  // no barrier: every thread reads back only its own column
+
+  uint32_t hm = 0;
+  int32_t pos[K];
+  {
+    int k = 0;
+#pragma unroll
+    for (int i = 0; i < KX; ++i) {
+#pragma unroll
+      for (int j = 0; j < KY; ++j) {
+#pragma unroll
+        for (int kk = 0; kk < KZ; ++kk, ++k) {
+          const uint32_t ax = (r0[0] & 3u) + i, ay = (r0[1] & 3u) + j, az = (r0[2] & 3u) + kk;
+          const int e = (int)(((ax >> 2) << 2) | ((ay >> 2) << 1) | (az >> 2));
+          const uint32_t bit = ((ax & 3u) << 4) | ((ay & 3u) << 2) | (az & 3u);
+          const unsigned long long mk = s_mask[e][tid];
+          const uint32_t hit = (uint32_t)((mk >> bit) & 1ull);
+          hm |= hit << k;
+          if (FILL) pos[k] = s_base[e][tid] + wcn_rank_below(mk, bit);
+        }
+      }
+    }
+  }
+
+  if (!FILL) {
+    int group_hits = 0;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int cnt = __popcll(__ballot((hm >> k) & 1u));
+      group_hits += cnt;
+      if (lane == 0) groups[(int64_t)k * (G + 1) + group] = cnt;
+    }
+    if (lane == 0) groups[(int64_t)K * (G + 1) + group] = group_hits;
+    return;
+  }
+
+  int32_t found[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) found[k] = ((hm >> k) & 1u) ? perm[pos[k]] : -1;
+
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const bool hit = (hm >> k) & 1u;
+    const unsigned long long hits = __ballot(hit);
+    if (hit) {
+      const int64_t p = offsets[k] + groups[(int64_t)k * (G + 1) + group] +
+                        __popcll(hits & ((1ull << lane) - 1ull));
+      o.in_maps[p] = found[k];
+      o.out_maps[p] = (int32_t)m;
     }
   }
 }
 
 // In-place exclusive prefix sum of each row of `groups` (one workgroup per row, G+1 entries; the
 // last entry receives the row total).
-__global__ void __launch_bounds__(256) kmap_scan_rows(int32_t* __restrict__ groups, int64_t G,
-                                                      int64_t* __restrict__ row_total) {
-  __shared__ int s_wave[4];
+__global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ groups, int64_t G,
+                                                       int64_t* __restrict__ row_total) {
+  __shared__ int s_wave[16];
   int32_t* row = groups + (int64_t)blockIdx.x * (G + 1);
   const int lane = wcn_lane(), wave = threadIdx.x >> 6;
   int64_t carry = 0;
-  for (int64_t start = 0; start < G; start += 256) {
-    const int64_t idx = start + threadIdx.x;
-    const int v = idx < G ? row[idx] : 0;
-    const int incl = wcn_wave_inclusive_sum(v);
+  for (int64_t start = 0; start < G; start += 4096) {
+    const int64_t idx = start + (int64_t)threadIdx.x * 4;
+    int v[4];
+    int sum = 0;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      v[t] = idx + t < G ? row[idx + t] : 0;
+      sum += v[t];
+    }
+    const int incl = wcn_wave_inclusive_sum(sum);
     if (lane == 63) s_wave[wave] = incl;
     __syncthreads();
     int before = 0, all = 0;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < 16; ++w) {
       const int t = s_wave[w];
       if (w < wave) before += t;
       all += t;
     }
-    if (idx < G) row[idx] = (int32_t)(carry + before + incl - v);
+    int run = (int)carry + before + incl - sum;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (idx + t < G) row[idx + t] = run;
+      run += v[t];
+    }
     carry += all;
     __syncthreads();
   }
   if (threadIdx.x == 0) {
-    // a row holds at most M < 2^31 pairs, so the int32 entries cannot overflow
+    // a row of the per-offset counts holds at most M < 2^31 pairs; the row of all hits can
+    // exceed int32, which the host turns into WCN_ERR_TOO_MANY_PAIRS
     row[G] = (int32_t)carry;
     row_total[blockIdx.x] = carry;
   }
 }
 
 // offsets[K+1] = exclusive prefix sum of the row totals; also copies the table's status out so
-// the host needs one read for everything.  Single workgroup, serial over K <= 1024 (tiny).
-__global__ void kmap_finish(int64_t* __restrict__ result, int32_t K,
-                            const WcnTableHeader* __restrict__ hdr) {
+// the host needs one read for everything.  Serial over K <= 1024 (tiny).
+__global__ void kmap_finish(int64_t* __restrict__ result, const int64_t* __restrict__ row_total,
+                            int32_t K, const WcnTableHeader* __restrict__ hdr) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  // result[1..K] currently hold the row totals (written at result[k+1] by the scan)
   int64_t run = 0;
   result[0] = 0;
   for (int k = 0; k < K; ++k) {
-    run += result[k + 1];
+    run += row_total[k];
     result[k + 1] = run;
   }
   result[K + 1] = hdr->status;
@@ -169,8 +328,32 @@ bool make_geom(const int32_t ks[3], const int32_t st[3], KmapGeom* g) {
   return true;
 }
 
+inline bool is_fixed_size(const KmapGeom& g, int x, int y, int z) {
+  return g.kx == x && g.ky == y && g.kz == z;
+}
+
 inline bool table_args_ok(const void* table, int64_t n_keys, int64_t capacity) {
   return table && n_keys >= 0 && capacity >= 64 && (capacity & (capacity - 1)) == 0;
+}
+
+template <bool FILL>
+void launch_pass(const WcnTableView& v, const int32_t* out_coords, int64_t num_out,
+                 const KmapGeom& g, const KmapWorkspace& w, const KmapOut& o, hipStream_t s) {
+  const dim3 grid(grid_for(num_out, 256)), block(256);
+  const uint32_t cap_mask = (uint32_t)(v.capacity - 1);
+  const int64_t* offsets = FILL ? (const int64_t*)w.result : nullptr;
+  if (is_fixed_size(g, 3, 3, 3)) {
+    hipLaunchKernelGGL((kmap_pass_fixed<3, 3, 3, FILL>), grid, block, 0, s, v.hdr, v.slots,
+                       cap_mask, v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G,
+                       offsets, o);
+  } else if (is_fixed_size(g, 2, 2, 2)) {
+    hipLaunchKernelGGL((kmap_pass_fixed<2, 2, 2, FILL>), grid, block, 0, s, v.hdr, v.slots,
+                       cap_mask, v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G,
+                       offsets, o);
+  } else {
+    hipLaunchKernelGGL(kmap_pass<FILL>, grid, block, 0, s, v.hdr, v.slots, cap_mask, v.perm,
+                       (const int4*)out_coords, num_out, g, w.groups, w.G, offsets, o);
+  }
 }
 
 // ---- strided output coordinates -----------------------------------------------------------------
@@ -261,6 +444,11 @@ __global__ void stride_finish(int64_t* __restrict__ result, const int32_t* __res
 
 }  // namespace
 
+// Row-wise exclusive scan, shared with the contraction's map conversion.
+void wcn_scan_rows_launch(int32_t* groups, int64_t G, int rows, int64_t* row_total, hipStream_t s) {
+  hipLaunchKernelGGL(kmap_scan_rows, dim3(rows), dim3(1024), 0, s, groups, G, row_total);
+}
+
 extern "C" {
 
 size_t wcn_kmap_workspace_bytes(int64_t num_out, int32_t num_offsets) {
@@ -281,14 +469,10 @@ int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const in
   wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
   KmapWorkspace w;
   kmap_layout(workspace, num_out, g.K, &w);
-  if (w.G > 0) {
-    hipLaunchKernelGGL(kmap_pass<false>, dim3(grid_for(num_out, 256)), dim3(256), 0, s, v.hdr,
-                       v.slots, (uint32_t)(capacity - 1), v.perm, (const int4*)out_coords, num_out,
-                       g, w.groups, w.G, (const int64_t*)nullptr, (int32_t*)nullptr,
-                       (int32_t*)nullptr);
-  }
-  hipLaunchKernelGGL(kmap_scan_rows, dim3(g.K), dim3(256), 0, s, w.groups, w.G, w.result + 1);
-  hipLaunchKernelGGL(kmap_finish, dim3(1), dim3(64), 0, s, w.result, g.K, v.hdr);
+  const KmapOut none = {nullptr, nullptr};
+  if (w.G > 0) launch_pass<false>(v, out_coords, num_out, g, w, none, s);
+  hipLaunchKernelGGL(kmap_scan_rows, dim3(g.K + 1), dim3(1024), 0, s, w.groups, w.G, w.row_total);
+  hipLaunchKernelGGL(kmap_finish, dim3(1), dim3(64), 0, s, w.result, w.row_total, g.K, v.hdr);
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }
@@ -326,10 +510,8 @@ int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int
   wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
   KmapWorkspace w;
   kmap_layout(const_cast<void*>(workspace), num_out, g.K, &w);
-  hipLaunchKernelGGL(kmap_pass<true>, dim3(grid_for(num_out, 256)), dim3(256), 0,
-                     (hipStream_t)stream, v.hdr, v.slots, (uint32_t)(capacity - 1), v.perm,
-                     (const int4*)out_coords, num_out, g, w.groups, w.G, (const int64_t*)w.result,
-                     in_maps, out_maps);
+  const KmapOut o = {in_maps, out_maps};
+  launch_pass<true>(v, out_coords, num_out, g, w, o, (hipStream_t)stream);
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }
@@ -370,7 +552,7 @@ int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_strid
                        (const int4*)w.coarse, n, v.hdr, v.slots, v.slot_of, v.perm, w.groups, w.G,
                        (int4*)nullptr, (int32_t*)nullptr);
   }
-  hipLaunchKernelGGL(kmap_scan_rows, dim3(1), dim3(256), 0, s, w.groups, w.G, w.result + 2);
+  hipLaunchKernelGGL(kmap_scan_rows, dim3(1), dim3(1024), 0, s, w.groups, w.G, w.result + 2);
   hipLaunchKernelGGL(stride_finish, dim3(1), dim3(64), 0, s, w.result, w.groups, w.G, v.hdr);
   if (n > 0) {
     hipLaunchKernelGGL(stride_pick<true>, dim3(grid_for(n, 256)), dim3(256), 0, s,

@@ -4,7 +4,7 @@
 //   table_clear   header, slots and perm to their empty values
 //   table_bbox    bounding box of the keys (LDS reduction, one atomic min/max per workgroup)
 //   table_insert  per key: claim / find the block slot with a 64-bit CAS, OR the voxel bit in
-//   table_base    per occupied slot: base = running sum of block populations (one atomic per wave)
+//   table_base    per slot: base = running sum of block populations (one atomic per 1024 slots)
 //   table_perm    per key: perm[base + rank of its bit] = min(row index)
 //
 // HBM traffic per key: 16 B read (bbox) + 16 B read (insert) + 4 B slot_of write + 4 B read +
@@ -82,9 +82,7 @@ __global__ void __launch_bounds__(256) table_bbox(const int4* __restrict__ keys,
 __global__ void __launch_bounds__(256) table_insert(const int4* __restrict__ keys, int64_t n_keys,
                                                     WcnTableHeader* __restrict__ hdr,
                                                     WcnSlot* __restrict__ slots, uint32_t cap_mask,
-                                                    int32_t* __restrict__ slot_of,
-                                                    int32_t* __restrict__ block_list,
-                                                    int64_t block_list_len) {
+                                                    int32_t* __restrict__ slot_of) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n_keys) return;
   const WcnLayout L = wcn_make_layout(hdr);
@@ -105,11 +103,7 @@ __global__ void __launch_bounds__(256) table_insert(const int4* __restrict__ key
     unsigned long long seen = __atomic_load_n(&slots[h].key, __ATOMIC_RELAXED);
     if (seen == WCN_EMPTY_KEY) {
       seen = atomicCAS(&slots[h].key, WCN_EMPTY_KEY, key);
-      if (seen == WCN_EMPTY_KEY) {
-        const int32_t at = atomicAdd(&hdr->num_blocks, 1);
-        if (at < block_list_len) block_list[at] = (int32_t)h;
-        seen = key;
-      }
+      if (seen == WCN_EMPTY_KEY) seen = key;  // this thread claimed the slot
     }
     if (seen == key) {
       atomicOr(&slots[h].mask, bit);
@@ -122,25 +116,36 @@ __global__ void __launch_bounds__(256) table_insert(const int4* __restrict__ key
   slot_of[i] = placed;
 }
 
-__global__ void __launch_bounds__(256) table_base(WcnTableHeader* __restrict__ hdr,
-                                                  WcnSlot* __restrict__ slots,
-                                                  const int32_t* __restrict__ block_list,
-                                                  int64_t block_list_len) {
+// base of every occupied slot = running sum of block populations.  One pass over all slots;
+// a 1024-thread workgroup scans its slots and takes its share of the running sum with a single
+// atomic, so the counter sees capacity / 1024 updates.
+__global__ void __launch_bounds__(1024) table_base(WcnTableHeader* __restrict__ hdr,
+                                                   WcnSlot* __restrict__ slots, int64_t capacity) {
+  __shared__ int s_wave[16];
+  __shared__ int s_occ[16];
+  __shared__ int s_group_base;
   const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t nb = hdr->num_blocks;
-  if (nb > block_list_len) nb = block_list_len;
-  // whole waves leave together: the prefix sum below needs every lane of a live wave
-  if ((j & ~(int64_t)63) >= nb) return;
-  int32_t h = -1, cnt = 0;
-  if (j < nb) {
-    h = block_list[j];
-    cnt = __popcll(slots[h].mask);
-  }
+  const int lane = wcn_lane(), wave = threadIdx.x >> 6;
+  int cnt = 0;
+  if (j < capacity) cnt = __popcll(slots[j].mask);
   const int incl = wcn_wave_inclusive_sum(cnt);
-  int wave_base = 0;
-  if (wcn_lane() == 63) wave_base = atomicAdd(&hdr->total, incl);
-  wave_base = __shfl(wave_base, 63, 64);
-  if (h >= 0) slots[h].base = wave_base + incl - cnt;
+  const unsigned long long occupied = __ballot(cnt > 0);
+  if (lane == 63) s_wave[wave] = incl;
+  if (lane == 0) s_occ[wave] = __popcll(occupied);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int total = 0, occ = 0;
+    for (int w = 0; w < 16; ++w) {
+      const int t = s_wave[w];
+      s_wave[w] = total;  // exclusive prefix over the waves
+      total += t;
+      occ += s_occ[w];
+    }
+    s_group_base = total ? atomicAdd(&hdr->total, total) : 0;
+    if (occ) atomicAdd(&hdr->num_blocks, occ);
+  }
+  __syncthreads();
+  if (cnt > 0) slots[j].base = s_group_base + s_wave[wave] + incl - cnt;
 }
 
 __global__ void __launch_bounds__(256) table_perm(const int4* __restrict__ keys, int64_t n_keys,
@@ -198,7 +203,6 @@ inline int grid_for(int64_t n, int block, int cap = 1 << 20) {
 int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView& v,
                          hipStream_t s) {
   const uint32_t cap_mask = (uint32_t)(v.capacity - 1);
-  const int64_t list_len = v.capacity < n_keys ? v.capacity : n_keys;
   const int64_t clear_items = 2 * v.capacity > n_keys ? 2 * v.capacity : n_keys;
   hipLaunchKernelGGL(table_clear, dim3(grid_for(clear_items, 256, 4096)), dim3(256), 0, s, v.hdr,
                      v.slots, v.capacity, v.perm, n_keys);
@@ -206,10 +210,9 @@ int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView
     hipLaunchKernelGGL(table_bbox, dim3(grid_for(n_keys, 256 * 8, 2048)), dim3(256), 0, s,
                        (const int4*)keys, n_keys, v.hdr);
     hipLaunchKernelGGL(table_insert, dim3(grid_for(n_keys, 256)), dim3(256), 0, s,
-                       (const int4*)keys, n_keys, v.hdr, v.slots, cap_mask, v.slot_of,
-                       v.block_list, list_len);
-    hipLaunchKernelGGL(table_base, dim3(grid_for(list_len, 256)), dim3(256), 0, s, v.hdr, v.slots,
-                       v.block_list, list_len);
+                       (const int4*)keys, n_keys, v.hdr, v.slots, cap_mask, v.slot_of);
+    hipLaunchKernelGGL(table_base, dim3(grid_for(v.capacity, 1024)), dim3(1024), 0, s, v.hdr,
+                       v.slots, v.capacity);
     hipLaunchKernelGGL(table_perm, dim3(grid_for(n_keys, 256)), dim3(256), 0, s,
                        (const int4*)keys, n_keys, v.hdr, v.slots, v.slot_of, v.perm);
   }

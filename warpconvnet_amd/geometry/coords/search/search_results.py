@@ -24,11 +24,11 @@ class IntSearchResult:
         self.offsets = offsets
         self.identity_map_index = identity_map_index
         # Device-side helpers of the HIP contraction (not part of the reference interface):
-        # whether out_maps ascends inside every offset, and the per-64-row group starts the map
-        # builder produced as a by-product (None: the contraction derives them itself).
-        self._out_sorted: Optional[bool] = None
-        self._group_start: Optional[Tensor] = None
-        self._sorted_view: Optional["IntSearchResult"] = None
+        # whether out_maps ascends inside every offset (False: the contraction re-orders the
+        # pairs itself) and, from the map builder, (workspace, address, (K, M)) of the table of
+        # per-64-row group starts.
+        self._out_ascend = False
+        self._group_start = None
 
     @torch.no_grad()
     def __getitem__(self, idx: int) -> Tuple[Tensor, Tensor]:

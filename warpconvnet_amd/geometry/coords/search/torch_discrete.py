@@ -81,12 +81,10 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
                           ptr(out_maps), stream_ptr(device)), "wcn_kmap_fill")
     offsets = torch.tensor(list(host_offsets), dtype=torch.int32)
     result = IntSearchResult(in_maps, out_maps, offsets, identity_map_index=identity_map_index)
-    # by-products the contraction can reuse: pairs ascend in out index inside every offset, and
-    # the workspace holds the per-64-row group starts (kept alive by the reference below)
-    result._out_sorted = True
-    result._group_start = ws
-    result._group_start_ptr = L.wcn_kmap_group_start(ptr(ws), M, K)
-    result._group_start_shape = (K, M)
+    # by-products the contraction reuses: pairs ascend in output row inside every offset, and
+    # the workspace (kept alive by the reference below) holds their per-64-row group starts
+    result._out_ascend = True
+    result._group_start = (ws, L.wcn_kmap_group_start(ptr(ws), M, K), (K, M))
     return result
 
 
@@ -150,5 +148,5 @@ def generate_kernel_map(
         result = IntSearchResult(result.in_maps[:end], result.out_maps[:end],
                                  result.offsets[: half + 1].clone(),
                                  identity_map_index=identity_map_index)
-        result._out_sorted = True
+        result._out_ascend = True
     return result

@@ -64,29 +64,6 @@ def _is_random_order(order) -> bool:
 # ------------------------------------------------------------------------------------------------
 
 @torch.no_grad()
-def _sorted_by_out(kernel_map: IntSearchResult) -> IntSearchResult:
-    """A view of the map whose pairs ascend in out index inside every offset (what the device
-    contraction needs).  Maps from `generate_kernel_map` already do; the in/out-swapped map of a
-    transposed convolution does not and is reordered once, then cached on the map."""
-    if kernel_map._out_sorted:
-        return kernel_map
-    if kernel_map._sorted_view is not None:
-        return kernel_map._sorted_view
-    K = len(kernel_map)
-    offs = kernel_map.offsets.to(torch.int64)
-    counts = (offs[1:] - offs[:-1]).to(kernel_map.out_maps.device)
-    which = torch.repeat_interleave(torch.arange(K, device=counts.device), counts)
-    bound = int(kernel_map.out_maps.max().item()) + 1 if kernel_map.out_maps.numel() else 1
-    order = torch.argsort(which * bound + kernel_map.out_maps.long())
-    view = IntSearchResult(kernel_map.in_maps[order].contiguous(),
-                           kernel_map.out_maps[order].contiguous(), kernel_map.offsets,
-                           kernel_map.identity_map_index)
-    view._out_sorted = True
-    kernel_map._sorted_view = view
-    return view
-
-
-@torch.no_grad()
 def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSearchResult,
                         num_out_coords: int, bias: Optional[Tensor] = None,
                         compute_dtype: Optional[torch.dtype] = None) -> Tensor:
@@ -107,23 +84,25 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
         w = w.to(x.dtype)
     w = w.contiguous()
     b = None if bias is None else bias.detach().to(x.dtype).contiguous()
-    km = _sorted_by_out(kernel_map)
+    km = kernel_map
     K, c_in, c_out = w.shape
     device = x.device
     out = torch.empty((num_out_coords, c_out), dtype=x.dtype, device=device)
     L = lib()
-    nbytes = L.wcn_conv_workspace_bytes(num_out_coords, K, c_in, c_out, DTYPE_CODE[x.dtype])
+    ascend = 1 if km._out_ascend else 0
+    group_start = None
+    if ascend and km._group_start is not None and km._group_start[2] == (K, num_out_coords):
+        group_start = ctypes.c_void_p(km._group_start[1])
+    num_pairs = int(km.offsets[-1])
+    nbytes = L.wcn_conv_workspace_bytes(num_out_coords, K, c_in, c_out, DTYPE_CODE[x.dtype],
+                                        num_pairs, ascend)
     ws = workspace(nbytes, device)
     host_offsets = (ctypes.c_int64 * (K + 1))(*[int(v) for v in km.offsets.tolist()])
-    group_start = None
-    if getattr(km, "_group_start", None) is not None and \
-            getattr(km, "_group_start_shape", None) == (K, num_out_coords):
-        group_start = ctypes.c_void_p(km._group_start_ptr)
     iden = -1 if km.identity_map_index is None else int(km.identity_map_index)
     check(L.wcn_sparse_conv_fwd(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(w),
                                 DTYPE_CODE[w.dtype], K, c_out, ptr(b), ptr(km.in_maps),
-                                ptr(km.out_maps), host_offsets, iden, group_start, ptr(out),
-                                num_out_coords, ptr(ws), ws.numel(), stream_ptr(device)),
+                                ptr(km.out_maps), host_offsets, iden, ascend, group_start,
+                                ptr(out), num_out_coords, ptr(ws), ws.numel(), stream_ptr(device)),
           "wcn_sparse_conv_fwd")
     return out if out.dtype == in_features.dtype else out.to(in_features.dtype)
 
