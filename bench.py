@@ -24,6 +24,13 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
 
+# Bytes the contraction kernel moves between L2 and the memory fabric per launch on this workload,
+# from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch),
+# each scaled by what the same counter reads for the 1 GiB device copy of --calibrate-copy
+# (FETCH_SIZE reads 0.5 GiB for it -> x2.0; WRITE_SIZE reads 1 GiB -> x1.0).  Summary kept in
+# profiles/conv_fwd_cfg2_hbm_traffic.txt; to be re-measured whenever the kernel changes.
+CONV_FWD_TRAFFIC_BYTES = (277663 * 2.0 + 125000 * 1.0) * 1024
+
 METRIC = "voxels/sec, 3x3x3 C64->64 fp16 conv @1M voxels; kernel-map build ms"
 
 
@@ -76,6 +83,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this path is built and measured on a single MI355X; "
@@ -103,6 +112,13 @@ def main():
                                          ctypes.c_void_p(time_kernel[1].cuda_event))
         out = sparse_conv_forward(feats_d, weight_d, km, n)
         return km, out, mid
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         km, out, _ = step()
@@ -174,7 +190,8 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": CONV_FWD_TRAFFIC_BYTES,
+            "algorithmic_bytes": conv_bytes,
         },
     }
 

@@ -33,7 +33,8 @@ struct WcnTableHeader {  // first 256 bytes of a table workspace
   int32_t num_blocks;    // occupied slots
   int32_t status;        // WCN_DEV_* bits
   int32_t total;         // running sum of block populations (ends at the number of distinct keys)
-  int32_t reserved[53];
+  int32_t has_duplicates;  // some key was inserted more than once
+  int32_t reserved[52];
 };
 static_assert(sizeof(WcnTableHeader) == 256, "header is 256 bytes");
 

@@ -26,6 +26,7 @@ __global__ void __launch_bounds__(256) table_clear(WcnTableHeader* __restrict__ 
     hdr->num_blocks = 0;
     hdr->status = 0;
     hdr->total = 0;
+    hdr->has_duplicates = 0;
   }
   // each slot is two 16-byte stores: {EMPTY, 0} and {0, 0, 0, 0}
   uint4* raw = reinterpret_cast<uint4*>(slots);
@@ -95,18 +96,22 @@ __global__ void __launch_bounds__(256) table_insert(const int4* __restrict__ key
   uint32_t r[4];
   wcn_relative(L, c.x, c.y, c.z, c.w, r);  // always inside: the box was built from these keys
   const unsigned long long key = wcn_block_key(L, r);
-  const unsigned long long bit = 1ull << wcn_block_bit(r);
+  const uint32_t bit_index = wcn_block_bit(r);
+  const uint32_t bit = 1u << (bit_index & 31u);  // within the 32-bit half of the mask that holds it
   uint32_t h = wcn_mix(key, cap_mask);
   int32_t placed = -1;
   for (int p = 0; p < WCN_MAX_PROBE; ++p) {
     // cheap pre-read: most keys find their block already present
-    unsigned long long seen = __atomic_load_n(&slots[h].key, __ATOMIC_RELAXED);
+    // (a stale EMPTY from the vector cache only costs the CAS below; a non-empty key is final)
+    unsigned long long seen = *reinterpret_cast<const volatile unsigned long long*>(&slots[h].key);
     if (seen == WCN_EMPTY_KEY) {
       seen = atomicCAS(&slots[h].key, WCN_EMPTY_KEY, key);
       if (seen == WCN_EMPTY_KEY) seen = key;  // this thread claimed the slot
     }
     if (seen == key) {
-      atomicOr(&slots[h].mask, bit);
+      // a bit that is already set means the same coordinate was inserted before
+      uint32_t* half = reinterpret_cast<uint32_t*>(&slots[h].mask) + (bit_index >> 5);
+      if (atomicOr(half, bit) & bit) hdr->has_duplicates = 1;
       placed = (int32_t)h;
       break;
     }
@@ -163,7 +168,9 @@ __global__ void __launch_bounds__(256) table_perm(const int4* __restrict__ keys,
   wcn_relative(L, c.x, c.y, c.z, c.w, r);
   const ulonglong2 km = *reinterpret_cast<const ulonglong2*>(&slots[h]);
   const int32_t pos = slots[h].base + wcn_rank_below(km.y, wcn_block_bit(r));
-  if (pos >= 0 && pos < n_keys) atomicMin(&perm[pos], (int32_t)i);
+  if (pos < 0 || pos >= n_keys) return;
+  // without duplicate keys every position has exactly one writer
+  if (hdr->has_duplicates) atomicMin(&perm[pos], (int32_t)i); else perm[pos] = (int32_t)i;
 }
 
 __global__ void __launch_bounds__(256) table_query(const WcnTableHeader* __restrict__ hdr,
@@ -207,7 +214,7 @@ int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView
   hipLaunchKernelGGL(table_clear, dim3(grid_for(clear_items, 256, 4096)), dim3(256), 0, s, v.hdr,
                      v.slots, v.capacity, v.perm, n_keys);
   if (n_keys > 0) {
-    hipLaunchKernelGGL(table_bbox, dim3(grid_for(n_keys, 256 * 8, 2048)), dim3(256), 0, s,
+    hipLaunchKernelGGL(table_bbox, dim3(grid_for(n_keys, 256 * 16, 512)), dim3(256), 0, s,
                        (const int4*)keys, n_keys, v.hdr);
     hipLaunchKernelGGL(table_insert, dim3(grid_for(n_keys, 256)), dim3(256), 0, s,
                        (const int4*)keys, n_keys, v.hdr, v.slots, cap_mask, v.slot_of);
@@ -247,7 +254,7 @@ int64_t wcn_table_default_capacity(int64_t n_keys) {
   // Blocks hold up to 64 voxels; surface-like data fills ~10 per block.  One slot per two keys
   // keeps the load factor under 0.5 unless almost every voxel is alone in its block, in which
   // case the build reports WCN_ERR_TABLE_OVERFLOW and the caller retries with 4x the slots.
-  int64_t want = n_keys / 2 + 1;
+  int64_t want = n_keys + 1;
   int64_t cap = 1024;
   while (cap < want) cap <<= 1;
   return cap;
