@@ -1,0 +1,124 @@
+"""The benchmark configurations at (or near) their full sizes, checked through properties that do
+not need the CPU oracle to finish: identity weights, neighbour sums against torch index_add, the
+explicit per-offset algorithm written with plain torch fp32 operations on the GPU, and the map
+invariants of the strided / transposed pair."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import kaiming_weight, rel_err
+from warpconvnet_amd.utils import synthetic
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def torch_explicit_fp32(x, w, km, num_out):
+    """Plain torch fp32 restatement of the per-offset gather-GEMM-scatter on the GPU."""
+    out = torch.zeros(num_out, w.shape[-1], dtype=torch.float32, device=x.device)
+    xf, wf = x.float(), w.float()
+    for k in range(len(km)):
+        im, om = km[k]
+        if im.numel():
+            out.index_add_(0, om.long(), xf[im.long()] @ wf[k])
+    return out
+
+
+@pytest.fixture(scope="module")
+def scenes():
+    items, _ = synthetic.indoor_batch(4, 250_000)
+    return torch.as_tensor(synthetic.batch_indexed(items), device=DEV)
+
+
+def test_cfg2_full_size_identity_and_neighbour_sum(scenes):
+    """3x3x3, 64 -> 64, fp16, 4 x 250k voxels."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    n = scenes.shape[0]
+    km = generate_kernel_map(scenes, scenes, (1, 1, 1), (3, 3, 3))
+    x = torch.randn(n, 64, generator=torch.Generator().manual_seed(0)).half().to(DEV)
+    eye = torch.eye(64, dtype=torch.float16, device=DEV)
+    w = torch.zeros(27, 64, 64, dtype=torch.float16, device=DEV)
+    w[13] = eye
+    assert torch.equal(sparse_conv_forward(x, w, km, n), x)          # centre tap only: a copy
+    w[:] = eye                                                       # all taps: neighbour sum
+    want = torch.zeros(n, 64, dtype=torch.float32, device=DEV)
+    want.index_add_(0, km.out_maps.long(), x.float()[km.in_maps.long()])
+    got = sparse_conv_forward(x, w, km, n)
+    assert rel_err(got.float().cpu().numpy(), want.cpu().numpy()) <= 1e-2
+    w = kaiming_weight(27, 64, 64, seed=1, dtype=torch.float16).to(DEV)
+    got = sparse_conv_forward(x, w, km, n)
+    assert rel_err(got.float().cpu().numpy(), torch_explicit_fp32(x, w, km, n).cpu().numpy()) <= 1e-2
+    assert torch.equal(got, sparse_conv_forward(x, w, km, n))        # bitwise reproducible
+
+
+def test_cfg3_strided_and_transposed_full_size(scenes):
+    """2x2x2 stride-2 96 -> 128 and its transposed 128 -> 96, bf16."""
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    n = scenes.shape[0]
+    offsets = torch.tensor([0, 250_000, 500_000, 750_000, 1_000_000])
+    x = torch.randn(n, 96, generator=torch.Generator().manual_seed(2)).bfloat16().to(DEV)
+    fine = Voxels(scenes[:, 1:].contiguous(), x, offsets=offsets)
+    wd = kaiming_weight(8, 96, 128, seed=3, dtype=torch.bfloat16).to(DEV)
+    wu = kaiming_weight(8, 128, 96, seed=4, dtype=torch.bfloat16).to(DEV)
+    coarse = spatially_sparse_conv(fine, wd, 2, stride=2)
+    km = next(iter(fine.cache.values()))
+    assert int(km.offsets[-1]) == n and n // 8 <= len(coarse) < n
+    assert torch.equal(torch.sort(km.in_maps).values, torch.arange(n, dtype=torch.int32, device=DEV))
+    want = torch_explicit_fp32(x, wd, km, len(coarse))
+    assert rel_err(coarse.feature_tensor.float().cpu().numpy(), want.cpu().numpy()) <= 1e-2
+    back = spatially_sparse_conv(coarse, wu, 2, stride=2, transposed=True,
+                                 output_spatially_sparse_tensor=fine)
+    assert len(fine.cache) == 2
+    from warpconvnet_amd.geometry.coords.search.search_results import IntSearchResult
+    swapped = IntSearchResult(km.out_maps, km.in_maps, km.offsets)
+    want = torch_explicit_fp32(coarse.feature_tensor, wu, swapped, n)
+    assert rel_err(back.feature_tensor.float().cpu().numpy(), want.cpu().numpy()) <= 1e-2
+
+
+def test_cfg5a_5x5x5_map_bound(scenes):
+    """5x5x5 (125 offsets), 16 -> 16, fp16, 1M voxels."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    n = scenes.shape[0]
+    km = generate_kernel_map(scenes, scenes, (1, 1, 1), (5, 5, 5))
+    assert km.identity_map_index == 62 and len(km) == 125
+    i62, o62 = km[62]
+    ar = torch.arange(n, dtype=torch.int32, device=DEV)
+    assert torch.equal(i62, ar) and torch.equal(o62, ar)
+    counts = torch.diff(km.offsets)
+    assert torch.equal(counts, counts.flip(0))
+    for k in (0, 31, 61):  # (i, j) in map_k  <=>  (j, i) in map_{124-k}
+        a_in, a_out = km[k]
+        b_in, b_out = km[124 - k]
+        assert (torch.diff(a_out) > 0).all()
+        order = torch.argsort(b_in)
+        assert torch.equal(b_in[order], a_out) and torch.equal(b_out[order], a_in)
+    x = torch.randn(n, 16, generator=torch.Generator().manual_seed(5)).half().to(DEV)
+    w = kaiming_weight(125, 16, 16, seed=6, dtype=torch.float16).to(DEV)
+    got = sparse_conv_forward(x, w, km, n)
+    assert rel_err(got.float().cpu().numpy(), torch_explicit_fp32(x, w, km, n).cpu().numpy()) <= 1e-2
+
+
+def test_cfg5b_wide_channels_small_map():
+    """3x3x3, 256 -> 256, fp16, ~50k voxels from a 16 cm voxelisation of the same scenes; checked
+    against the torch-CPU restatement of the reference's explicit path."""
+    from oracle import cpu_oracle
+    from oracle.explicit_conv import explicit_gemm_forward
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    items = [synthetic.indoor_scene(b, None, 0.16) for b in range(4)]
+    bc = synthetic.batch_indexed(items)
+    n = len(bc)
+    assert 30_000 < n < 80_000
+    coords = torch.as_tensor(bc, device=DEV)
+    km = generate_kernel_map(coords, coords, (1, 1, 1), (3, 3, 3))
+    im, om, off, iden = cpu_oracle.kernel_map(bc, bc, (3, 3, 3))
+    assert np.array_equal(km.in_maps.cpu().numpy(), im) and np.array_equal(km.out_maps.cpu().numpy(), om)
+    x = torch.randn(n, 256, generator=torch.Generator().manual_seed(7)).half()
+    w = kaiming_weight(27, 256, 256, seed=8, dtype=torch.float16)
+    got = sparse_conv_forward(x.to(DEV), w.to(DEV), km, n)
+    want = explicit_gemm_forward(x, w, torch.as_tensor(im), torch.as_tensor(om), off, iden, n,
+                                 compute_dtype=torch.float32)
+    assert rel_err(got.float().cpu().numpy(), want.float().numpy()) <= 1e-2
