@@ -4,22 +4,25 @@
 //
 // Output-stationary, atomic-free, accumulators in registers.  A workgroup of four waves owns 256
 // consecutive output rows x 64 output channels; each wave keeps the fp32 accumulators of its 64
-// rows in MFMA result layout for the whole kernel.  The map is consumed in output-row form (per
-// row: bit mask of the offsets that hit, row pointer, hit input rows).
+// rows in MFMA result layout for the whole kernel, so the result is bitwise reproducible.
 //
-// The loop over offsets is cut into batches.  For a batch (up to 8 offsets, up to 256 hits) the
-// workgroup lists the hits of its rows, assigns each hit a slot, and gathers all hit input rows
-// into LDS with every load issued back to back (this is what keeps tens of KB in flight per CU;
-// a gather per offset would leave the kernel latency bound).  Then, offset by offset, W[k]^T is
-// staged in LDS (double buffered, fetched one offset ahead) and each wave multiplies its 64 rows:
-// lane l of a 16-row block reads the gathered row of output row (l & 15) through its slot, or
-// zeros if that output row has no hit for this offset, so the product lands in the accumulator
-// rows directly (v_mfma_f32_16x16x32_{f16,bf16}, v_mfma_f32_16x16x4_f32).  16-row blocks without
-// any hit are skipped.  One rounding to the feature dtype when the tile is written.
+// The map is consumed as the reference's pair lists, which ascend in output row inside every
+// offset: the pairs of one offset that touch the workgroup's rows are one contiguous run, found
+// with the group_start table (pairs of offset k below output row 64 * g).
 //
-// Compulsory HBM bytes: every hit input row once (L * C_in * s; revisits are served by the L2 /
-// Infinity Cache), the map once (8 M + 4 L), the output once (M * C_out * s); the weights
-// (K * C_in * C_out * s) stay cache resident.
+// The loop over offsets is cut into batches (up to 7 offsets, up to 256 pairs).  For a batch every
+// thread fetches one pair, the pairs become slots, and all their input rows are gathered into
+// LDS with the loads issued back to back (a gather per offset would leave the kernel latency
+// bound).  Then, offset by offset, W[k]^T is staged in LDS (double buffered, fetched two offsets
+// ahead through registers) and each wave multiplies its 64 rows: lane l of a 16-row block reads
+// the gathered row of output row (l & 15) through the slot table, or zeros if that output row has
+// no pair for this offset, so the product lands in the accumulator rows directly
+// (v_mfma_f32_16x16x32_{f16,bf16}, v_mfma_f32_16x16x4_f32).  16-row blocks without any pair are
+// skipped.  One rounding to the feature dtype when the tile is written.
+//
+// Compulsory HBM bytes: every gathered input row once (L * C_in * s; revisits are served by the
+// L2 / Infinity Cache when the voxel order has locality), the map once (8 L), the output once
+// (M * C_out * s); the weights (K * C_in * C_out * s) stay cache resident.
 #include <algorithm>
 #include <type_traits>
 
