@@ -10,15 +10,17 @@
 // offset: the pairs of one offset that touch the workgroup's rows are one contiguous run, found
 // with the group_start table (pairs of offset k below output row 64 * g).
 //
-// The loop over offsets is cut into batches (up to 7 offsets, up to 256 pairs).  For a batch every
-// thread fetches one pair, the pairs become slots, and all their input rows are gathered into
-// LDS with the loads issued back to back (a gather per offset would leave the kernel latency
-// bound).  Then, offset by offset, W[k]^T is staged in LDS (double buffered, fetched two offsets
-// ahead through registers) and each wave multiplies its 64 rows: lane l of a 16-row block reads
-// the gathered row of output row (l & 15) through the slot table, or zeros if that output row has
-// no pair for this offset, so the product lands in the accumulator rows directly
-// (v_mfma_f32_16x16x32_{f16,bf16}, v_mfma_f32_16x16x4_f32).  16-row blocks without any pair are
-// skipped.  One rounding to the feature dtype when the tile is written.
+// The loop over offsets is cut into batches (up to 4 offsets, up to 128 pairs; the pairs of one
+// offset may continue in the next batch).  The batches run as a software pipeline: while batch b
+// is multiplied, the gathered input rows and the W[k]^T tiles of batch b + 1 are in flight into
+// registers and the pairs of batch b + 2 are being read, so no global load is waited for right
+// after it is issued.  Per batch every thread fetches at most one pair, the pairs become slots of
+// the gathered-row buffer, and a slot table maps (offset of the batch, output row) to its slot.
+// In the multiply, lane l of a 16-row block reads the gathered row of output row (l & 15) through
+// the slot table, or a row of zeros if that output row has no pair for this offset, so the
+// product lands in the accumulator rows directly (v_mfma_f32_16x16x32_{f16,bf16},
+// v_mfma_f32_16x16x4_f32).  16-row blocks without any pair skip their MFMAs.  One rounding to the
+// feature dtype when the tile is written.
 //
 // Compulsory HBM bytes: every gathered input row once (L * C_in * s; revisits are served by the
 // L2 / Infinity Cache when the voxel order has locality), the map once (8 L), the output once
@@ -41,9 +43,8 @@ constexpr int ROWS = 256;    // output rows per workgroup
 constexpr int TN = 64;       // output channels per workgroup
 constexpr int THREADS = 256; // wave w owns rows 64 * (w & 3) .. +63 and channel blocks of column group (w >> 2)
 constexpr int NBW = TN / 16 / (THREADS / 256);  // 16-channel blocks per wave
-constexpr int BPT = TN * 8 / THREADS;           // 16-byte parts of a weight tile per thread
-constexpr int A_ROWS = 256;  // gathered input rows resident in LDS
-constexpr int BATCH = 7;     // offsets per gather batch, at most
+constexpr int A_ROWS = 128;  // gathered input rows resident in LDS (pairs per batch)
+constexpr int BATCH = 4;     // offsets per batch, at most
 
 __device__ __forceinline__ float to_float(_Float16 v) { return (float)v; }
 __device__ __forceinline__ float to_float(__bf16 v) { return (float)v; }
@@ -130,14 +131,19 @@ struct ConvArgs {
   int32_t vec_out;  // same for output rows
 };
 
-struct WTile {
-  u32x4 p[BPT];
-};
-
 // LDS rows are 128 bytes (eight 16-byte parts) with no padding; part p of row r is stored at
 // part p ^ ((r >> 1) & 7), which makes the 16-byte operand reads of 16 consecutive rows (and of
 // most scattered row sets) hit distinct banks.
 __device__ __forceinline__ int lds_part(int row, int part) { return part ^ ((row >> 1) & 7); }
+
+// One batch = up to BATCH offsets and A_ROWS pairs; the pairs of one offset may be split over
+// consecutive batches.  Packed descriptor of one (batch, offset) entry.
+__device__ __forceinline__ uint32_t pack_run(int k, int first, int num) {
+  return (uint32_t)k | ((uint32_t)first << 8) | ((uint32_t)num << 20);  // k < 32, first <= 256, num <= 128
+}
+__device__ __forceinline__ int run_k(uint32_t r) { return (int)(r & 0xFFu); }
+__device__ __forceinline__ int run_first(uint32_t r) { return (int)((r >> 8) & 0xFFFu); }
+__device__ __forceinline__ int run_num(uint32_t r) { return (int)(r >> 20); }
 
 template <typename T>
 __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
@@ -146,12 +152,20 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
   constexpr int CK = M::CK, KS = M::KS;
   constexpr int VEC = 16 / sizeof(T);  // elements per 16-byte part; a row is CK = 8 * VEC elements
   static_assert(CK == 8 * VEC, "a staged row is eight 16-byte parts");
-  __shared__ __attribute__((aligned(16))) T As[A_ROWS * CK + VEC];  // + one all-zero 16-byte part
-  __shared__ __attribute__((aligned(16))) T Bs[2][TN * CK];
-  __shared__ uint16_t s_slot[BATCH][ROWS];  // gathered row of (offset, output row); A_ROWS = none
-  __shared__ int32_t s_gidx[A_ROWS];
+  constexpr int A_PIECES = A_ROWS * 8 / THREADS;      // 16-byte parts of gathered rows per thread
+  constexpr int B_PIECES = BATCH * TN * 8 / THREADS;  // 16-byte parts of the batch's weight tiles
+  constexpr int MAX_BATCHES = 32 * ROWS / A_ROWS + 32 / BATCH + 2;  // per chunk of 32 offsets
+  static_assert(A_ROWS <= 128 && A_ROWS <= THREADS, "slot ids take 7 bits; one pair per thread");
+  __shared__ __attribute__((aligned(16))) T As[(A_ROWS + 1) * CK];  // last row: zeros
+  __shared__ __attribute__((aligned(16))) T Bs[BATCH][TN * CK];
+  // gathered row of (batch offset, output row), tagged with the batch it was written for:
+  // entry = (batch & 255) << 8 | row; an entry of another batch means "no pair"
+  __shared__ __attribute__((aligned(8))) uint16_t s_slot[2][ROWS][BATCH];
+  __shared__ int32_t s_gidx[2][A_ROWS];
+  __shared__ __attribute__((aligned(16))) uint32_t s_run[MAX_BATCHES + 2][BATCH];  // two empty batches after the last
   __shared__ int32_t s_cnt[32];
   __shared__ int32_t s_start[32];
+  __shared__ int32_t s_num_batches;
 
   const T* __restrict__ X = (const T*)a.X;
   const T* __restrict__ Wt = (const T*)a.Wt;
@@ -163,23 +177,25 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
   const int64_t g0 = m0 >> 6;
   const int64_t g1 = g0 + ROWS / 64 < a.G ? g0 + ROWS / 64 : a.G;
 
-  if (tid < VEC) As[A_ROWS * CK + tid] = from_float<T>(0.f);
-
   f32x4 acc[4][NBW];
 #pragma unroll
   for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
     for (int nb = 0; nb < NBW; ++nb) acc[rb][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  if (tid < 8) *reinterpret_cast<u32x4*>(&As[A_ROWS * CK + tid * VEC]) = (u32x4){0u, 0u, 0u, 0u};
 
-  // this thread's 16-byte parts of a (TN x CK) weight tile (rows b_n + h * THREADS / 8)
-  const int b_n = tid >> 3, b_part = tid & 7;
   // MFMA operand addressing: lane l reads row (l & 15) of a 16-row block, k-group (l >> 4)
   const int kgrp = lane >> 4;
 
+  const size_t w_tile_stride = (size_t)a.c_out_pad * a.c_in_pad;
+  const uint32_t w_step = (uint32_t)(THREADS / 8) * (uint32_t)a.c_in_pad;  // weight rows one piece apart
   for (int c0 = 0; c0 < a.c_in_pad; c0 += CK) {
+    const uint32_t w_lane_off = (uint32_t)(n0 + (tid >> 3)) * (uint32_t)a.c_in_pad + c0 + (tid & 7) * VEC;
+    const uint32_t x_lane_off = (uint32_t)(c0 + (tid & 7) * VEC);
+    const bool x_part_ok = (int)x_lane_off < a.c_in;
     for (int kbase = 0; kbase < a.K; kbase += 32) {
       const int nk = a.K - kbase < 32 ? a.K - kbase : 32;
-      __syncthreads();  // the previous chunk's readers of s_cnt / s_start are done
+      __syncthreads();  // the previous chunk is completely done with the shared tables
       if (tid < 32) {
         int cnt = 0;
         int32_t start = 0;
@@ -198,153 +214,205 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
         s_cnt[tid] = cnt;
         s_start[tid] = start;
       }
+      for (int i = tid; i < 2 * BATCH * ROWS; i += THREADS) (&s_slot[0][0][0])[i] = 0xFFFFu;
       __syncthreads();
-
-      int b0 = 0;
-      while (b0 < nk) {
-        // batch [b0, b1): as many offsets as fit the LDS row budget (one offset always fits)
-        int b1 = b0, total = 0;
-        while (b1 < nk && b1 - b0 < BATCH && total + s_cnt[b1] <= A_ROWS) total += s_cnt[b1++];
-        if (total == 0) {
-          b0 = b1;
-          continue;
+      if (tid == 0) {  // cut the chunk into batches (a few dozen steps at most)
+        int nb = 0, k = 0, done = 0;
+        while (k < nk && s_cnt[k] == 0) ++k;
+        while (k < nk && nb < MAX_BATCHES) {
+          int total = 0;
+          for (int j = 0; j < BATCH; ++j) {
+            uint32_t run = pack_run(0, 0, 0);
+            if (k < nk && total < A_ROWS) {
+              const int left = s_cnt[k] - done;
+              const int take = left < A_ROWS - total ? left : A_ROWS - total;
+              run = pack_run(k, done, take);
+              total += take;
+              done += take;
+              if (done == s_cnt[k]) {
+                done = 0;
+                ++k;
+                while (k < nk && s_cnt[k] == 0) ++k;
+              }
+            }
+            s_run[nb][j] = run;
+          }
+          ++nb;
         }
-        // the pair that becomes gathered row `tid` of this batch
-        int my_j = -1, my_in = -1, my_out = -1;
-        if (tid < ROWS) {
+        for (int j = 0; j < BATCH; ++j) s_run[nb][j] = s_run[nb + 1][j] = pack_run(0, 0, 0);
+        s_num_batches = nb;
+      }
+      __syncthreads();
+      const int num_batches = s_num_batches;
+
+      // ---- software pipeline over the batches ------------------------------------------------
+      // While batch b is multiplied, the input rows and weight tiles of batch b + 1 are in flight
+      // (held in registers until the multiply is over) and so are the pairs of batch b + 2.
+      int pr_j = -1, pr_in = -1, pr_out = -1;  // this thread's pair of the batch after the next store
+      auto load_pair = [&](int b) {
+        pr_j = -1;
+        if (b < num_batches && tid < A_ROWS) {
           int before = 0;
 #pragma unroll
           for (int j = 0; j < BATCH; ++j) {
-            const int c = b0 + j < b1 ? s_cnt[b0 + j] : 0;
-            if (my_j < 0 && tid >= before && tid < before + c) {
-              my_j = j;
-              const int i = tid - before;
-              if (kbase + b0 + j == a.identity) {
-                my_in = (int)(m0 + i);
-                my_out = i;
+            const uint32_t run = s_run[b][j];
+            const int num = run_num(run);
+            if (pr_j < 0 && tid >= before && tid < before + num) {
+              pr_j = j;
+              const int k = run_k(run), i = run_first(run) + tid - before;
+              if (kbase + k == a.identity) {
+                pr_in = (int)(m0 + i);
+                pr_out = i;
               } else {
-                const int64_t p = (int64_t)s_start[b0 + j] + i;
-                my_in = a.in_maps[p];
-                my_out = (int)(a.out_maps[p] - m0);
+                const int64_t p = (int64_t)s_start[k] + i;
+                pr_in = a.in_maps[p];
+                pr_out = (int)(a.out_maps[p] - m0);
               }
             }
-            before += c;
+            before += num;
           }
         }
-        // weight tiles travel through two register slots: the first two offsets of the batch are
-        // requested together with the gather, offset j + 2 as soon as offset j left its slot
-        WTile wa, wb;
-        auto fetch_b = [&](int j, WTile& r) {
-          if (j < BATCH && b0 + j < b1 && s_cnt[b0 + j] > 0) {
+      };
+      auto publish_pair = [&](int b) {  // slot table and row list of batch b
+        if (b < num_batches && tid < A_ROWS) {
+          int32_t g = -1;
+          if (pr_j >= 0) {
+            g = pr_in;
+            if ((uint32_t)g >= (uint64_t)a.num_in) g = -1;  // malformed map: zeros
+            if ((uint32_t)pr_out < (uint32_t)tile_rows)
+              s_slot[b & 1][pr_out][pr_j] = (uint16_t)(((b & 255) << 8) | tid);
+          }
+          s_gidx[b & 1][tid] = g;
+        }
+      };
+      u32x4 piece[A_PIECES], wpiece[B_PIECES];
+      // runs of a batch as wave-uniform scalars (one 16-byte LDS read)
+      auto read_runs = [&](int b, uint32_t (&run)[BATCH]) {
+        static_assert(BATCH == 4, "one 16-byte read");
+        const u32x4 r = *reinterpret_cast<const u32x4*>(&s_run[b][0]);
 #pragma unroll
-            for (int h = 0; h < BPT; ++h)
-              r.p[h] = *reinterpret_cast<const u32x4*>(
-                  Wt + ((int64_t)(kbase + b0 + j) * a.c_out_pad + n0 + b_n + h * (THREADS / 8)) * a.c_in_pad +
-                  c0 + b_part * VEC);
+        for (int j = 0; j < BATCH; ++j) run[j] = __builtin_amdgcn_readfirstlane(r[j]);
+      };
+      auto fetch_rows = [&](int b, const uint32_t (&run)[BATCH]) {  // rows and weight tiles of batch b -> registers
+        if (b >= num_batches) return;
+        int32_t g[A_PIECES];
+#pragma unroll
+        for (int i = 0; i < A_PIECES; ++i) g[i] = s_gidx[b & 1][(tid >> 3) + i * (THREADS / 8)];
+#pragma unroll
+        for (int i = 0; i < B_PIECES; ++i) {
+          constexpr int PER = TN * 8 / THREADS;  // pieces of one weight tile per thread
+          const int j = i / PER;
+          wpiece[i] = (u32x4){0u, 0u, 0u, 0u};
+          if (run_num(run[j]) > 0) {  // uniform
+            const T* wk = Wt + (size_t)(kbase + run_k(run[j])) * w_tile_stride;
+            wpiece[i] = *reinterpret_cast<const u32x4*>(wk + w_lane_off + (uint32_t)(i % PER) * w_step);
           }
-        };
-        fetch_b(0, wa);
-        fetch_b(1, wb);
-        // slot table of the batch: "no hit" everywhere, then one entry per pair
-        if (tid < BATCH * ROWS / 8)
-          *reinterpret_cast<u32x4*>(&s_slot[0][0] + tid * 8) =
-              (u32x4){A_ROWS * 0x10001u, A_ROWS * 0x10001u, A_ROWS * 0x10001u, A_ROWS * 0x10001u};
-        __syncthreads();
-        if (my_j >= 0) {
-          if ((uint32_t)my_in >= (uint64_t)a.num_in) my_in = -1;  // malformed map: zeros
-          s_gidx[tid] = my_in;
-          if ((uint32_t)my_out < (uint32_t)tile_rows) s_slot[my_j][my_out] = (uint16_t)tid;
         }
-        __syncthreads();
-
-        // gather every hit row of the batch: loads first, all independent, then the LDS stores
         if (a.vec_in) {
-          u32x4 piece[A_ROWS * 8 / THREADS];
 #pragma unroll
-          for (int i = 0; i < A_ROWS * 8 / THREADS; ++i) {
-            const int seg = tid + i * THREADS, sl = seg >> 3, part = seg & 7;
+          for (int i = 0; i < A_PIECES; ++i) {
             piece[i] = (u32x4){0u, 0u, 0u, 0u};
-            if (seg < total * 8) {
-              const int32_t g = s_gidx[sl];
-              if (g >= 0 && c0 + part * VEC < a.c_in)
-                piece[i] = *reinterpret_cast<const u32x4*>(X + (int64_t)g * a.c_in + c0 + part * VEC);
+            if (g[i] >= 0 && x_part_ok)
+              piece[i] = *reinterpret_cast<const u32x4*>(X + ((uint64_t)(uint32_t)g[i] * (uint32_t)a.c_in + x_lane_off));
+          }
+        } else {  // rows that are not whole 16-byte vectors: element by element
+#pragma unroll
+          for (int i = 0; i < A_PIECES; ++i) {
+            piece[i] = (u32x4){0u, 0u, 0u, 0u};
+            if (g[i] >= 0 && x_part_ok) {
+              T tmp[VEC];
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) {
+                const int c = (int)x_lane_off + e;
+                tmp[e] = c < a.c_in ? X[(uint64_t)(uint32_t)g[i] * (uint32_t)a.c_in + c] : from_float<T>(0.f);
+              }
+              piece[i] = *reinterpret_cast<const u32x4*>(tmp);
             }
           }
-#pragma unroll
-          for (int i = 0; i < A_ROWS * 8 / THREADS; ++i) {
-            const int seg = tid + i * THREADS, sl = seg >> 3, part = seg & 7;
-            if (seg < total * 8)
-              *reinterpret_cast<u32x4*>(&As[sl * CK + lds_part(sl, part) * VEC]) = piece[i];
-          }
-        } else {
-          for (int e = tid; e < total * CK; e += THREADS) {
-            const int sl = e / CK, c = e % CK;
-            const int32_t g = s_gidx[sl];
-            T val = from_float<T>(0.f);
-            if (g >= 0 && c0 + c < a.c_in) val = X[(int64_t)g * a.c_in + c0 + c];
-            As[sl * CK + lds_part(sl, c / VEC) * VEC + c % VEC] = val;
-          }
         }
+      };
 
-        // One barrier per offset: W[k]^T goes to the buffer the previous offset did not use, the
-        // barrier publishes it (and, the first time, the gathered rows), then every wave multiplies.
-        // A wave can only overwrite a buffer after all waves passed the barrier that follows its
-        // last use.
-        int buf = 0;
-        auto multiply = [&](int j, WTile& r) {
-          if (b0 + j >= b1) return;  // uniform
-          if (s_cnt[b0 + j] == 0) {
-            fetch_b(j + 2, r);  // keep the ring moving
-            return;
-          }
+      uint32_t run_cur[BATCH], run_next[BATCH];
+      if (num_batches > 0) {
+        load_pair(0);
+        publish_pair(0);
+        load_pair(1);
+        __syncthreads();
+        read_runs(0, run_next);
+        fetch_rows(0, run_next);
+      }
+      for (int b = 0; b < num_batches; ++b) {
 #pragma unroll
-          for (int h = 0; h < BPT; ++h) {
-            const int n = b_n + h * (THREADS / 8);
-            *reinterpret_cast<u32x4*>(&Bs[buf][n * CK + lds_part(n, b_part) * VEC]) = r.p[h];
-          }
-          fetch_b(j + 2, r);
-          // gathered rows of this wave's four 16-row blocks
+        for (int j = 0; j < BATCH; ++j) run_cur[j] = run_next[j];
+        // registers -> LDS for batch b (this is where the loads issued one batch ago are awaited)
+#pragma unroll
+        for (int i = 0; i < A_PIECES; ++i) {
+          const int seg = tid + i * THREADS, sl = seg >> 3, part = seg & 7;
+          *reinterpret_cast<u32x4*>(&As[sl * CK + lds_part(sl, part) * VEC]) = piece[i];
+        }
+#pragma unroll
+        for (int i = 0; i < B_PIECES; ++i) {
+          const int v = tid + i * THREADS, j = v / (TN * 8), n = (v >> 3) % TN, part = v & 7;
+          *reinterpret_cast<u32x4*>(&Bs[j][n * CK + lds_part(n, part) * VEC]) = wpiece[i];
+        }
+        publish_pair(b + 1);
+        load_pair(b + 2);
+        __syncthreads();
+        // slot entries of this lane's four row blocks, all offsets of the batch (8 bytes each)
+        uint32_t se[4][2];
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+          const uint2 t = *reinterpret_cast<const uint2*>(&s_slot[b & 1][wrow + rb * 16 + (lane & 15)][0]);
+          se[rb][0] = t.x;
+          se[rb][1] = t.y;
+        }
+        read_runs(b + 1, run_next);
+        fetch_rows(b + 1, run_next);
+
+        // multiply batch b: no barrier between its offsets, the waves run freely
+        const uint16_t tag = (uint16_t)(b & 255);
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+          if (run_num(run_cur[j]) == 0) continue;  // uniform
           int sl[4];
 #pragma unroll
-          for (int rb = 0; rb < 4; ++rb) sl[rb] = s_slot[j][wrow + rb * 16 + (lane & 15)];
-          __syncthreads();
+          for (int rb = 0; rb < 4; ++rb) {
+            const uint32_t e = (se[rb][j >> 1] >> (16 * (j & 1))) & 0xFFFFu;
+            sl[rb] = (e >> 8) == tag ? (int)(e & 0xFFu) : A_ROWS;  // no pair: the row of zeros
+          }
           V bfr[NBW][KS];
 #pragma unroll
           for (int nb = 0; nb < NBW; ++nb) {
             const int n = wcol + nb * 16 + (lane & 15);
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) bfr[nb][ks] = M::load(&Bs[buf][n * CK], n, ks, kgrp);
+            for (int ks = 0; ks < KS; ++ks) bfr[nb][ks] = M::load(&Bs[j][n * CK], n, ks, kgrp);
           }
+          V av[4][KS];
+#pragma unroll
+          for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) av[rb][ks] = M::load(&As[sl[rb] * CK], sl[rb], ks, kgrp);
 #pragma unroll
           for (int rb = 0; rb < 4; ++rb) {
-            if (__ballot(sl[rb] != A_ROWS) == 0ull) continue;  // no hit in these 16 rows
-            V av[KS];  // rows without a hit read zeros
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
-              av[ks] = sl[rb] != A_ROWS ? M::load(&As[sl[rb] * CK], sl[rb], ks, kgrp) : M::zero();
+            if (__ballot(sl[rb] < A_ROWS) == 0ull) continue;  // no pair in these 16 rows
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-              for (int nb = 0; nb < NBW; ++nb) acc[rb][nb] = M::mma(av[ks], bfr[nb][ks], acc[rb][nb]);
+              for (int nb = 0; nb < NBW; ++nb) acc[rb][nb] = M::mma(av[rb][ks], bfr[nb][ks], acc[rb][nb]);
           }
-          buf ^= 1;
-        };
-#pragma nounroll
-        for (int j = 0; j < BATCH; j += 2) {
-          multiply(j, wa);
-          multiply(j + 1, wb);
         }
-        __syncthreads();  // every wave is done with the gathered rows and the slot table
-        b0 = b1;
+        __syncthreads();  // every wave is done with the gathered rows and weight tiles of batch b
       }
     }
   }
-
   // epilogue: bias add, one rounding to T
   T* __restrict__ out = (T*)a.out;
   const T* __restrict__ bias = (const T*)a.bias;
   if (sizeof(T) == 2 && a.vec_out) {
-    // stage the tile in LDS (As is free: the last batch ended with a barrier) for 16-byte stores
+    // stage the tile in LDS (the weight buffers are free: the last batch ended with a barrier) for
+    // 16-byte stores
+    static_assert(BATCH * TN >= ROWS, "the weight buffers hold one output tile");
+    T* stage = &Bs[0][0];
     __syncthreads();
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
@@ -355,7 +423,7 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int lr = wrow + rb * 16 + kgrp * 4 + r;
-          As[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC] = from_float<T>(acc[rb][nb][r] + bv);
+          stage[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC] = from_float<T>(acc[rb][nb][r] + bv);
         }
       }
     __syncthreads();
@@ -363,7 +431,7 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
       const int r = v >> 3, part = v & 7;
       if (m0 + r < a.num_out && n0 + part * VEC < a.c_out)
         *reinterpret_cast<u32x4*>(out + (m0 + r) * a.c_out + n0 + part * VEC) =
-            *reinterpret_cast<const u32x4*>(&As[r * CK + lds_part(r, part) * VEC]);
+            *reinterpret_cast<const u32x4*>(&stage[r * CK + lds_part(r, part) * VEC]);
     }
   } else {
 #pragma unroll
@@ -704,3 +772,4 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
 }
 
 }  // extern "C"
+
