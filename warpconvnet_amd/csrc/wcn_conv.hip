@@ -461,32 +461,42 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
 // ---- ring kernel: input rows, weight tiles and pairs go from memory straight into LDS ------------
 //
 // Used when feature rows are whole 16-byte vectors.  The offsets of a tile are cut into steps of
-// at most 64 pairs of one offset.  Three streams of global_load_lds run ahead of the multiply,
-// none of them through registers:
-//   pairs of step s      -> pair ring (8 slots),     issued DP = 8 steps ahead
-//   input rows of step s -> row ring (5 x 64 rows),  issued DG = 4 steps ahead
-//   W[k]^T of step s     -> weight ring (4 tiles),   issued DW = 3 steps ahead
-// Every wave issues the same loads in every iteration, in the order weights, rows, pairs (lanes
-// without work read a block of zeros), so "what step i needs has landed" is one fixed
+// at most 64 pairs of one offset.  A workgroup has eight waves:
+//   waves 0..3  multiply: each owns 64 output rows of the tile and their accumulators; per step it
+//               reads its operands from LDS and issues the MFMAs, nothing else
+//   waves 4..7  request: each a quarter of W[k]^T of step r + DW (weight ring, 4 tiles) and a
+//               quarter of the input rows of step r + DG (row ring, 5 x 64 rows); wave 4 also the
+//               input rows and wave 5 the output rows of the pairs of step r + DP (pair ring, 8
+//               slots); wave 6 writes the slot table of step r + DG, wave 7 clears the next one
+// The requests are global_load_lds: the data goes from memory into LDS without passing through
+// registers.  A wave issues at most one instruction every four cycles, so the bookkeeping of the
+// requests would otherwise sit between the MFMAs of every wave; here it runs beside them.
+// (Workgroups of more than four waves are co-resident on a CU only if every SIMD has room for
+// two waves of each, hence the budget of 128 vector registers.)
+// A requesting wave issues the same loads in every iteration, in the order weights, rows, pairs
+// (lanes without work read a block of zeros), so "what step r needs has landed" is one fixed
 // s_waitcnt vmcnt(n): the counter retires in order, and with DG = DW + 1 and DP = 2 DG the rows of
-// step i, the pairs of step i + DG and the weights of step i are the oldest loads still wanted.
-// One barrier per step publishes what has landed.  A slot table per step (one byte per output
-// row: the row's position in the step's slot, or none) is written when the rows are requested
-// and read when the step is multiplied.
+// step r, the pairs of step r + DG and the weights of step r are the oldest loads still wanted.
+// One barrier per step publishes what has landed and hands the slots read in the previous step
+// back to the requesting waves.  A slot table per step (one byte per output row: the row's
+// position in the step's slot, or none) is written when the rows are requested and read when
+// the step is multiplied.
+constexpr int RING_THREADS = 512;
 constexpr int STEP_ROWS = 64;
 constexpr int A_SLOTS = 5, W_SLOTS = 4, P_SLOTS = 8, T_SLOTS = 8;
 constexpr int DG = A_SLOTS - 1, DW = W_SLOTS - 1, DP = 2 * DG;
 constexpr int MAX_STEPS = 32 * (ROWS / STEP_ROWS);
 constexpr int SLOT_BYTES = STEP_ROWS * 128;   // a row of the rings is 128 bytes for every dtype
 static_assert(TN * 128 == SLOT_BYTES, "weight tile and row slot have the same size");
-static_assert(DP < P_SLOTS + DG && T_SLOTS > DG + 1 && DG == DW + 1, "ring reuse distances");
+static_assert(DP < P_SLOTS + DG && DG == DW + 1 && T_SLOTS > DG + 1, "ring reuse distances");
+static_assert(DG * 5 < 64, "outstanding loads per wave fit the 6-bit vmcnt");
 constexpr int RING_OFF = 0;
 constexpr int WRING_OFF = RING_OFF + A_SLOTS * SLOT_BYTES;
 constexpr int PIN_OFF = WRING_OFF + W_SLOTS * SLOT_BYTES;
 constexpr int POUT_OFF = PIN_OFF + P_SLOTS * STEP_ROWS * 4;
 constexpr int TAB_OFF = POUT_OFF + P_SLOTS * STEP_ROWS * 4;
 constexpr int ZERO_OFF = TAB_OFF + T_SLOTS * ROWS;
-constexpr int STEP_OFF = ZERO_OFF + 256;  // the first 128 bytes are the row of zeros
+constexpr int STEP_OFF = ZERO_OFF + 128;  // after the row of zeros
 constexpr int MISC_OFF = STEP_OFF + (MAX_STEPS + 2 * DP) * 8;  // DP empty steps before and after the plan
 constexpr int RING_LDS_BYTES = (MISC_OFF + 16 + 511) / 512 * 512;
 static_assert(2 * RING_LDS_BYTES <= 160 * 1024, "two workgroups per CU");
@@ -514,11 +524,12 @@ __device__ __forceinline__ int step_first(uint32_t w0) { return (int)((w0 >> 16)
 __device__ __forceinline__ bool step_identity(uint32_t w0) { return (w0 >> 31) != 0u; }
 
 template <typename T>
-__global__ void __launch_bounds__(THREADS, 2) conv_fwd_ring(ConvArgs a) {
+__global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
   typedef Mma<T> M;
   typedef typename M::V V;
   constexpr int CK = M::CK, KS = M::KS;
   constexpr int VEC = 16 / sizeof(T);
+  constexpr int NB = TN / 16;
   static_assert(CK * sizeof(T) == 128, "ring rows are 128 bytes");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint8_t* const ring = smem + RING_OFF;
@@ -535,7 +546,7 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd_ring(ConvArgs a) {
   const uint8_t* const zsrc = (const uint8_t*)a.zeros;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wrow = wave * 64;
+  const int wrow = (wave & 3) * 64;  // multiplying waves: first row in the tile
   const int64_t m0 = (int64_t)blockIdx.x * ROWS;
   const int n0 = blockIdx.y * TN;
   const int tile_rows = (int)(a.num_out - m0 < ROWS ? a.num_out - m0 : ROWS);
@@ -544,148 +555,218 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd_ring(ConvArgs a) {
   const int kgrp = lane >> 4;
   const int sub = lane >> 3, lpart = lane & 7;  // row inside an 8-row load, 16-byte part in LDS
 
-  f32x4 acc[4][NBW];
-#pragma unroll
-  for (int rb = 0; rb < 4; ++rb)
-#pragma unroll
-    for (int nb = 0; nb < NBW; ++nb) acc[rb][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  if (tid < 64) ((uint32_t*)(smem + ZERO_OFF))[tid] = 0u;
+  if (tid < 32) ((uint32_t*)(smem + ZERO_OFF))[tid] = 0u;
+  T* __restrict__ out = (T*)a.out;
+  T* const stage = (T*)ring;  // output tile staged for 16-byte stores: 256 rows x 128 bytes
+  const bool staged = sizeof(T) == 2 && a.vec_out;
 
-  for (int c0 = 0; c0 < a.c_in_pad; c0 += CK) {
-    for (int kbase = 0; kbase < a.K; kbase += 32) {
-      const int nk = a.K - kbase < 32 ? a.K - kbase : 32;
-      // the previous chunk is completely done: every load_to_lds has landed, every wave is past
-      // its last multiply
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-      if (wave == 0) {  // cut the chunk into steps
-        int cnt = 0;
-        int32_t start = 0;
-        bool ident = false;
-        if (lane < nk) {
-          const int k = kbase + lane;
-          if (k == a.identity) {  // every row reads its own input row; the map's pairs are ignored
-            const int64_t left = a.num_in - m0;
-            cnt = (int)(left < 0 ? 0 : (left < tile_rows ? left : tile_rows));
-            ident = true;
-          } else {
-            const int32_t* gs = a.group_start + (int64_t)k * (a.G + 1);
-            start = (int32_t)(a.offsets[k] + gs[g0]);
-            cnt = gs[g1] - gs[g0];
-            if (cnt < 0 || cnt > ROWS) cnt = 0;  // inconsistent table: contribute nothing
-          }
+  // Start of a chunk (up to 32 offsets of one slice of input channels): the step plan and clean
+  // slot tables.  Every wave runs it; returns the number of steps.
+  auto begin_chunk = [&](int kbase) -> int {
+    const int nk = a.K - kbase < 32 ? a.K - kbase : 32;
+    // the previous chunk is completely done: every load_to_lds has landed, every wave is past
+    // its last multiply
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (wave == 0) {  // cut the chunk into steps
+      int cnt = 0;
+      int32_t start = 0;
+      bool ident = false;
+      if (lane < nk) {
+        const int k = kbase + lane;
+        if (k == a.identity) {  // every row reads its own input row; the map's pairs are ignored
+          const int64_t left = a.num_in - m0;
+          cnt = (int)(left < 0 ? 0 : (left < tile_rows ? left : tile_rows));
+          ident = true;
+        } else {
+          const int32_t* gs = a.group_start + (int64_t)k * (a.G + 1);
+          start = (int32_t)(a.offsets[k] + gs[g0]);
+          cnt = gs[g1] - gs[g0];
+          if (cnt < 0 || cnt > ROWS) cnt = 0;  // inconsistent table: contribute nothing
         }
-        const int ns = (cnt + STEP_ROWS - 1) / STEP_ROWS;
-        const int incl = wcn_wave_inclusive_sum(ns);
-        for (int j = 0; j < ns; ++j) {
-          const int num = cnt - j * STEP_ROWS < STEP_ROWS ? cnt - j * STEP_ROWS : STEP_ROWS;
-          s_step[DP + incl - ns + j] =
-              make_uint2((uint32_t)lane | ((uint32_t)num << 8) | ((uint32_t)(j * STEP_ROWS) << 16) |
-                             (ident ? 0x80000000u : 0u),
-                         (uint32_t)(start + j * STEP_ROWS));
-        }
-        const int total = __builtin_amdgcn_readlane(incl, 63);
-        if (lane < DP) s_step[lane] = s_step[DP + total + lane] = make_uint2(0u, 0u);
-        if (lane == 63) *s_nsteps = total;
       }
-      for (int i = tid; i < T_SLOTS * ROWS / 4; i += THREADS) ((uint32_t*)s_tab)[i] = 0xFFFFFFFFu;
-      __syncthreads();
-      const int S = *s_nsteps;
-      if (S == 0) continue;
+      const int ns = (cnt + STEP_ROWS - 1) / STEP_ROWS;
+      const int incl = wcn_wave_inclusive_sum(ns);
+      for (int j = 0; j < ns; ++j) {
+        const int num = cnt - j * STEP_ROWS < STEP_ROWS ? cnt - j * STEP_ROWS : STEP_ROWS;
+        s_step[DP + incl - ns + j] =
+            make_uint2((uint32_t)lane | ((uint32_t)num << 8) | ((uint32_t)(j * STEP_ROWS) << 16) |
+                           (ident ? 0x80000000u : 0u),
+                       (uint32_t)(start + j * STEP_ROWS));
+      }
+      const int total = __builtin_amdgcn_readlane(incl, 63);
+      if (lane < DP) s_step[lane] = s_step[DP + total + lane] = make_uint2(0u, 0u);
+      if (lane == 63) *s_nsteps = total;
+    }
+    for (int i = tid; i < T_SLOTS * ROWS / 4; i += RING_THREADS) ((uint32_t*)s_tab)[i] = 0xFFFFFFFFu;
+    __syncthreads();
+    return *s_nsteps;
+  };
+  // descriptors are fetched one iteration ahead (raw, made wave-uniform when used)
+  auto step_raw = [&](int s, int S) -> uint2 {  // -DP <= s; steps past the plan's padding read as its last entry
+    const int idx = s + DP < S + 2 * DP - 1 ? s + DP : S + 2 * DP - 1;
+    return s_step[idx];
+  };
+  auto uniform = [&](uint2 d) -> uint2 {
+    d.x = __builtin_amdgcn_readfirstlane(d.x);
+    d.y = __builtin_amdgcn_readfirstlane(d.y);
+    return d;
+  };
 
-      // descriptors and slot entries are fetched one iteration ahead (raw, made uniform when used)
-      auto step_raw = [&](int s) -> uint2 {  // -DP <= s; steps past the plan's padding read as its last entry
-        const int idx = s + DP < S + 2 * DP - 1 ? s + DP : S + 2 * DP - 1;
-        return s_step[idx];
-      };
-      auto uniform = [&](uint2 d) -> uint2 {
-        d.x = __builtin_amdgcn_readfirstlane(d.x);
-        d.y = __builtin_amdgcn_readfirstlane(d.y);
-        return d;
-      };
-      uint2 rR = step_raw(-DP), rG = step_raw(-DP + DG), rW = step_raw(-DP + DW), rP = step_raw(0);
-      uint32_t sw_next = 0xFFFFFFFFu;
-      int ia = (A_SLOTS - (DP - DG) % A_SLOTS) % A_SLOTS;  // (r + DG) mod A_SLOTS, kept incrementally
-      int iw = (W_SLOTS - (DP - DW) % W_SLOTS) % W_SLOTS;  // (r + DW) mod W_SLOTS
-      int im = (A_SLOTS - DP % A_SLOTS) % A_SLOTS;         // r mod A_SLOTS
-      int imw = (W_SLOTS - DP % W_SLOTS) % W_SLOTS;        // r mod W_SLOTS
-
-      // One iteration: operands of step r from LDS into one register set, while the MFMAs of
-      // step r - 1 run from the other set; then the requests for the steps ahead.
-      V bfr0[NBW][KS], av0[4][KS], bfr1[NBW][KS], av1[4][KS];
-      bool any0[4] = {false, false, false, false}, any1[4] = {false, false, false, false};
-      auto iteration = [&](int r, V (&bfr)[NBW][KS], V (&av)[4][KS], bool (&any)[4],
-                           const V (&pbfr)[NBW][KS], const V (&pav)[4][KS], const bool (&pany)[4]) {
-        const uint2 dR = uniform(rR), dG = uniform(rG), dW = uniform(rW), dP = uniform(rP);
-        const uint32_t sw = sw_next;  // slot entries of this lane's four row blocks for step r
-        // everything step r needs (and the pairs of step r + DG) has landed, for all waves
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 + 5 * (DW - 1)) : "memory");
-
-        // ---- LDS reads of this iteration, all issued before anything waits for them
+  // The two kinds of waves run separate code from here on (the accumulators exist only in the
+  // multiplying waves); both pass the same sequence of barriers.
+  if (wave < 4) {
+    f32x4 acc[4][NB];
 #pragma unroll
-        for (int rb = 0; rb < 4; ++rb) any[rb] = false;
-        if (r >= 0 && step_num(dR.x) > 0) {
-          const T* const abase = (const T*)(ring + im * SLOT_BYTES);
-          const T* const bbase = (const T*)(wring + imw * SLOT_BYTES);
+    for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
-          for (int nb = 0; nb < NBW; ++nb) {
-            const int n = nb * 16 + (lane & 15);
+      for (int nb = 0; nb < NB; ++nb) acc[rb][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int c0 = 0; c0 < a.c_in_pad; c0 += CK) {
+      for (int kbase = 0; kbase < a.K; kbase += 32) {
+        const int S = begin_chunk(kbase);
+        if (S == 0) continue;
+        // ================= multiplying waves =================
+        uint2 rR = step_raw(-DP, S);
+        uint32_t sw = 0xFFFFFFFFu;  // slot entries of this lane's four row blocks for step r
+        int im = (A_SLOTS - DP % A_SLOTS) % A_SLOTS;   // r mod A_SLOTS, kept incrementally
+        int imw = (W_SLOTS - DP % W_SLOTS) % W_SLOTS;  // r mod W_SLOTS
+#pragma nounroll
+        for (int r = -DP; r < S; ++r) {
+          const uint2 dR = uniform(rR);
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          rR = step_raw(r + 1, S);
+          const uint32_t sw_cur = sw;
+          sw = *(const uint32_t*)(s_tab + ((r + 1) & (T_SLOTS - 1)) * ROWS + wrow + (lane & 15) * 4);
+          if (r >= 0 && step_num(dR.x) > 0) {
+            const T* const abase = (const T*)(ring + im * SLOT_BYTES);
+            const T* const bbase = (const T*)(wring + imw * SLOT_BYTES);
+            V bfr[NB][KS], av[2][KS];  // the A operands of a row block are read while the one before multiplies
+            bool any[4];
+            const T* arow[4];
+            int aswz[4];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) bfr[nb][ks] = M::load(bbase + n * CK, n, ks, kgrp);
+            for (int nb = 0; nb < NB; ++nb) {
+              const int n = nb * 16 + (lane & 15);
+#pragma unroll
+              for (int ks = 0; ks < KS; ++ks) bfr[nb][ks] = M::load(bbase + n * CK, n, ks, kgrp);
+            }
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+              const int e = (int)((sw_cur >> (8 * rb)) & 0xFFu);
+              const bool has = e != 0xFF;
+              any[rb] = __ballot(has) != 0ull;  // no pair in these 16 rows: skipped
+              arow[rb] = has ? abase + e * CK : s_zero;
+              aswz[rb] = has ? e : 0;
+            }
+            if (any[0]) {
+#pragma unroll
+              for (int ks = 0; ks < KS; ++ks) av[0][ks] = M::load(arow[0], aswz[0], ks, kgrp);
+            }
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+              if (rb + 1 < 4 && any[rb + 1]) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                  av[(rb + 1) & 1][ks] = M::load(arow[rb + 1], aswz[rb + 1], ks, kgrp);
+              }
+              if (!any[rb]) continue;
+#pragma unroll
+              for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                  acc[rb][nb] = M::mma(av[rb & 1][ks], bfr[nb][ks], acc[rb][nb]);
+            }
           }
+          im = im + 1 == A_SLOTS ? 0 : im + 1;
+          imw = imw + 1 == W_SLOTS ? 0 : imw + 1;
+        }
+      }
+    }
+    // epilogue: bias add, one rounding to T
+    const T* __restrict__ bias = (const T*)a.bias;
+    float bias_v[NB];  // this lane's bias values, fetched together
 #pragma unroll
-          for (int rb = 0; rb < 4; ++rb) {
-            const int e = (int)((sw >> (8 * rb)) & 0xFFu);
-            const bool has = e != 0xFF;
-            any[rb] = __ballot(has) != 0ull;
-            if (!any[rb]) continue;  // no pair in these 16 rows
-            const T* row = has ? abase + e * CK : s_zero;
-            const int rr = has ? e : 0;
+    for (int nb = 0; nb < NB; ++nb) {
+      const int col = n0 + nb * 16 + (lane & 15);
+      bias_v[nb] = (bias && col < a.c_out) ? to_float(bias[col]) : 0.f;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the loads of the empty steps after the last one
+    __syncthreads();  // every wave is done with the rings, every load has landed
+    if (staged) {
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) av[rb][ks] = M::load(row, rr, ks, kgrp);
+      for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const int col = nb * 16 + (lane & 15);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int lr = wrow + rb * 16 + kgrp * 4 + r;
+            stage[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC] =
+                from_float<T>(acc[rb][nb][r] + bias_v[nb]);
           }
         }
-        const int gi = r + DG;
-        const int32_t* pin = s_pin + (gi & (P_SLOTS - 1)) * STEP_ROWS;
-        const int32_t* pout = s_pout + (gi & (P_SLOTS - 1)) * STEP_ROWS;
-        // (slots past the step's pairs hold stale values that are not used)
-        int32_t pv[2];
+    } else {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) pv[j] = pin[(wave * 2 + j) * 8 + sub];
-        const int32_t pin_l = pin[lane], pout_l = pout[lane];
-        rR = step_raw(r + 1);
-        rG = step_raw(r + 1 + DG);
-        rW = step_raw(r + 1 + DW);
-        rP = step_raw(r + 1 + DP);
-        sw_next = *(const uint32_t*)(s_tab + ((r + 1) & (T_SLOTS - 1)) * ROWS + wrow + (lane & 15) * 4);
-
-        // ---- multiply step r - 1 (operands read in the previous iteration)
+      for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
-        for (int rb = 0; rb < 4; ++rb) {
-          if (!pany[rb]) continue;
+        for (int nb = 0; nb < NB; ++nb) {
+          const int col = n0 + nb * 16 + (lane & 15);
+          if (col >= a.c_out) continue;
 #pragma unroll
-          for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-            for (int nb = 0; nb < NBW; ++nb) acc[rb][nb] = M::mma(pav[rb][ks], pbfr[nb][ks], acc[rb][nb]);
+          for (int r = 0; r < 4; ++r) {
+            const int64_t orow = m0 + wrow + rb * 16 + kgrp * 4 + r;
+            if (orow < a.num_out) out[orow * a.c_out + col] = from_float<T>(acc[rb][nb][r] + bias_v[nb]);
+          }
         }
-
-        // ---- requests: W[k]^T of step r + DW, input rows of step r + DG, pairs of step r + DP
-        const int numG = step_num(dG.x);
-        const bool identG = step_identity(dG.x);
-        const int firstG = step_first(dG.x);
-        {
+    }
+  } else {
+    for (int c0 = 0; c0 < a.c_in_pad; c0 += CK) {
+      for (int kbase = 0; kbase < a.K; kbase += 32) {
+        const int S = begin_chunk(kbase);
+        if (S == 0) continue;
+        // ================= requesting waves =================
+        const int q = wave - 4;  // which quarter of the weight tile and of the step's rows
+        uint2 rW = step_raw(-DP + DW, S), rG = step_raw(-DP + DG, S), rP = step_raw(0, S);
+        int iw = (W_SLOTS - (DP - DW) % W_SLOTS) % W_SLOTS;  // (r + DW) mod W_SLOTS
+        int ia = (A_SLOTS - (DP - DG) % A_SLOTS) % A_SLOTS;  // (r + DG) mod A_SLOTS
+#pragma nounroll
+        for (int r = -DP; r < S; ++r) {
+          const uint2 dW = uniform(rW), dG = uniform(rG), dP = uniform(rP);
+          // this wave's share of what step r needs, and of the pairs of step r + DG, has landed:
+          // everything but the rows and pairs requested DW iterations ago and all that came later
+          if (q < 2) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 + 5 * (DW - 1)) : "memory");
+          } else {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 + 4 * (DW - 1)) : "memory");
+          }
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          const int gi = r + DG;
+          const int32_t* pin = s_pin + (gi & (P_SLOTS - 1)) * STEP_ROWS;
+          const int32_t* pout = s_pout + (gi & (P_SLOTS - 1)) * STEP_ROWS;
+          // all LDS reads first and unconditionally (slots past the step's pairs hold stale
+          // values that are not used)
+          int32_t pv[2];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) pv[j] = pin[(q * 2 + j) * 8 + sub];
+          const int32_t pin_l = pin[lane], pout_l = pout[lane];
+          rW = step_raw(r + 1 + DW, S);
+          rG = step_raw(r + 1 + DG, S);
+          rP = step_raw(r + 1 + DP, S);
+          const int numG = step_num(dG.x);
+          const bool identG = step_identity(dG.x);
+          const int firstG = step_first(dG.x);
           const int kW = kbase + step_k(dW.x);
           const T* wk = Wt + ((size_t)kW * a.c_out_pad + n0) * a.c_in_pad + c0;
           const T* wsrc[2];
           const uint8_t* xsrc[2];
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            const int n = (wave * 2 + j) * 8 + sub;
+            const int n = (q * 2 + j) * 8 + sub;
             wsrc[j] = wk + (uint32_t)n * (uint32_t)a.c_in_pad + (lpart ^ ((n >> 1) & 7)) * VEC;
           }
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            const int row = (wave * 2 + j) * 8 + sub;
+            const int row = (q * 2 + j) * 8 + sub;
             int32_t in = identG ? (int32_t)(m0 + firstG + row) : pv[j];
             if (row >= numG) in = -1;
             const int ps = lpart ^ ((row >> 1) & 7);  // source part kept at this LDS position
@@ -694,91 +775,45 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd_ring(ConvArgs a) {
                 (const uint8_t*)(X + ((uint64_t)(uint32_t)in * (uint32_t)a.c_in + (uint32_t)(c0 + ps * VEC)));
             xsrc[j] = ok ? real : zsrc + lane * 16;
           }
-          const int numP = step_identity(dP.x) ? 0 : step_num(dP.x);
-          const int32_t* list = wave == 0 ? a.in_maps : a.out_maps;
-          const uint8_t* psrc = zsrc + lane * 4;
-          if (wave < 2 && lane < numP) psrc = (const uint8_t*)(list + ((int64_t)dP.y + lane));
-          const uint8_t* pdst = smem + ZERO_OFF;  // waves 2 and 3: zeros onto the block of zeros
-          if (wave < 2) pdst = (const uint8_t*)((wave == 0 ? s_pin : s_pout) + ((r + DP) & (P_SLOTS - 1)) * STEP_ROWS);
-          const uint32_t wdst = lds_offset(wring + iw * SLOT_BYTES + wave * 2 * 1024);
-          const uint32_t xdst = lds_offset(ring + ia * SLOT_BYTES + wave * 2 * 1024);
+          const uint32_t wdst = lds_offset(wring + iw * SLOT_BYTES + q * 2 * 1024);
+          const uint32_t xdst = lds_offset(ring + ia * SLOT_BYTES + q * 2 * 1024);
 #pragma unroll
           for (int j = 0; j < 2; ++j) load_to_lds_16(wsrc[j], __builtin_amdgcn_readfirstlane(wdst + j * 1024));
 #pragma unroll
           for (int j = 0; j < 2; ++j) load_to_lds_16(xsrc[j], __builtin_amdgcn_readfirstlane(xdst + j * 1024));
-          load_to_lds_4(psrc, __builtin_amdgcn_readfirstlane(lds_offset(pdst)));
+          if (q < 2) {  // pairs of step r + DP: wave 4 the input rows, wave 5 the output rows
+            const int numP = step_identity(dP.x) ? 0 : step_num(dP.x);
+            const int32_t* list = q == 0 ? a.in_maps : a.out_maps;
+            const uint8_t* psrc = zsrc + lane * 4;
+            if (lane < numP) psrc = (const uint8_t*)(list + ((int64_t)dP.y + lane));
+            const uint32_t pdst = lds_offset(q == 0 ? s_pin : s_pout) +
+                                  (uint32_t)(((r + DP) & (P_SLOTS - 1)) * STEP_ROWS * 4);
+            load_to_lds_4(psrc, __builtin_amdgcn_readfirstlane(pdst));
+          } else if (q == 2) {  // slot table of step r + DG
+            int32_t pub_in = identG ? (int32_t)(m0 + firstG + lane) : pin_l;
+            const int pub_out = identG ? firstG + lane : (int)(pout_l - m0);
+            if (lane >= numG) pub_in = -1;
+            if ((uint32_t)pub_in < (uint64_t)a.num_in && (uint32_t)pub_out < (uint32_t)tile_rows)
+              s_tab[(gi & (T_SLOTS - 1)) * ROWS + (pub_out & ~63) + (pub_out & 15) * 4 + ((pub_out >> 4) & 3)] = (uint8_t)lane;
+          } else {  // the slot table after it starts empty
+            ((uint32_t*)(s_tab + ((gi + 1) & (T_SLOTS - 1)) * ROWS))[lane] = 0xFFFFFFFFu;
+          }
+          iw = iw + 1 == W_SLOTS ? 0 : iw + 1;
+          ia = ia + 1 == A_SLOTS ? 0 : ia + 1;
         }
-        // slot table of step r + DG (wave 2), clearing of the one after it (wave 3)
-        if (wave == 2) {
-          int32_t pub_in = identG ? (int32_t)(m0 + firstG + lane) : pin_l;
-          const int pub_out = identG ? firstG + lane : (int)(pout_l - m0);
-          if (lane >= numG) pub_in = -1;
-          if ((uint32_t)pub_in < (uint64_t)a.num_in && (uint32_t)pub_out < (uint32_t)tile_rows)
-            s_tab[(gi & (T_SLOTS - 1)) * ROWS + (pub_out & ~63) + (pub_out & 15) * 4 + ((pub_out >> 4) & 3)] = (uint8_t)lane;
-        } else if (wave == 3) {
-          ((uint32_t*)(s_tab + ((gi + 1) & (T_SLOTS - 1)) * ROWS))[lane] = 0xFFFFFFFFu;
-        }
-        ia = ia + 1 == A_SLOTS ? 0 : ia + 1;
-        im = im + 1 == A_SLOTS ? 0 : im + 1;
-        iw = iw + 1 == W_SLOTS ? 0 : iw + 1;
-        imw = imw + 1 == W_SLOTS ? 0 : imw + 1;
-      };
-      // r runs to S inclusive (the last iteration multiplies step S - 1); two iterations per trip
-      // so that the register sets alternate without copies (a surplus iteration is an empty step)
-#pragma nounroll
-      for (int r = -DP; r <= S; r += 2) {
-        iteration(r, bfr0, av0, any0, bfr1, av1, any1);
-        iteration(r + 1, bfr1, av1, any1, bfr0, av0, any0);
       }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the loads of the empty steps after the last one
+    __syncthreads();  // every wave is done with the rings, every load has landed
   }
-
-  // epilogue: bias add, one rounding to T
-  T* __restrict__ out = (T*)a.out;
-  const T* __restrict__ bias = (const T*)a.bias;
-  float bias_v[NBW];  // this lane's bias values, fetched together
-#pragma unroll
-  for (int nb = 0; nb < NBW; ++nb) {
-    const int col = n0 + nb * 16 + (lane & 15);
-    bias_v[nb] = (bias && col < a.c_out) ? to_float(bias[col]) : 0.f;
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the loads of the empty steps after the last one
-  __syncthreads();  // every wave is done with the rings
-  if (sizeof(T) == 2 && a.vec_out) {
-    T* stage = (T*)ring;  // 256 rows x 128 bytes
-#pragma unroll
-    for (int rb = 0; rb < 4; ++rb)
-#pragma unroll
-      for (int nb = 0; nb < NBW; ++nb) {
-        const int col = nb * 16 + (lane & 15);
-        const float bv = bias_v[nb];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int lr = wrow + rb * 16 + kgrp * 4 + r;
-          stage[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC] = from_float<T>(acc[rb][nb][r] + bv);
-        }
-      }
+  if (staged) {
     __syncthreads();
-    for (int v = tid; v < ROWS * 8; v += THREADS) {
+    for (int v = tid; v < ROWS * 8; v += RING_THREADS) {
       const int r = v >> 3, part = v & 7;
       if (m0 + r < a.num_out && n0 + part * VEC < a.c_out)
         *reinterpret_cast<u32x4*>(out + (m0 + r) * a.c_out + n0 + part * VEC) =
             *reinterpret_cast<const u32x4*>(&stage[r * CK + lds_part(r, part) * VEC]);
     }
-  } else {
-#pragma unroll
-    for (int rb = 0; rb < 4; ++rb)
-#pragma unroll
-      for (int nb = 0; nb < NBW; ++nb) {
-        const int col = n0 + nb * 16 + (lane & 15);
-        if (col >= a.c_out) continue;
-        const float bv = bias_v[nb];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int64_t orow = m0 + wrow + rb * 16 + kgrp * 4 + r;
-          if (orow < a.num_out) out[orow * a.c_out + col] = from_float<T>(acc[rb][nb][r] + bv);
-        }
-      }
   }
 }
 
@@ -988,7 +1023,7 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
     if (hipFuncSetAttribute((const void*)conv_fwd_ring<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             RING_LDS_BYTES) != hipSuccess)
       return WCN_ERR_LAUNCH;
-    hipLaunchKernelGGL(conv_fwd_ring<T>, grid, dim3(THREADS), RING_LDS_BYTES, s, a);
+    hipLaunchKernelGGL(conv_fwd_ring<T>, grid, dim3(RING_THREADS), RING_LDS_BYTES, s, a);
   } else {
     hipLaunchKernelGGL(conv_fwd<T>, grid, dim3(THREADS), 0, s, a);
   }
@@ -1115,5 +1150,6 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
 }
 
 }  // extern "C"
+
 
 
