@@ -131,6 +131,7 @@ struct ConvArgs {
   int32_t K, c_in, c_out, c_in_pad, c_out_pad, identity;
   int32_t vec_in;   // feature rows are 16-byte aligned and a whole number of 16-byte vectors
   int32_t vec_out;  // same for output rows
+  int32_t flat_in;  // c_in is a multiple of the staged row and the feature matrix is below 4 GiB
 };
 
 // LDS rows are 128 bytes (eight 16-byte parts) with no padding; part p of row r is stored at
@@ -512,6 +513,17 @@ __device__ __forceinline__ void load_to_lds_16(const void* g, uint32_t lds_off) 
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_off)
                : "memory", "m0");
 }
+// the same with a wave-uniform base address and a 32-bit unsigned byte offset per lane
+__device__ __forceinline__ void load_to_lds_16(const void* base, uint32_t lane_off, uint32_t lds_off) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base),
+               "s"(lds_off)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void load_to_lds_4(const void* base, uint32_t lane_off, uint32_t lds_off) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_off), "s"(base),
+               "s"(lds_off)
+               : "memory", "m0");
+}
 __device__ __forceinline__ void load_to_lds_4(const void* g, uint32_t lds_off) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_off)
                : "memory", "m0");
@@ -726,6 +738,18 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
         if (S == 0) continue;
         // ================= requesting waves =================
         const int q = wave - 4;  // which quarter of the weight tile and of the step's rows
+        const size_t w_tile_bytes = (size_t)a.c_out_pad * a.c_in_pad * sizeof(T);
+        const uint8_t* const wbase0 = (const uint8_t*)(Wt + (size_t)n0 * a.c_in_pad + c0);
+        const uint8_t* const xbase0 = a.num_in > 0 ? (const uint8_t*)(X + c0) : zsrc;
+        const uint32_t row_bytes = (uint32_t)a.c_in * (uint32_t)sizeof(T);
+        uint32_t w_lane_off[2], x_lane_off[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int n = (q * 2 + j) * 8 + sub;  // also the row inside the step's slot
+          const uint32_t part_off = (uint32_t)(lpart ^ ((n >> 1) & 7)) * 16u;  // source part kept at this LDS position
+          w_lane_off[j] = (uint32_t)n * (uint32_t)a.c_in_pad * (uint32_t)sizeof(T) + part_off;
+          x_lane_off[j] = part_off;
+        }
         uint2 rW = step_raw(-DP + DW, S), rG = step_raw(-DP + DG, S), rP = step_raw(0, S);
         int iw = (W_SLOTS - (DP - DW) % W_SLOTS) % W_SLOTS;  // (r + DW) mod W_SLOTS
         int ia = (A_SLOTS - (DP - DG) % A_SLOTS) % A_SLOTS;  // (r + DG) mod A_SLOTS
@@ -756,39 +780,50 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
           const bool identG = step_identity(dG.x);
           const int firstG = step_first(dG.x);
           const int kW = kbase + step_k(dW.x);
-          const T* wk = Wt + ((size_t)kW * a.c_out_pad + n0) * a.c_in_pad + c0;
-          const T* wsrc[2];
-          const uint8_t* xsrc[2];
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            const int n = (q * 2 + j) * 8 + sub;
-            wsrc[j] = wk + (uint32_t)n * (uint32_t)a.c_in_pad + (lpart ^ ((n >> 1) & 7)) * VEC;
-          }
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            const int row = (q * 2 + j) * 8 + sub;
-            int32_t in = identG ? (int32_t)(m0 + firstG + row) : pv[j];
-            if (row >= numG) in = -1;
-            const int ps = lpart ^ ((row >> 1) & 7);  // source part kept at this LDS position
-            const bool ok = (uint32_t)in < (uint64_t)a.num_in && c0 + ps * VEC < a.c_in;
-            const uint8_t* real =
-                (const uint8_t*)(X + ((uint64_t)(uint32_t)in * (uint32_t)a.c_in + (uint32_t)(c0 + ps * VEC)));
-            xsrc[j] = ok ? real : zsrc + lane * 16;
-          }
           const uint32_t wdst = lds_offset(wring + iw * SLOT_BYTES + q * 2 * 1024);
           const uint32_t xdst = lds_offset(ring + ia * SLOT_BYTES + q * 2 * 1024);
+          // weights: uniform base of the tile, this lane's fixed offset inside it
+          const uint8_t* const wk = wbase0 + (size_t)kW * w_tile_bytes;
 #pragma unroll
-          for (int j = 0; j < 2; ++j) load_to_lds_16(wsrc[j], __builtin_amdgcn_readfirstlane(wdst + j * 1024));
+          for (int j = 0; j < 2; ++j) load_to_lds_16(wk, w_lane_off[j], __builtin_amdgcn_readfirstlane(wdst + j * 1024));
+          if (a.flat_in) {
+            // rows: uniform base, row index times row size plus this lane's part (rows past the
+            // step's pairs and malformed indices fetch row 0; no slot entry ever points at them)
+            uint32_t xoff[2];
 #pragma unroll
-          for (int j = 0; j < 2; ++j) load_to_lds_16(xsrc[j], __builtin_amdgcn_readfirstlane(xdst + j * 1024));
+            for (int j = 0; j < 2; ++j) {
+              const int row = (q * 2 + j) * 8 + sub;
+              uint32_t in = identG ? (uint32_t)(m0 + firstG + row) : (uint32_t)pv[j];
+              if (row >= numG || in >= (uint32_t)a.num_in) in = 0u;
+              xoff[j] = in * row_bytes + x_lane_off[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) load_to_lds_16(xbase0, xoff[j], __builtin_amdgcn_readfirstlane(xdst + j * 1024));
+          } else {
+            const uint8_t* xsrc[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const int row = (q * 2 + j) * 8 + sub;
+              int32_t in = identG ? (int32_t)(m0 + firstG + row) : pv[j];
+              if (row >= numG) in = -1;
+              const int ps = lpart ^ ((row >> 1) & 7);  // source part kept at this LDS position
+              const bool ok = (uint32_t)in < (uint64_t)a.num_in && c0 + ps * VEC < a.c_in;
+              const uint8_t* real =
+                  (const uint8_t*)(X + ((uint64_t)(uint32_t)in * (uint32_t)a.c_in + (uint32_t)(c0 + ps * VEC)));
+              xsrc[j] = ok ? real : zsrc + lane * 16;
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) load_to_lds_16(xsrc[j], __builtin_amdgcn_readfirstlane(xdst + j * 1024));
+          }
           if (q < 2) {  // pairs of step r + DP: wave 4 the input rows, wave 5 the output rows
             const int numP = step_identity(dP.x) ? 0 : step_num(dP.x);
             const int32_t* list = q == 0 ? a.in_maps : a.out_maps;
-            const uint8_t* psrc = zsrc + lane * 4;
-            if (lane < numP) psrc = (const uint8_t*)(list + ((int64_t)dP.y + lane));
+            // lanes past the step's pairs repeat its last pair (never used); empty steps read zeros
+            const uint8_t* pbase = numP > 0 ? (const uint8_t*)(list + (int64_t)dP.y) : zsrc;
+            const uint32_t poff = (uint32_t)(numP > 0 ? (lane < numP ? lane : numP - 1) : lane) * 4u;
             const uint32_t pdst = lds_offset(q == 0 ? s_pin : s_pout) +
                                   (uint32_t)(((r + DP) & (P_SLOTS - 1)) * STEP_ROWS * 4);
-            load_to_lds_4(psrc, __builtin_amdgcn_readfirstlane(pdst));
+            load_to_lds_4(pbase, poff, __builtin_amdgcn_readfirstlane(pdst));
           } else if (q == 2) {  // slot table of step r + DG
             int32_t pub_in = identG ? (int32_t)(m0 + firstG + lane) : pin_l;
             const int pub_out = identG ? firstG + lane : (int)(pout_l - m0);
@@ -1142,6 +1177,7 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
   const size_t es = elem_size(dtype);
   a.vec_in = (((size_t)c_in * es) % 16 == 0 && ((uintptr_t)features % 16) == 0) ? 1 : 0;
   a.vec_out = (((size_t)c_out * es) % 16 == 0 && ((uintptr_t)out % 16) == 0) ? 1 : 0;
+  a.flat_in = (c_in % ck_of(dtype) == 0 && (uint64_t)num_in * c_in * es < (1ull << 32)) ? 1 : 0;
   switch (dtype) {
     case WCN_DTYPE_F32: return launch_conv<float>(a, weight, weight_dtype, dtype, s);
     case WCN_DTYPE_F16: return launch_conv<_Float16>(a, weight, weight_dtype, dtype, s);
