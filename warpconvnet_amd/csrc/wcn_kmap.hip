@@ -2,12 +2,14 @@
 //
 // The reference materialises a dense (K, M) table of probe results and compacts it with several
 // passes (torch_discrete.py:80-157).  Here one thread owns one output voxel and resolves its K
-// offsets in registers; a wave's 64 voxels form a "group".  Pass 1 (count) stores, per offset and
-// group, how many of the 64 probes hit (a ballot popcount); a row-wise exclusive scan turns the
-// counts into start positions; pass 2 (fill) repeats the probes and each lane writes its pair at
-// start + (number of hits in lower lanes).  Because groups are 64 consecutive output rows and
-// lanes ascend within a group, pairs come out in ascending output index for each offset, exactly
-// the reference's order (discrete_kernels.cu:183-213), with no (K, M) intermediate in HBM.
+// offsets in registers; a wave's 64 voxels form a "group".  The probe pass stores, per offset and
+// group, the 64-bit mask of lanes that hit and its popcount, and each hit lane parks the input
+// row it found at (offset, output row) of a scratch table (only hits are written).  A row-wise
+// exclusive scan turns the counts into start positions; the emit pass then reads masks, starts
+// and parked rows -- no table probes -- and every hit lane writes its pair at start + (number of
+// hits in lower lanes).  Because groups are 64 consecutive output rows and lanes ascend within a
+// group, pairs come out in ascending output index for each offset, exactly the reference's order
+// (discrete_kernels.cu:183-213).
 #include "wcn_common.h"
 
 int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView& v,
@@ -28,6 +30,8 @@ struct KmapWorkspace {  // host-computed addresses inside a kmap workspace
   int64_t* row_total;   // [K+1] totals of the rows of `groups`
   int32_t* groups;      // (K+1, G+1): rows 0..K-1 per-offset hit counts of each 64-row group, row K
                         // all hits of the group; after the scan, exclusive prefix sums
+  unsigned long long* hits;  // (G, K): lanes of the group that hit, per offset
+  int32_t* found;       // (K, 64 G): input row found by (offset, output row); hits only
   int64_t G;            // number of 64-row groups
 };
 
@@ -41,6 +45,10 @@ inline size_t kmap_layout(void* base, int64_t num_out, int32_t K, KmapWorkspace*
   off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
   if (w) w->groups = (int32_t*)(p + off);
   off += wcn_align256(sizeof(int32_t) * (size_t)(K + 1) * (size_t)(G + 1));
+  if (w) w->hits = (unsigned long long*)(p + off);
+  off += wcn_align256(sizeof(unsigned long long) * (size_t)K * (size_t)G);
+  if (w) w->found = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)K * (size_t)G * 64);
   if (w) w->G = G;
   return off;
 }
@@ -50,15 +58,14 @@ inline int grid_for(int64_t n, int block) {
   return (int)(g < 1 ? 1 : g);
 }
 
-struct KmapOut {        // outputs of the fill pass (all may be null in the count pass)
-  int32_t* in_maps;
-  int32_t* out_maps;
+struct KmapProbe {      // what the probe pass leaves for the emit pass
+  unsigned long long* hits;
+  int32_t* found;
 };
 
 // ---- generic kernel: any kernel size up to WCN_MAX_OFFSETS offsets -----------------------------
 // Probe results are produced offset by offset; consecutive offsets differ in z (the fastest
 // digit) and mostly fall in the block of the previous probe, whose slot is kept in registers.
-template <bool FILL>
 __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restrict__ hdr,
                                                  const WcnSlot* __restrict__ slots,
                                                  uint32_t cap_mask,
@@ -66,7 +73,7 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
                                                  const int4* __restrict__ out_coords,
                                                  int64_t num_out, KmapGeom g,
                                                  int32_t* __restrict__ groups, int64_t G,
-                                                 const int64_t* __restrict__ offsets, KmapOut o) {
+                                                 KmapProbe o) {
   const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t group = m >> 6;  // wave-uniform
   if (group >= G) return;
@@ -100,28 +107,25 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
           if ((cached_mask >> bit) & 1ull) found = perm[cached_base + wcn_rank_below(cached_mask, bit)];
         }
         const unsigned long long hits = __ballot(found >= 0);
-        if (!FILL) {
-          const int cnt = __popcll(hits);
-          group_hits += cnt;
-          if (lane == 0) groups[(int64_t)k * (G + 1) + group] = cnt;
-        } else if (found >= 0) {
-          const int64_t pos = offsets[k] + groups[(int64_t)k * (G + 1) + group] +
-                              __popcll(hits & ((1ull << lane) - 1ull));
-          o.in_maps[pos] = found;
-          o.out_maps[pos] = (int32_t)m;
+        const int cnt = __popcll(hits);
+        group_hits += cnt;
+        if (lane == 0) {
+          groups[(int64_t)k * (G + 1) + group] = cnt;
+          o.hits[group * g.K + k] = hits;
         }
+        if (found >= 0) o.found[(int64_t)k * (G * 64) + m] = found;
       }
     }
   }
-  if (!FILL && lane == 0) groups[(int64_t)g.K * (G + 1) + group] = group_hits;
+  if (lane == 0) groups[(int64_t)g.K * (G + 1) + group] = group_hits;
 }
 
 // ---- fixed-size kernel: compile-time kernel size, every dimension spans at most 2 blocks -------
 // Phase 1 requests the (up to) 8 block slots the neighbourhood can touch, all at once, so their
 // memory latencies overlap; phase 2 derives the hit bit of each of the K offsets from the cached
-// masks (no memory traffic); phase 3 (fill only) reads the hit rows from `perm`, again as
-// independent loads, and writes both forms of the map.
-template <int KX, int KY, int KZ, bool FILL>
+// masks (no memory traffic); phase 3 reads the hit rows from `perm`, again as independent loads,
+// and leaves masks, counts and rows for the emit pass.
+template <int KX, int KY, int KZ>
 __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __restrict__ hdr,
                                                        const WcnSlot* __restrict__ slots,
                                                        uint32_t cap_mask,
@@ -129,8 +133,7 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
                                                        const int4* __restrict__ out_coords,
                                                        int64_t num_out, KmapGeom g,
                                                        int32_t* __restrict__ groups, int64_t G,
-                                                       const int64_t* __restrict__ offsets,
-                                                       KmapOut o) {
+                                                       KmapProbe o) {
   constexpr int K = KX * KY * KZ;
   static_assert(K <= 32 && KX <= 5 && KY <= 5 && KZ <= 5, "fixed kernel covers small kernels");
   __shared__ unsigned long long s_mask[8][256];
@@ -219,37 +222,83 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
           const unsigned long long mk = s_mask[e][tid];
           const uint32_t hit = (uint32_t)((mk >> bit) & 1ull);
           hm |= hit << k;
-          if (FILL) pos[k] = s_base[e][tid] + wcn_rank_below(mk, bit);
+          pos[k] = s_base[e][tid] + wcn_rank_below(mk, bit);
         }
       }
     }
-  }
-
-  if (!FILL) {
-    int group_hits = 0;
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-      const int cnt = __popcll(__ballot((hm >> k) & 1u));
-      group_hits += cnt;
-      if (lane == 0) groups[(int64_t)k * (G + 1) + group] = cnt;
-    }
-    if (lane == 0) groups[(int64_t)K * (G + 1) + group] = group_hits;
-    return;
   }
 
   int32_t found[K];
 #pragma unroll
   for (int k = 0; k < K; ++k) found[k] = ((hm >> k) & 1u) ? perm[pos[k]] : -1;
 
+  int group_hits = 0;
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     const bool hit = (hm >> k) & 1u;
     const unsigned long long hits = __ballot(hit);
-    if (hit) {
-      const int64_t p = offsets[k] + groups[(int64_t)k * (G + 1) + group] +
-                        __popcll(hits & ((1ull << lane) - 1ull));
-      o.in_maps[p] = found[k];
-      o.out_maps[p] = (int32_t)m;
+    const int cnt = __popcll(hits);
+    group_hits += cnt;
+    if (lane == 0) {
+      groups[(int64_t)k * (G + 1) + group] = cnt;
+      o.hits[group * K + k] = hits;
+    }
+    if (hit) o.found[(int64_t)k * (G * 64) + m] = found[k];
+  }
+  if (lane == 0) groups[(int64_t)K * (G + 1) + group] = group_hits;
+}
+
+// Emit pass: pair lists from the masks, scanned counts and parked rows of the probe pass.  Lane j
+// fetches mask and start of offset k0 + j for the whole group; the lanes then walk the offsets
+// together.
+template <int KFIX>
+__global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __restrict__ hits,
+                                                 const int32_t* __restrict__ found,
+                                                 const int32_t* __restrict__ groups,
+                                                 const int64_t* __restrict__ offsets, int K_runtime,
+                                                 int64_t G, int32_t* __restrict__ in_maps,
+                                                 int32_t* __restrict__ out_maps) {
+  const int K = KFIX > 0 ? KFIX : K_runtime;
+  const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t group = m >> 6;  // wave-uniform
+  if (group >= G) return;
+  const int lane = wcn_lane();
+  const unsigned long long below = (1ull << lane) - 1ull;
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    unsigned long long h = 0ull;
+    long long st = 0;
+    if (k0 + lane < K) {
+      h = hits[group * K + k0 + lane];
+      st = offsets[k0 + lane] + groups[(int64_t)(k0 + lane) * (G + 1) + group];
+    }
+    const int n = K - k0 < 64 ? K - k0 : 64;
+    if (KFIX > 0) {
+      int32_t row[KFIX > 0 ? KFIX : 1];
+#pragma unroll
+      for (int j = 0; j < KFIX; ++j) {
+        const unsigned long long hj = __shfl(h, j, 64);
+        row[j] = ((hj >> lane) & 1ull) ? found[(int64_t)j * (G * 64) + m] : -1;
+      }
+#pragma unroll
+      for (int j = 0; j < KFIX; ++j) {
+        const unsigned long long hj = __shfl(h, j, 64);
+        const long long sj = __shfl(st, j, 64);
+        if ((hj >> lane) & 1ull) {
+          const long long p = sj + __popcll(hj & below);
+          in_maps[p] = row[j];
+          out_maps[p] = (int32_t)m;
+        }
+      }
+    } else {
+      for (int j = 0; j < n; ++j) {
+        const unsigned long long hj = __shfl(h, j, 64);
+        const long long sj = __shfl(st, j, 64);
+        if ((hj >> lane) & 1ull) {
+          const long long p = sj + __popcll(hj & below);
+          in_maps[p] = found[(int64_t)(k0 + j) * (G * 64) + m];
+          out_maps[p] = (int32_t)m;
+        }
+      }
     }
   }
 }
@@ -336,23 +385,36 @@ inline bool table_args_ok(const void* table, int64_t n_keys, int64_t capacity) {
   return table && n_keys >= 0 && capacity >= 64 && (capacity & (capacity - 1)) == 0;
 }
 
-template <bool FILL>
-void launch_pass(const WcnTableView& v, const int32_t* out_coords, int64_t num_out,
-                 const KmapGeom& g, const KmapWorkspace& w, const KmapOut& o, hipStream_t s) {
+void launch_probe(const WcnTableView& v, const int32_t* out_coords, int64_t num_out,
+                  const KmapGeom& g, const KmapWorkspace& w, hipStream_t s) {
   const dim3 grid(grid_for(num_out, 256)), block(256);
   const uint32_t cap_mask = (uint32_t)(v.capacity - 1);
-  const int64_t* offsets = FILL ? (const int64_t*)w.result : nullptr;
+  const KmapProbe o = {w.hits, w.found};
   if (is_fixed_size(g, 3, 3, 3)) {
-    hipLaunchKernelGGL((kmap_pass_fixed<3, 3, 3, FILL>), grid, block, 0, s, v.hdr, v.slots,
-                       cap_mask, v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G,
-                       offsets, o);
+    hipLaunchKernelGGL((kmap_pass_fixed<3, 3, 3>), grid, block, 0, s, v.hdr, v.slots, cap_mask,
+                       v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G, o);
   } else if (is_fixed_size(g, 2, 2, 2)) {
-    hipLaunchKernelGGL((kmap_pass_fixed<2, 2, 2, FILL>), grid, block, 0, s, v.hdr, v.slots,
-                       cap_mask, v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G,
-                       offsets, o);
+    hipLaunchKernelGGL((kmap_pass_fixed<2, 2, 2>), grid, block, 0, s, v.hdr, v.slots, cap_mask,
+                       v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G, o);
   } else {
-    hipLaunchKernelGGL(kmap_pass<FILL>, grid, block, 0, s, v.hdr, v.slots, cap_mask, v.perm,
-                       (const int4*)out_coords, num_out, g, w.groups, w.G, offsets, o);
+    hipLaunchKernelGGL(kmap_pass, grid, block, 0, s, v.hdr, v.slots, cap_mask, v.perm,
+                       (const int4*)out_coords, num_out, g, w.groups, w.G, o);
+  }
+}
+
+void launch_emit(int64_t num_out, const KmapGeom& g, const KmapWorkspace& w, int32_t* in_maps,
+                 int32_t* out_maps, hipStream_t s) {
+  const dim3 grid(grid_for(num_out, 256)), block(256);
+  const int64_t* offsets = (const int64_t*)w.result;
+  if (g.K == 27) {
+    hipLaunchKernelGGL(kmap_emit<27>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
+                       w.G, in_maps, out_maps);
+  } else if (g.K == 8) {
+    hipLaunchKernelGGL(kmap_emit<8>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
+                       w.G, in_maps, out_maps);
+  } else {
+    hipLaunchKernelGGL(kmap_emit<0>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
+                       w.G, in_maps, out_maps);
   }
 }
 
@@ -469,8 +531,7 @@ int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const in
   wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
   KmapWorkspace w;
   kmap_layout(workspace, num_out, g.K, &w);
-  const KmapOut none = {nullptr, nullptr};
-  if (w.G > 0) launch_pass<false>(v, out_coords, num_out, g, w, none, s);
+  if (w.G > 0) launch_probe(v, out_coords, num_out, g, w, s);
   hipLaunchKernelGGL(kmap_scan_rows, dim3(g.K + 1), dim3(1024), 0, s, w.groups, w.G, w.row_total);
   hipLaunchKernelGGL(kmap_finish, dim3(1), dim3(64), 0, s, w.result, w.row_total, g.K, v.hdr);
   WCN_LAUNCH_CHECK();
@@ -510,8 +571,7 @@ int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int
   wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
   KmapWorkspace w;
   kmap_layout(const_cast<void*>(workspace), num_out, g.K, &w);
-  const KmapOut o = {in_maps, out_maps};
-  launch_pass<true>(v, out_coords, num_out, g, w, o, (hipStream_t)stream);
+  launch_emit(num_out, g, w, in_maps, out_maps, (hipStream_t)stream);
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }
