@@ -3,8 +3,8 @@
 // The reference materialises a dense (K, M) table of probe results and compacts it with several
 // passes (torch_discrete.py:80-157).  Here one thread owns one output voxel and resolves its K
 // offsets in registers; a wave's 64 voxels form a "group".  The probe pass stores, per offset and
-// group, the 64-bit mask of lanes that hit and its popcount, and each hit lane parks the input
-// row it found at (offset, output row) of a scratch table (only hits are written).  A row-wise
+// group, the 64-bit mask of lanes that hit and its popcount, and the hit lanes park the input
+// rows they found, packed in lane order, in the (offset, group) cell of a scratch table.  A row-wise
 // exclusive scan turns the counts into start positions; the emit pass then reads masks, starts
 // and parked rows -- no table probes -- and every hit lane writes its pair at start + (number of
 // hits in lower lanes).  Because groups are 64 consecutive output rows and lanes ascend within a
@@ -31,7 +31,7 @@ struct KmapWorkspace {  // host-computed addresses inside a kmap workspace
   int32_t* groups;      // (K+1, G+1): rows 0..K-1 per-offset hit counts of each 64-row group, row K
                         // all hits of the group; after the scan, exclusive prefix sums
   unsigned long long* hits;  // (G, K): lanes of the group that hit, per offset
-  int32_t* found;       // (K, 64 G): input row found by (offset, output row); hits only
+  int32_t* found;       // (K, 64 G): input rows found by the hit lanes of (offset, group), packed
   int64_t G;            // number of 64-row groups
 };
 
@@ -113,7 +113,8 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
           groups[(int64_t)k * (G + 1) + group] = cnt;
           o.hits[group * g.K + k] = hits;
         }
-        if (found >= 0) o.found[(int64_t)k * (G * 64) + m] = found;
+        if (found >= 0)  // hits of a group are parked contiguously, in lane order
+          o.found[(int64_t)k * (G * 64) + group * 64 + __popcll(hits & ((1ull << lane) - 1ull))] = found;
       }
     }
   }
@@ -243,7 +244,8 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
       groups[(int64_t)k * (G + 1) + group] = cnt;
       o.hits[group * K + k] = hits;
     }
-    if (hit) o.found[(int64_t)k * (G * 64) + m] = found[k];
+    if (hit)  // hits of a group are parked contiguously, in lane order
+      o.found[(int64_t)k * (G * 64) + group * 64 + __popcll(hits & ((1ull << lane) - 1ull))] = found[k];
   }
   if (lane == 0) groups[(int64_t)K * (G + 1) + group] = group_hits;
 }
@@ -277,7 +279,7 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
 #pragma unroll
       for (int j = 0; j < KFIX; ++j) {
         const unsigned long long hj = __shfl(h, j, 64);
-        row[j] = ((hj >> lane) & 1ull) ? found[(int64_t)j * (G * 64) + m] : -1;
+        row[j] = ((hj >> lane) & 1ull) ? found[(int64_t)j * (G * 64) + group * 64 + __popcll(hj & below)] : -1;
       }
 #pragma unroll
       for (int j = 0; j < KFIX; ++j) {
@@ -295,7 +297,7 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
         const long long sj = __shfl(st, j, 64);
         if ((hj >> lane) & 1ull) {
           const long long p = sj + __popcll(hj & below);
-          in_maps[p] = found[(int64_t)(k0 + j) * (G * 64) + m];
+          in_maps[p] = found[(int64_t)(k0 + j) * (G * 64) + group * 64 + __popcll(hj & below)];
           out_maps[p] = (int32_t)m;
         }
       }

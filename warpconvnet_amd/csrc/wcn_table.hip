@@ -37,10 +37,12 @@ __global__ void __launch_bounds__(256) table_clear(WcnTableHeader* __restrict__ 
   for (int64_t i = tid; i < n_keys; i += nthreads) perm[i] = INT32_MAX;
 }
 
-__global__ void __launch_bounds__(256) table_bbox(const int4* __restrict__ keys, int64_t n_keys,
-                                                  WcnTableHeader* __restrict__ hdr) {
-  __shared__ int s_mn[4][4];
-  __shared__ int s_mx[4][4];
+// Bounding box of the keys.  Few, wide workgroups: the eight atomics a workgroup ends with all
+// land on the same eight words and serialise, so their number decides the run time.
+__global__ void __launch_bounds__(1024) table_bbox(const int4* __restrict__ keys, int64_t n_keys,
+                                                   WcnTableHeader* __restrict__ hdr) {
+  __shared__ int s_mn[16][4];
+  __shared__ int s_mx[16][4];
   int mn[4] = {INT32_MAX, INT32_MAX, INT32_MAX, INT32_MAX};
   int mx[4] = {INT32_MIN, INT32_MIN, INT32_MIN, INT32_MIN};
   const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
@@ -71,7 +73,7 @@ __global__ void __launch_bounds__(256) table_bbox(const int4* __restrict__ keys,
   if (threadIdx.x < 4) {
     const int d = threadIdx.x;
     int a = s_mn[0][d], b = s_mx[0][d];
-    for (int w = 1; w < 4; ++w) {
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) {
       a = min(a, s_mn[w][d]);
       b = max(b, s_mx[w][d]);
     }
@@ -121,36 +123,47 @@ __global__ void __launch_bounds__(256) table_insert(const int4* __restrict__ key
   slot_of[i] = placed;
 }
 
-// base of every occupied slot = running sum of block populations.  One pass over all slots;
-// a 1024-thread workgroup scans its slots and takes its share of the running sum with a single
-// atomic, so the counter sees capacity / 1024 updates.
+// base of every occupied slot = running sum of block populations.  A 1024-thread workgroup owns
+// BASE_CHUNKS x 1024 consecutive slots, scans them and takes its share of the running sum with a
+// single atomic (the atomics of all workgroups serialise on one word, so there should be few).
+constexpr int BASE_CHUNKS = 8;
 __global__ void __launch_bounds__(1024) table_base(WcnTableHeader* __restrict__ hdr,
                                                    WcnSlot* __restrict__ slots, int64_t capacity) {
-  __shared__ int s_wave[16];
+  __shared__ int s_wave[BASE_CHUNKS][16];
   __shared__ int s_occ[16];
   __shared__ int s_group_base;
-  const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t j0 = (int64_t)blockIdx.x * (BASE_CHUNKS * 1024) + threadIdx.x;
   const int lane = wcn_lane(), wave = threadIdx.x >> 6;
-  int cnt = 0;
-  if (j < capacity) cnt = __popcll(slots[j].mask);
-  const int incl = wcn_wave_inclusive_sum(cnt);
-  const unsigned long long occupied = __ballot(cnt > 0);
-  if (lane == 63) s_wave[wave] = incl;
-  if (lane == 0) s_occ[wave] = __popcll(occupied);
+  int cnt[BASE_CHUNKS], incl[BASE_CHUNKS], occ = 0;
+#pragma unroll
+  for (int t = 0; t < BASE_CHUNKS; ++t) {
+    const int64_t j = j0 + (int64_t)t * 1024;
+    cnt[t] = j < capacity ? __popcll(slots[j].mask) : 0;
+  }
+#pragma unroll
+  for (int t = 0; t < BASE_CHUNKS; ++t) {
+    incl[t] = wcn_wave_inclusive_sum(cnt[t]);
+    occ += __popcll(__ballot(cnt[t] > 0));
+    if (lane == 63) s_wave[t][wave] = incl[t];
+  }
+  if (lane == 0) s_occ[wave] = occ;
   __syncthreads();
   if (threadIdx.x == 0) {
-    int total = 0, occ = 0;
-    for (int w = 0; w < 16; ++w) {
-      const int t = s_wave[w];
-      s_wave[w] = total;  // exclusive prefix over the waves
-      total += t;
-      occ += s_occ[w];
-    }
+    int total = 0, blocks = 0;
+    for (int t = 0; t < BASE_CHUNKS; ++t)
+      for (int w = 0; w < 16; ++w) {
+        const int v = s_wave[t][w];
+        s_wave[t][w] = total;  // exclusive prefix over (chunk, wave)
+        total += v;
+      }
+    for (int w = 0; w < 16; ++w) blocks += s_occ[w];
     s_group_base = total ? atomicAdd(&hdr->total, total) : 0;
-    if (occ) atomicAdd(&hdr->num_blocks, occ);
+    if (blocks) atomicAdd(&hdr->num_blocks, blocks);
   }
   __syncthreads();
-  if (cnt > 0) slots[j].base = s_group_base + s_wave[wave] + incl - cnt;
+#pragma unroll
+  for (int t = 0; t < BASE_CHUNKS; ++t)
+    if (cnt[t] > 0) slots[j0 + (int64_t)t * 1024].base = s_group_base + s_wave[t][wave] + incl[t] - cnt[t];
 }
 
 __global__ void __launch_bounds__(256) table_perm(const int4* __restrict__ keys, int64_t n_keys,
@@ -214,11 +227,11 @@ int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView
   hipLaunchKernelGGL(table_clear, dim3(grid_for(clear_items, 256, 4096)), dim3(256), 0, s, v.hdr,
                      v.slots, v.capacity, v.perm, n_keys);
   if (n_keys > 0) {
-    hipLaunchKernelGGL(table_bbox, dim3(grid_for(n_keys, 256 * 16, 512)), dim3(256), 0, s,
+    hipLaunchKernelGGL(table_bbox, dim3(grid_for(n_keys, 1024 * 8, 128)), dim3(1024), 0, s,
                        (const int4*)keys, n_keys, v.hdr);
     hipLaunchKernelGGL(table_insert, dim3(grid_for(n_keys, 256)), dim3(256), 0, s,
                        (const int4*)keys, n_keys, v.hdr, v.slots, cap_mask, v.slot_of);
-    hipLaunchKernelGGL(table_base, dim3(grid_for(v.capacity, 1024)), dim3(1024), 0, s, v.hdr,
+    hipLaunchKernelGGL(table_base, dim3(grid_for(v.capacity, 1024 * BASE_CHUNKS)), dim3(1024), 0, s, v.hdr,
                        v.slots, v.capacity);
     hipLaunchKernelGGL(table_perm, dim3(grid_for(n_keys, 256)), dim3(256), 0, s,
                        (const int4*)keys, n_keys, v.hdr, v.slots, v.slot_of, v.perm);
