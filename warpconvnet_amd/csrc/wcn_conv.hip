@@ -686,7 +686,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
               for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
-                  acc[rb][nb] = M::mma(av[rb & 1][ks], bfr[nb][ks], acc[rb][nb]);
+                  acc[rb][nb] = M::mma(bfr[nb][ks], av[rb & 1][ks], acc[rb][nb]);  // (W^T X^T): channels x rows
             }
           }
           im = im + 1 == A_SLOTS ? 0 : im + 1;
@@ -694,42 +694,43 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
         }
       }
     }
-    // epilogue: bias add, one rounding to T
+    // epilogue: bias add, one rounding to T.  The products were taken transposed, so a lane holds
+    // four consecutive output channels (4 * kgrp ..) of output row (lane & 15) of every 16 x 16
+    // block.  16-bit outputs are staged in LDS (8 bytes per lane and block) for whole-row stores.
     const T* __restrict__ bias = (const T*)a.bias;
-    float bias_v[NB];  // this lane's bias values, fetched together
+    float bias_v[NB][4];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      const int col = n0 + nb * 16 + (lane & 15);
-      bias_v[nb] = (bias && col < a.c_out) ? to_float(bias[col]) : 0.f;
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the loads of the empty steps after the last one
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int col = n0 + nb * 16 + kgrp * 4 + r;
+        bias_v[nb][r] = (bias && col < a.c_out) ? to_float(bias[col]) : 0.f;
+      }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // every wave is done with the rings, every load has landed
-    if (staged) {
 #pragma unroll
-      for (int rb = 0; rb < 4; ++rb)
+    for (int rb = 0; rb < 4; ++rb) {
+      const int lr = wrow + rb * 16 + (lane & 15);
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          const int col = nb * 16 + (lane & 15);
+      for (int nb = 0; nb < NB; ++nb) {
+        const int col = nb * 16 + kgrp * 4;
+        T v[4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int lr = wrow + rb * 16 + kgrp * 4 + r;
-            stage[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC] =
-                from_float<T>(acc[rb][nb][r] + bias_v[nb]);
+        for (int r = 0; r < 4; ++r) v[r] = from_float<T>(acc[rb][nb][r] + bias_v[nb][r]);
+        if (staged) {
+          *reinterpret_cast<uint2*>(&stage[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC]) =
+              *reinterpret_cast<const uint2*>(v);
+        } else if (m0 + lr < a.num_out) {
+          T* dst = out + (m0 + lr) * a.c_out + n0 + col;
+          if (sizeof(T) == 4 && a.vec_out && n0 + col + 3 < a.c_out) {
+            *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(v);
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (n0 + col + r < a.c_out) dst[r] = v[r];
           }
         }
-    } else {
-#pragma unroll
-      for (int rb = 0; rb < 4; ++rb)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          const int col = n0 + nb * 16 + (lane & 15);
-          if (col >= a.c_out) continue;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int64_t orow = m0 + wrow + rb * 16 + kgrp * 4 + r;
-            if (orow < a.num_out) out[orow * a.c_out + col] = from_float<T>(acc[rb][nb][r] + bias_v[nb]);
-          }
-        }
+      }
     }
   } else {
     for (int c0 = 0; c0 < a.c_in_pad; c0 += CK) {
@@ -1053,11 +1054,20 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
                        (T*)a.Wt, (uint32_t*)a.zeros);
   }
   const dim3 grid((unsigned)((a.num_out + ROWS - 1) / ROWS), (unsigned)(a.c_out_pad / TN));
+  if (a.vec_in) {
+    // more than 64 KiB of dynamic LDS has to be allowed once per device
+    static thread_local int allowed_device = -1;
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return WCN_ERR_LAUNCH;
+    if (allowed_device != device) {
+      if (hipFuncSetAttribute((const void*)conv_fwd_ring<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              RING_LDS_BYTES) != hipSuccess)
+        return WCN_ERR_LAUNCH;
+      allowed_device = device;
+    }
+  }
   if (g_time_start) (void)hipEventRecord(g_time_start, s);
   if (a.vec_in) {
-    if (hipFuncSetAttribute((const void*)conv_fwd_ring<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            RING_LDS_BYTES) != hipSuccess)
-      return WCN_ERR_LAUNCH;
     hipLaunchKernelGGL(conv_fwd_ring<T>, grid, dim3(RING_THREADS), RING_LDS_BYTES, s, a);
   } else {
     hipLaunchKernelGGL(conv_fwd<T>, grid, dim3(THREADS), 0, s, a);
