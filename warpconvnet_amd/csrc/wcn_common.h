@@ -173,6 +173,16 @@ __device__ __forceinline__ int wcn_wave_inclusive_sum(int v) {
   return v;
 }
 
+#endif  // __HIPCC__
+
+// Small device-to-host reads (map offsets, table status, row counts): copied into pinned memory
+// and awaited by polling an event, which returns within a few microseconds of the copy's end (a
+// blocking stream synchronisation wakes the host tens of microseconds later).  One staging buffer
+// and one event per host thread, created on first use and kept until the process ends.
+int wcn_read_small(void* host_dst, const void* device_src, size_t bytes, hipStream_t stream);
+
+#ifdef __HIPCC__
+
 #define WCN_LAUNCH_CHECK()                      \
   do {                                          \
     if (hipGetLastError() != hipSuccess) return WCN_ERR_LAUNCH; \

@@ -548,10 +548,7 @@ int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_off
   kmap_layout(const_cast<void*>(workspace), num_out, num_offsets, &w);
   int64_t tmp[WCN_MAX_OFFSETS + 3];
   const size_t bytes = sizeof(int64_t) * (size_t)(num_offsets + 3);
-  if (hipMemcpyAsync(tmp, w.result, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream) !=
-      hipSuccess)
-    return WCN_ERR_LAUNCH;
-  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return WCN_ERR_LAUNCH;
+  if (wcn_read_small(tmp, w.result, bytes, (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
   for (int k = 0; k <= num_offsets; ++k) host_offsets[k] = tmp[k];
   const int st = wcn_table_status_from_bits((int32_t)tmp[num_offsets + 1]);
   if (st != WCN_OK) return st;
@@ -631,10 +628,7 @@ int wcn_stride_unique_read_count(const void* workspace, int64_t n, int64_t capac
   StrideWorkspace w;
   stride_layout(const_cast<void*>(workspace), n, capacity, &w);
   int64_t tmp[2];
-  if (hipMemcpyAsync(tmp, w.result, sizeof(tmp), hipMemcpyDeviceToHost, (hipStream_t)stream) !=
-      hipSuccess)
-    return WCN_ERR_LAUNCH;
-  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return WCN_ERR_LAUNCH;
+  if (wcn_read_small(tmp, w.result, sizeof(tmp), (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
   *host_count = tmp[0];
   return wcn_table_status_from_bits((int32_t)tmp[1]);
 }

@@ -9,6 +9,8 @@
 //
 // HBM traffic per key: 16 B read (bbox) + 16 B read (insert) + 4 B slot_of write + 4 B read +
 // 4 B perm write, plus 32 B per table slot to clear and one 32 B slot touched per key.
+#include <string.h>
+
 #include "wcn_common.h"
 
 namespace {
@@ -240,6 +242,40 @@ int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView
   return WCN_OK;
 }
 
+int wcn_read_small(void* host_dst, const void* device_src, size_t bytes, hipStream_t stream) {
+  constexpr size_t kStaging = 16384;
+  thread_local void* staging = nullptr;
+  thread_local hipEvent_t done = nullptr;
+  thread_local int staging_device = -1;
+  if (bytes > kStaging) return WCN_ERR_INVALID_ARGUMENT;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return WCN_ERR_LAUNCH;
+  if (!staging) {
+    if (hipHostMalloc(&staging, kStaging, hipHostMallocDefault) != hipSuccess) {
+      staging = nullptr;
+      return WCN_ERR_LAUNCH;
+    }
+  }
+  if (!done || staging_device != device) {  // events belong to the device they were created on
+    if (done) (void)hipEventDestroy(done);
+    if (hipEventCreateWithFlags(&done, hipEventDisableTiming) != hipSuccess) {
+      done = nullptr;
+      return WCN_ERR_LAUNCH;
+    }
+    staging_device = device;
+  }
+  if (hipMemcpyAsync(staging, device_src, bytes, hipMemcpyDeviceToHost, stream) != hipSuccess)
+    return WCN_ERR_LAUNCH;
+  if (hipEventRecord(done, stream) != hipSuccess) return WCN_ERR_LAUNCH;
+  for (;;) {
+    const hipError_t e = hipEventQuery(done);
+    if (e == hipSuccess) break;
+    if (e != hipErrorNotReady) return WCN_ERR_LAUNCH;
+  }
+  memcpy(host_dst, staging, bytes);
+  return WCN_OK;
+}
+
 int wcn_table_status_from_bits(int32_t bits) {
   if (bits & WCN_DEV_RANGE) return WCN_ERR_COORD_RANGE;
   if (bits & WCN_DEV_OVERFLOW) return WCN_ERR_TABLE_OVERFLOW;
@@ -306,10 +342,7 @@ int wcn_table_query(const void* table, int64_t n_keys, int64_t capacity, const i
 int wcn_table_read_status(const void* table, int32_t* host_num_blocks, void* stream) {
   if (!table) return WCN_ERR_INVALID_ARGUMENT;
   WcnTableHeader h;
-  if (hipMemcpyAsync(&h, table, sizeof(h), hipMemcpyDeviceToHost, (hipStream_t)stream) !=
-      hipSuccess)
-    return WCN_ERR_LAUNCH;
-  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return WCN_ERR_LAUNCH;
+  if (wcn_read_small(&h, table, sizeof(h), (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
   if (host_num_blocks) *host_num_blocks = h.num_blocks;
   return wcn_table_status_from_bits(h.status);
 }
