@@ -28,6 +28,7 @@ struct KmapGeom {
 struct KmapWorkspace {  // host-computed addresses inside a kmap workspace
   int64_t* result;      // [0..K] offsets, [K+1] = table status bits, [K+2] = occupied slots
   int64_t* row_total;   // [K+1] totals of the rows of `groups`
+  int32_t* ticket;      // arrival counter of the scan's workgroups (zeroed by the probe pass)
   int32_t* groups;      // (K+1, G+1): rows 0..K-1 per-offset hit counts of each 64-row group, row K
                         // all hits of the group; after the scan, exclusive prefix sums
   unsigned long long* hits;  // (G, K): lanes of the group that hit, per offset
@@ -43,6 +44,8 @@ inline size_t kmap_layout(void* base, int64_t num_out, int32_t K, KmapWorkspace*
   off += wcn_align256(sizeof(int64_t) * (size_t)(K + 3));
   if (w) w->row_total = (int64_t*)(p + off);
   off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
+  if (w) w->ticket = (int32_t*)(p + off);
+  off += 256;
   if (w) w->groups = (int32_t*)(p + off);
   off += wcn_align256(sizeof(int32_t) * (size_t)(K + 1) * (size_t)(G + 1));
   if (w) w->hits = (unsigned long long*)(p + off);
@@ -58,9 +61,10 @@ inline int grid_for(int64_t n, int block) {
   return (int)(g < 1 ? 1 : g);
 }
 
-struct KmapProbe {      // what the probe pass leaves for the emit pass
+struct KmapProbe {      // what the probe pass leaves for the scan and the emit pass
   unsigned long long* hits;
   int32_t* found;
+  int32_t* ticket;      // set to zero
 };
 
 // ---- generic kernel: any kernel size up to WCN_MAX_OFFSETS offsets -----------------------------
@@ -75,6 +79,7 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
                                                  int32_t* __restrict__ groups, int64_t G,
                                                  KmapProbe o) {
   const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (m == 0) *o.ticket = 0;
   const int64_t group = m >> 6;  // wave-uniform
   if (group >= G) return;
   const int lane = wcn_lane();
@@ -141,6 +146,7 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
   __shared__ int32_t s_base[8][256];
   const int tid = threadIdx.x;
   const int64_t m = (int64_t)blockIdx.x * blockDim.x + tid;
+  if (m == 0) *o.ticket = 0;
   const int64_t group = m >> 6;  // wave-uniform
   if (group >= G) return;
   const int lane = wcn_lane();
@@ -307,8 +313,18 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
 
 // In-place exclusive prefix sum of each row of `groups` (one workgroup per row, G+1 entries; the
 // last entry receives the row total).
+__global__ void kmap_zero_ticket(int32_t* ticket) { *ticket = 0; }
+
+struct KmapFinish {  // null `result`: no finishing step
+  int64_t* result;              // [0..K] offsets, [K+1] table status bits, [K+2] occupied slots
+  int32_t* ticket;              // zero before the launch; left at zero
+  const WcnTableHeader* hdr;
+  int32_t K;
+};
+
 __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ groups, int64_t G,
-                                                       int64_t* __restrict__ row_total) {
+                                                       int64_t* __restrict__ row_total,
+                                                       KmapFinish fin) {
   __shared__ int s_wave[16];
   int32_t* row = groups + (int64_t)blockIdx.x * (G + 1);
   const int lane = wcn_lane(), wave = threadIdx.x >> 6;
@@ -346,22 +362,24 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
     // exceed int32, which the host turns into WCN_ERR_TOO_MANY_PAIRS
     row[G] = (int32_t)carry;
     row_total[blockIdx.x] = carry;
+    if (fin.result) {
+      // the workgroup that finishes last turns the row totals into offsets[K+1] and copies the
+      // table's status next to them, so the host needs one read for everything
+      __threadfence();
+      if (atomicAdd(fin.ticket, 1) == (int32_t)gridDim.x - 1) {
+        __threadfence();
+        int64_t run = 0;
+        fin.result[0] = 0;
+        for (int k = 0; k < fin.K; ++k) {
+          run += __hip_atomic_load(&row_total[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          fin.result[k + 1] = run;
+        }
+        fin.result[fin.K + 1] = fin.hdr->status;
+        fin.result[fin.K + 2] = fin.hdr->num_blocks;
+        *fin.ticket = 0;
+      }
+    }
   }
-}
-
-// offsets[K+1] = exclusive prefix sum of the row totals; also copies the table's status out so
-// the host needs one read for everything.  Serial over K <= 1024 (tiny).
-__global__ void kmap_finish(int64_t* __restrict__ result, const int64_t* __restrict__ row_total,
-                            int32_t K, const WcnTableHeader* __restrict__ hdr) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  int64_t run = 0;
-  result[0] = 0;
-  for (int k = 0; k < K; ++k) {
-    run += row_total[k];
-    result[k + 1] = run;
-  }
-  result[K + 1] = hdr->status;
-  result[K + 2] = hdr->num_blocks;
 }
 
 bool make_geom(const int32_t ks[3], const int32_t st[3], KmapGeom* g) {
@@ -391,7 +409,7 @@ void launch_probe(const WcnTableView& v, const int32_t* out_coords, int64_t num_
                   const KmapGeom& g, const KmapWorkspace& w, hipStream_t s) {
   const dim3 grid(grid_for(num_out, 256)), block(256);
   const uint32_t cap_mask = (uint32_t)(v.capacity - 1);
-  const KmapProbe o = {w.hits, w.found};
+  const KmapProbe o = {w.hits, w.found, w.ticket};
   if (is_fixed_size(g, 3, 3, 3)) {
     hipLaunchKernelGGL((kmap_pass_fixed<3, 3, 3>), grid, block, 0, s, v.hdr, v.slots, cap_mask,
                        v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G, o);
@@ -510,7 +528,8 @@ __global__ void stride_finish(int64_t* __restrict__ result, const int32_t* __res
 
 // Row-wise exclusive scan, shared with the contraction's map conversion.
 void wcn_scan_rows_launch(int32_t* groups, int64_t G, int rows, int64_t* row_total, hipStream_t s) {
-  hipLaunchKernelGGL(kmap_scan_rows, dim3(rows), dim3(1024), 0, s, groups, G, row_total);
+  const KmapFinish none = {nullptr, nullptr, nullptr, 0};
+  hipLaunchKernelGGL(kmap_scan_rows, dim3(rows), dim3(1024), 0, s, groups, G, row_total, none);
 }
 
 extern "C" {
@@ -533,9 +552,13 @@ int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const in
   wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
   KmapWorkspace w;
   kmap_layout(workspace, num_out, g.K, &w);
-  if (w.G > 0) launch_probe(v, out_coords, num_out, g, w, s);
-  hipLaunchKernelGGL(kmap_scan_rows, dim3(g.K + 1), dim3(1024), 0, s, w.groups, w.G, w.row_total);
-  hipLaunchKernelGGL(kmap_finish, dim3(1), dim3(64), 0, s, w.result, w.row_total, g.K, v.hdr);
+  if (w.G > 0) {
+    launch_probe(v, out_coords, num_out, g, w, s);
+  } else {
+    hipLaunchKernelGGL(kmap_zero_ticket, dim3(1), dim3(1), 0, s, w.ticket);
+  }
+  const KmapFinish fin = {w.result, w.ticket, v.hdr, g.K};
+  hipLaunchKernelGGL(kmap_scan_rows, dim3(g.K + 1), dim3(1024), 0, s, w.groups, w.G, w.row_total, fin);
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }
@@ -611,7 +634,10 @@ int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_strid
                        (const int4*)w.coarse, n, v.hdr, v.slots, v.slot_of, v.perm, w.groups, w.G,
                        (int4*)nullptr, (int32_t*)nullptr);
   }
-  hipLaunchKernelGGL(kmap_scan_rows, dim3(1), dim3(1024), 0, s, w.groups, w.G, w.result + 2);
+  {
+    const KmapFinish none = {nullptr, nullptr, nullptr, 0};
+    hipLaunchKernelGGL(kmap_scan_rows, dim3(1), dim3(1024), 0, s, w.groups, w.G, w.result + 2, none);
+  }
   hipLaunchKernelGGL(stride_finish, dim3(1), dim3(64), 0, s, w.result, w.groups, w.G, v.hdr);
   if (n > 0) {
     hipLaunchKernelGGL(stride_pick<true>, dim3(grid_for(n, 256)), dim3(256), 0, s,
