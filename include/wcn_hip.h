@@ -81,10 +81,12 @@ int wcn_table_read_status(const void* table, int32_t* host_num_blocks, void* str
  * Kernel map.  Replaces generate_kernel_map's device work (torch_discrete.py:244-337,80-157;
  * discrete_kernels.cu:264-334,183-213) with two calls and one host read in between:
  *
- *   wcn_kmap_count  -> per-offset pair counts, their prefix sums (device)
+ *   wcn_kmap_count  -> probes the table once; per-offset pair counts, their prefix sums and the
+ *                      found rows stay in the workspace (device)
  *   wcn_kmap_read_result (waits; host learns offsets[K+1], allocates in_maps/out_maps of L)
  *   wcn_kmap_fill   -> in_maps[L], out_maps[L] in the reference's order: offsets concatenated
  *                      in k order (k = (i*ky + j)*kz + kk), pairs ascending in output index.
+ *                      Reads only the workspace wcn_kmap_count filled for the same arguments.
  *
  * Query coordinate of output m and offset k: out[m] * [1, sx, sy, sz] + (0, i-cx, j-cy, kk-cz)
  * with c = size/2 for odd sizes and 0 for even ones (discrete_kernels.cu:291-314).
