@@ -462,13 +462,14 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
 // ---- ring kernel: input rows, weight tiles and pairs go from memory straight into LDS ------------
 //
 // Used when feature rows are whole 16-byte vectors.  The offsets of a tile are cut into steps of
-// at most 64 pairs of one offset.  A workgroup has eight waves:
-//   waves 0..3  multiply: each owns 64 output rows of the tile and their accumulators; per step it
-//               reads its operands from LDS and issues the MFMAs, nothing else
-//   waves 4..7  request: each a quarter of W[k]^T of step r + DW (weight ring, 4 tiles) and a
-//               quarter of the input rows of step r + DG (row ring, 5 x 64 rows); wave 4 also the
-//               input rows and wave 5 the output rows of the pairs of step r + DP (pair ring, 8
-//               slots); wave 6 writes the slot table of step r + DG, wave 7 clears the next one
+// at most 64 pairs of one offset.  A workgroup has eight waves in two roles; NC of them multiply,
+// 8 - NC request (NC = 6 by default: tiles of 384 rows; NC = 4 gives 256-row tiles):
+//   multiplying waves  each owns 64 output rows of the tile and their accumulators; per step it
+//                      reads its operands from LDS and issues the MFMAs, nothing else
+//   requesting waves   each an equal share of W[k]^T of step r + DW (weight ring, 4 tiles) and of
+//                      the input rows of step r + DG (row ring, 5 x 64 rows); the first two also
+//                      the in_maps / out_maps entries of step r + DP (pair ring); the last but
+//                      one writes the slot table of step r + DG, the last clears the next one
 // The requests are global_load_lds: the data goes from memory into LDS without passing through
 // registers.  A wave issues at most one instruction every four cycles, so the bookkeeping of the
 // requests would otherwise sit between the MFMAs of every wave; here it runs beside them.
@@ -482,25 +483,44 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
 // back to the requesting waves.  A slot table per step (one byte per output row: the row's
 // position in the step's slot, or none) is written when the rows are requested and read when
 // the step is multiplied.
+#ifndef WCN_RING_NC
+#define WCN_RING_NC 6
+#endif
 constexpr int RING_THREADS = 512;
 constexpr int STEP_ROWS = 64;
-constexpr int A_SLOTS = 5, W_SLOTS = 4, P_SLOTS = 8, T_SLOTS = 8;
+constexpr int A_SLOTS = 5, W_SLOTS = 4;
 constexpr int DG = A_SLOTS - 1, DW = W_SLOTS - 1, DP = 2 * DG;
-constexpr int MAX_STEPS = 32 * (ROWS / STEP_ROWS);
 constexpr int SLOT_BYTES = STEP_ROWS * 128;   // a row of the rings is 128 bytes for every dtype
 static_assert(TN * 128 == SLOT_BYTES, "weight tile and row slot have the same size");
-static_assert(DP < P_SLOTS + DG && DG == DW + 1 && T_SLOTS > DG + 1, "ring reuse distances");
-static_assert(DG * 5 < 64, "outstanding loads per wave fit the 6-bit vmcnt");
-constexpr int RING_OFF = 0;
-constexpr int WRING_OFF = RING_OFF + A_SLOTS * SLOT_BYTES;
-constexpr int PIN_OFF = WRING_OFF + W_SLOTS * SLOT_BYTES;
-constexpr int POUT_OFF = PIN_OFF + P_SLOTS * STEP_ROWS * 4;
-constexpr int TAB_OFF = POUT_OFF + P_SLOTS * STEP_ROWS * 4;
-constexpr int ZERO_OFF = TAB_OFF + T_SLOTS * ROWS;
-constexpr int STEP_OFF = ZERO_OFF + 128;  // after the row of zeros
-constexpr int MISC_OFF = STEP_OFF + (MAX_STEPS + 2 * DP) * 8;  // DP empty steps before and after the plan
-constexpr int RING_LDS_BYTES = (MISC_OFF + 16 + 511) / 512 * 512;
-static_assert(2 * RING_LDS_BYTES <= 160 * 1024, "two workgroups per CU");
+static_assert(DG == DW + 1, "rows and weights share the requesting waves");
+
+// Layout for NC multiplying waves (tile of 64 NC rows) and 8 - NC requesting waves.
+template <int NC>
+struct RingCfg {
+  static constexpr int RROWS = 64 * NC;
+  static constexpr int NP = 8 - NC;
+  static constexpr int PER = 8 / NP;                 // row loads and weight loads per requesting wave and step
+  static constexpr int P_SLOTS = NC == 4 ? 8 : 6;    // pair ring
+  static constexpr int T_SLOTS = NC == 4 ? 8 : 6;    // slot tables
+  static constexpr int MAX_STEPS = 32 * NC;
+  static constexpr int RING_OFF = 0;
+  static constexpr int WRING_OFF = RING_OFF + A_SLOTS * SLOT_BYTES;
+  static constexpr int PIN_OFF = WRING_OFF + W_SLOTS * SLOT_BYTES;
+  static constexpr int POUT_OFF = PIN_OFF + P_SLOTS * STEP_ROWS * 4;
+  static constexpr int TAB_OFF = POUT_OFF + P_SLOTS * STEP_ROWS * 4;
+  static constexpr int ZERO_OFF = TAB_OFF + T_SLOTS * RROWS;
+  static constexpr int STEP_OFF = ZERO_OFF + 128;  // after the row of zeros
+  static constexpr int MISC_OFF = STEP_OFF + (MAX_STEPS + 2 * DP) * 8;  // DP empty steps before and after the plan
+  static constexpr int LDS_BYTES = (MISC_OFF + 16 + 511) / 512 * 512;
+  static_assert(NP == 4 || NP == 2, "8 loads per step split evenly");
+  static_assert(DP < P_SLOTS + DG && T_SLOTS > DG + 1, "ring reuse distances");
+  static_assert(DG * (2 * PER + 1) < 64, "outstanding loads per wave fit the 6-bit vmcnt");
+  static_assert(2 * LDS_BYTES <= 160 * 1024, "two workgroups per CU");
+  static_assert(A_SLOTS * SLOT_BYTES + W_SLOTS * SLOT_BYTES >= RROWS * 128, "the rings hold a staged output tile");
+  // position in a ring of P_SLOTS / T_SLOTS entries (x >= -48)
+  static __device__ __forceinline__ int pslot(int x) { return (int)((uint32_t)(x + 48) % (uint32_t)P_SLOTS); }
+  static __device__ __forceinline__ int tslot(int x) { return (int)((uint32_t)(x + 48) % (uint32_t)T_SLOTS); }
+};
 
 // global_load_lds_*: lane l of the wave copies 16 (4) bytes from its own global address to LDS
 // byte offset `lds_off` + 16 (4) * l; the data never passes through registers and the load is
@@ -535,41 +555,43 @@ __device__ __forceinline__ int step_num(uint32_t w0) { return (int)((w0 >> 8) & 
 __device__ __forceinline__ int step_first(uint32_t w0) { return (int)((w0 >> 16) & 0x1FFu); }
 __device__ __forceinline__ bool step_identity(uint32_t w0) { return (w0 >> 31) != 0u; }
 
-template <typename T>
+template <typename T, int NC>
 __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
   typedef Mma<T> M;
   typedef typename M::V V;
+  typedef RingCfg<NC> C;
   constexpr int CK = M::CK, KS = M::KS;
   constexpr int VEC = 16 / sizeof(T);
   constexpr int NB = TN / 16;
+  constexpr int RROWS = C::RROWS, NP = C::NP, PER = C::PER;
   static_assert(CK * sizeof(T) == 128, "ring rows are 128 bytes");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint8_t* const ring = smem + RING_OFF;
-  uint8_t* const wring = smem + WRING_OFF;
-  int32_t* const s_pin = (int32_t*)(smem + PIN_OFF);
-  int32_t* const s_pout = (int32_t*)(smem + POUT_OFF);
-  uint8_t* const s_tab = smem + TAB_OFF;
-  const T* const s_zero = (const T*)(smem + ZERO_OFF);
-  uint2* const s_step = (uint2*)(smem + STEP_OFF);
-  int32_t* const s_nsteps = (int32_t*)(smem + MISC_OFF);
+  uint8_t* const ring = smem + C::RING_OFF;
+  uint8_t* const wring = smem + C::WRING_OFF;
+  int32_t* const s_pin = (int32_t*)(smem + C::PIN_OFF);
+  int32_t* const s_pout = (int32_t*)(smem + C::POUT_OFF);
+  uint8_t* const s_tab = smem + C::TAB_OFF;
+  const T* const s_zero = (const T*)(smem + C::ZERO_OFF);
+  uint2* const s_step = (uint2*)(smem + C::STEP_OFF);
+  int32_t* const s_nsteps = (int32_t*)(smem + C::MISC_OFF);
 
   const T* __restrict__ X = (const T*)a.X;
   const T* __restrict__ Wt = (const T*)a.Wt;
   const uint8_t* const zsrc = (const uint8_t*)a.zeros;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wrow = (wave & 3) * 64;  // multiplying waves: first row in the tile
-  const int64_t m0 = (int64_t)blockIdx.x * ROWS;
+  const int wrow = (wave < NC ? wave : 0) * 64;  // multiplying waves: first row in the tile
+  const int64_t m0 = (int64_t)blockIdx.x * RROWS;
   const int n0 = blockIdx.y * TN;
-  const int tile_rows = (int)(a.num_out - m0 < ROWS ? a.num_out - m0 : ROWS);
+  const int tile_rows = (int)(a.num_out - m0 < RROWS ? a.num_out - m0 : RROWS);
   const int64_t g0 = m0 >> 6;
-  const int64_t g1 = g0 + ROWS / 64 < a.G ? g0 + ROWS / 64 : a.G;
+  const int64_t g1 = g0 + RROWS / 64 < a.G ? g0 + RROWS / 64 : a.G;
   const int kgrp = lane >> 4;
   const int sub = lane >> 3, lpart = lane & 7;  // row inside an 8-row load, 16-byte part in LDS
 
-  if (tid < 32) ((uint32_t*)(smem + ZERO_OFF))[tid] = 0u;
+  if (tid < 32) ((uint32_t*)(smem + C::ZERO_OFF))[tid] = 0u;
   T* __restrict__ out = (T*)a.out;
-  T* const stage = (T*)ring;  // output tile staged for 16-byte stores: 256 rows x 128 bytes
+  T* const stage = (T*)ring;  // output tile staged for 16-byte stores: RROWS x 128 bytes (the rings are contiguous)
   const bool staged = sizeof(T) == 2 && a.vec_out;
 
   // Start of a chunk (up to 32 offsets of one slice of input channels): the step plan and clean
@@ -594,7 +616,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
           const int32_t* gs = a.group_start + (int64_t)k * (a.G + 1);
           start = (int32_t)(a.offsets[k] + gs[g0]);
           cnt = gs[g1] - gs[g0];
-          if (cnt < 0 || cnt > ROWS) cnt = 0;  // inconsistent table: contribute nothing
+          if (cnt < 0 || cnt > RROWS) cnt = 0;  // inconsistent table: contribute nothing
         }
       }
       const int ns = (cnt + STEP_ROWS - 1) / STEP_ROWS;
@@ -610,7 +632,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
       if (lane < DP) s_step[lane] = s_step[DP + total + lane] = make_uint2(0u, 0u);
       if (lane == 63) *s_nsteps = total;
     }
-    for (int i = tid; i < T_SLOTS * ROWS / 4; i += RING_THREADS) ((uint32_t*)s_tab)[i] = 0xFFFFFFFFu;
+    for (int i = tid; i < C::T_SLOTS * RROWS / 4; i += RING_THREADS) ((uint32_t*)s_tab)[i] = 0xFFFFFFFFu;
     __syncthreads();
     return *s_nsteps;
   };
@@ -627,7 +649,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
 
   // The two kinds of waves run separate code from here on (the accumulators exist only in the
   // multiplying waves); both pass the same sequence of barriers.
-  if (wave < 4) {
+  if (wave < NC) {
     f32x4 acc[4][NB];
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
@@ -648,7 +670,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
           rR = step_raw(r + 1, S);
           const uint32_t sw_cur = sw;
-          sw = *(const uint32_t*)(s_tab + ((r + 1) & (T_SLOTS - 1)) * ROWS + wrow + (lane & 15) * 4);
+          sw = *(const uint32_t*)(s_tab + C::tslot(r + 1) * RROWS + wrow + (lane & 15) * 4);
           if (r >= 0 && step_num(dR.x) > 0) {
             const T* const abase = (const T*)(ring + im * SLOT_BYTES);
             const T* const bbase = (const T*)(wring + imw * SLOT_BYTES);
@@ -738,15 +760,15 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
         const int S = begin_chunk(kbase);
         if (S == 0) continue;
         // ================= requesting waves =================
-        const int q = wave - 4;  // which quarter of the weight tile and of the step's rows
+        const int q = wave - NC;  // which share of the weight tile and of the step's rows
         const size_t w_tile_bytes = (size_t)a.c_out_pad * a.c_in_pad * sizeof(T);
         const uint8_t* const wbase0 = (const uint8_t*)(Wt + (size_t)n0 * a.c_in_pad + c0);
         const uint8_t* const xbase0 = a.num_in > 0 ? (const uint8_t*)(X + c0) : zsrc;
         const uint32_t row_bytes = (uint32_t)a.c_in * (uint32_t)sizeof(T);
-        uint32_t w_lane_off[2], x_lane_off[2];
+        uint32_t w_lane_off[PER], x_lane_off[PER];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int n = (q * 2 + j) * 8 + sub;  // also the row inside the step's slot
+        for (int j = 0; j < PER; ++j) {
+          const int n = (q * PER + j) * 8 + sub;  // also the row inside the step's slot
           const uint32_t part_off = (uint32_t)(lpart ^ ((n >> 1) & 7)) * 16u;  // source part kept at this LDS position
           w_lane_off[j] = (uint32_t)n * (uint32_t)a.c_in_pad * (uint32_t)sizeof(T) + part_off;
           x_lane_off[j] = part_off;
@@ -760,19 +782,19 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
           // this wave's share of what step r needs, and of the pairs of step r + DG, has landed:
           // everything but the rows and pairs requested DW iterations ago and all that came later
           if (q < 2) {
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 + 5 * (DW - 1)) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PER + 1) + (2 * PER + 1) * (DW - 1)) : "memory");
           } else {
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 + 4 * (DW - 1)) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER + 2 * PER * (DW - 1)) : "memory");
           }
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
           const int gi = r + DG;
-          const int32_t* pin = s_pin + (gi & (P_SLOTS - 1)) * STEP_ROWS;
-          const int32_t* pout = s_pout + (gi & (P_SLOTS - 1)) * STEP_ROWS;
+          const int32_t* pin = s_pin + C::pslot(gi) * STEP_ROWS;
+          const int32_t* pout = s_pout + C::pslot(gi) * STEP_ROWS;
           // all LDS reads first and unconditionally (slots past the step's pairs hold stale
           // values that are not used)
-          int32_t pv[2];
+          int32_t pv[PER];
 #pragma unroll
-          for (int j = 0; j < 2; ++j) pv[j] = pin[(q * 2 + j) * 8 + sub];
+          for (int j = 0; j < PER; ++j) pv[j] = pin[(q * PER + j) * 8 + sub];
           const int32_t pin_l = pin[lane], pout_l = pout[lane];
           rW = step_raw(r + 1 + DW, S);
           rG = step_raw(r + 1 + DG, S);
@@ -781,30 +803,30 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
           const bool identG = step_identity(dG.x);
           const int firstG = step_first(dG.x);
           const int kW = kbase + step_k(dW.x);
-          const uint32_t wdst = lds_offset(wring + iw * SLOT_BYTES + q * 2 * 1024);
-          const uint32_t xdst = lds_offset(ring + ia * SLOT_BYTES + q * 2 * 1024);
+          const uint32_t wdst = lds_offset(wring + iw * SLOT_BYTES + q * PER * 1024);
+          const uint32_t xdst = lds_offset(ring + ia * SLOT_BYTES + q * PER * 1024);
           // weights: uniform base of the tile, this lane's fixed offset inside it
           const uint8_t* const wk = wbase0 + (size_t)kW * w_tile_bytes;
 #pragma unroll
-          for (int j = 0; j < 2; ++j) load_to_lds_16(wk, w_lane_off[j], __builtin_amdgcn_readfirstlane(wdst + j * 1024));
+          for (int j = 0; j < PER; ++j) load_to_lds_16(wk, w_lane_off[j], __builtin_amdgcn_readfirstlane(wdst + j * 1024));
           if (a.flat_in) {
             // rows: uniform base, row index times row size plus this lane's part (rows past the
             // step's pairs and malformed indices fetch row 0; no slot entry ever points at them)
-            uint32_t xoff[2];
+            uint32_t xoff[PER];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const int row = (q * 2 + j) * 8 + sub;
+            for (int j = 0; j < PER; ++j) {
+              const int row = (q * PER + j) * 8 + sub;
               uint32_t in = identG ? (uint32_t)(m0 + firstG + row) : (uint32_t)pv[j];
               if (row >= numG || in >= (uint32_t)a.num_in) in = 0u;
               xoff[j] = in * row_bytes + x_lane_off[j];
             }
 #pragma unroll
-            for (int j = 0; j < 2; ++j) load_to_lds_16(xbase0, xoff[j], __builtin_amdgcn_readfirstlane(xdst + j * 1024));
+            for (int j = 0; j < PER; ++j) load_to_lds_16(xbase0, xoff[j], __builtin_amdgcn_readfirstlane(xdst + j * 1024));
           } else {
-            const uint8_t* xsrc[2];
+            const uint8_t* xsrc[PER];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const int row = (q * 2 + j) * 8 + sub;
+            for (int j = 0; j < PER; ++j) {
+              const int row = (q * PER + j) * 8 + sub;
               int32_t in = identG ? (int32_t)(m0 + firstG + row) : pv[j];
               if (row >= numG) in = -1;
               const int ps = lpart ^ ((row >> 1) & 7);  // source part kept at this LDS position
@@ -814,7 +836,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
               xsrc[j] = ok ? real : zsrc + lane * 16;
             }
 #pragma unroll
-            for (int j = 0; j < 2; ++j) load_to_lds_16(xsrc[j], __builtin_amdgcn_readfirstlane(xdst + j * 1024));
+            for (int j = 0; j < PER; ++j) load_to_lds_16(xsrc[j], __builtin_amdgcn_readfirstlane(xdst + j * 1024));
           }
           if (q < 2) {  // pairs of step r + DP: wave 4 the input rows, wave 5 the output rows
             const int numP = step_identity(dP.x) ? 0 : step_num(dP.x);
@@ -823,16 +845,18 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
             const uint8_t* pbase = numP > 0 ? (const uint8_t*)(list + (int64_t)dP.y) : zsrc;
             const uint32_t poff = (uint32_t)(numP > 0 ? (lane < numP ? lane : numP - 1) : lane) * 4u;
             const uint32_t pdst = lds_offset(q == 0 ? s_pin : s_pout) +
-                                  (uint32_t)(((r + DP) & (P_SLOTS - 1)) * STEP_ROWS * 4);
+                                  (uint32_t)(C::pslot(r + DP) * STEP_ROWS * 4);
             load_to_lds_4(pbase, poff, __builtin_amdgcn_readfirstlane(pdst));
-          } else if (q == 2) {  // slot table of step r + DG
+          }
+          if (q == NP - 2) {  // slot table of step r + DG
             int32_t pub_in = identG ? (int32_t)(m0 + firstG + lane) : pin_l;
             const int pub_out = identG ? firstG + lane : (int)(pout_l - m0);
             if (lane >= numG) pub_in = -1;
             if ((uint32_t)pub_in < (uint64_t)a.num_in && (uint32_t)pub_out < (uint32_t)tile_rows)
-              s_tab[(gi & (T_SLOTS - 1)) * ROWS + (pub_out & ~63) + (pub_out & 15) * 4 + ((pub_out >> 4) & 3)] = (uint8_t)lane;
-          } else {  // the slot table after it starts empty
-            ((uint32_t*)(s_tab + ((gi + 1) & (T_SLOTS - 1)) * ROWS))[lane] = 0xFFFFFFFFu;
+              s_tab[C::tslot(gi) * RROWS + (pub_out & ~63) + (pub_out & 15) * 4 + ((pub_out >> 4) & 3)] = (uint8_t)lane;
+          } else if (q == NP - 1) {  // the slot table after it starts empty
+            for (int i = lane; i < RROWS / 4; i += 64)
+              ((uint32_t*)(s_tab + C::tslot(gi + 1) * RROWS))[i] = 0xFFFFFFFFu;
           }
           iw = iw + 1 == W_SLOTS ? 0 : iw + 1;
           ia = ia + 1 == A_SLOTS ? 0 : ia + 1;
@@ -844,7 +868,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
   }
   if (staged) {
     __syncthreads();
-    for (int v = tid; v < ROWS * 8; v += RING_THREADS) {
+    for (int v = tid; v < RROWS * 8; v += RING_THREADS) {
       const int r = v >> 3, part = v & 7;
       if (m0 + r < a.num_out && n0 + part * VEC < a.c_out)
         *reinterpret_cast<u32x4*>(out + (m0 + r) * a.c_out + n0 + part * VEC) =
@@ -1054,21 +1078,23 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
                        (T*)a.Wt, (uint32_t*)a.zeros);
   }
   const dim3 grid((unsigned)((a.num_out + ROWS - 1) / ROWS), (unsigned)(a.c_out_pad / TN));
+  constexpr int NC = WCN_RING_NC;  // multiplying waves per workgroup of the ring kernel
   if (a.vec_in) {
     // more than 64 KiB of dynamic LDS has to be allowed once per device
     static thread_local int allowed_device = -1;
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) return WCN_ERR_LAUNCH;
     if (allowed_device != device) {
-      if (hipFuncSetAttribute((const void*)conv_fwd_ring<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              RING_LDS_BYTES) != hipSuccess)
+      if (hipFuncSetAttribute((const void*)conv_fwd_ring<T, NC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              RingCfg<NC>::LDS_BYTES) != hipSuccess)
         return WCN_ERR_LAUNCH;
       allowed_device = device;
     }
   }
   if (g_time_start) (void)hipEventRecord(g_time_start, s);
   if (a.vec_in) {
-    hipLaunchKernelGGL(conv_fwd_ring<T>, grid, dim3(RING_THREADS), RING_LDS_BYTES, s, a);
+    const dim3 rgrid((unsigned)((a.num_out + RingCfg<NC>::RROWS - 1) / RingCfg<NC>::RROWS), grid.y);
+    hipLaunchKernelGGL((conv_fwd_ring<T, NC>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
   } else {
     hipLaunchKernelGGL(conv_fwd<T>, grid, dim3(THREADS), 0, s, a);
   }
