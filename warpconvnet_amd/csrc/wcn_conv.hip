@@ -464,8 +464,9 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
 // Used when feature rows are whole 16-byte vectors.  The offsets of a tile are cut into steps of
 // at most 64 pairs of one offset.  A workgroup has eight waves in two roles; NC of them multiply,
 // 8 - NC request (NC = 6 by default: tiles of 384 rows; NC = 4 gives 256-row tiles):
-//   multiplying waves  each owns 64 output rows of the tile and their accumulators; per step it
-//                      reads its operands from LDS and issues the MFMAs, nothing else
+//   multiplying waves  each owns four 16-row blocks of the tile (dealt in turn) and their
+//                      accumulators; per step it reads its operands from LDS and issues the
+//                      MFMAs, nothing else
 //   requesting waves   each an equal share of W[k]^T of step r + DW (weight ring, 4 tiles) and of
 //                      the input rows of step r + DG (row ring, 5 x 64 rows); the first two also
 //                      the in_maps / out_maps entries of step r + DP (pair ring); the last but
@@ -520,6 +521,14 @@ struct RingCfg {
   // position in a ring of P_SLOTS / T_SLOTS entries (x >= -48)
   static __device__ __forceinline__ int pslot(int x) { return (int)((uint32_t)(x + 48) % (uint32_t)P_SLOTS); }
   static __device__ __forceinline__ int tslot(int x) { return (int)((uint32_t)(x + 48) % (uint32_t)T_SLOTS); }
+  // The 16-row blocks of a tile are dealt to the multiplying waves in turn (block b belongs to
+  // wave b % NC as its block b / NC), so that the pairs of a step, which cover a contiguous range
+  // of output rows, spread over all of them.  Byte of tile row t in a slot table: the four blocks
+  // of a wave's row (t & 15) are adjacent.
+  static __device__ __forceinline__ int tab_index(int t) {
+    const uint32_t b = (uint32_t)t >> 4, rb = b / (uint32_t)NC, w = b - rb * (uint32_t)NC;
+    return (int)(w * 64u + ((uint32_t)t & 15u) * 4u + rb);
+  }
 };
 
 // global_load_lds_*: lane l of the wave copies 16 (4) bytes from its own global address to LDS
@@ -580,7 +589,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
   const uint8_t* const zsrc = (const uint8_t*)a.zeros;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wrow = (wave < NC ? wave : 0) * 64;  // multiplying waves: first row in the tile
+  const int wrow = (wave < NC ? wave : 0) * 64;  // multiplying waves: first byte of the wave's entries in a slot table
   const int64_t m0 = (int64_t)blockIdx.x * RROWS;
   const int n0 = blockIdx.y * TN;
   const int tile_rows = (int)(a.num_out - m0 < RROWS ? a.num_out - m0 : RROWS);
@@ -732,7 +741,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
     __syncthreads();  // every wave is done with the rings, every load has landed
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
-      const int lr = wrow + rb * 16 + (lane & 15);
+      const int lr = (rb * NC + wave) * 16 + (lane & 15);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         const int col = nb * 16 + kgrp * 4;
@@ -853,7 +862,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
             const int pub_out = identG ? firstG + lane : (int)(pout_l - m0);
             if (lane >= numG) pub_in = -1;
             if ((uint32_t)pub_in < (uint64_t)a.num_in && (uint32_t)pub_out < (uint32_t)tile_rows)
-              s_tab[C::tslot(gi) * RROWS + (pub_out & ~63) + (pub_out & 15) * 4 + ((pub_out >> 4) & 3)] = (uint8_t)lane;
+              s_tab[C::tslot(gi) * RROWS + C::tab_index(pub_out)] = (uint8_t)lane;
           } else if (q == NP - 1) {  // the slot table after it starts empty
             for (int i = lane; i < RROWS / 4; i += 64)
               ((uint32_t*)(s_tab + C::tslot(gi + 1) * RROWS))[i] = 0xFFFFFFFFu;
