@@ -103,6 +103,13 @@ int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const in
 int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_offsets,
                          int64_t* host_offsets, void* stream);
 
+/* Flags of the table behind the last wcn_kmap_read_result call of this host thread (no device
+ * access).  Bit 0: some key was inserted more than once.  Without duplicates, a stride-1 map of
+ * a coordinate set onto itself with odd kernel sizes is symmetric (the pairs of offset k with in
+ * and out exchanged are the pairs of offset K - 1 - k), which wcn_sparse_conv_dgrad exploits.
+ * No counterpart in the reference. */
+int32_t wcn_kmap_last_table_flags(void);
+
 int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
                   int64_t num_out, const int32_t host_kernel_size[3], const int32_t host_stride[3],
                   const void* workspace, int32_t* in_maps, int32_t* out_maps, void* stream);
@@ -162,6 +169,49 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
                         int32_t identity_offset, int32_t out_maps_ascend,
                         const int32_t* group_start_or_null, void* out, int64_t num_out,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Gradients of the contraction.  Replace the per-offset loops of the reference backward
+ * (sparse_conv.py:314-355 explicit, :418-492 implicit, :547-627 CUTLASS) and the native calls
+ * they make (_C.gemm.cutlass_gemm_AD_gather_scatter with the maps exchanged,
+ * _C.gemm.cutlass_gemm_trAB_gather, _C.gemm.split_k_implicit_gemm):
+ *
+ *   grad_in[n, :]  = sum_k sum_{pairs p of offset k with in_maps[p] == n} grad_out[out_maps[p], :] @ W[k]^T
+ *   grad_weight[k] = sum_{pairs p of offset k} X[in_maps[p], :]^T (x) grad_out[out_maps[p], :]
+ *
+ * fp32 accumulation, one rounding; both results are fully written and bitwise reproducible.
+ * With identity_offset >= 0 that offset is taken over the rows m < min(N, M) with in = out = m and
+ * its pairs in the map are ignored (sparse_conv.py:332-336).
+ *
+ * wcn_sparse_conv_dgrad is the forward contraction over the map with in and out exchanged; its
+ * workspace is wcn_conv_workspace_bytes(num_in, K, c_out, c_in, dtype, num_pairs, ascend) with
+ * ascend = map_is_symmetric || in_maps_ascend.  map_is_symmetric = 1 promises that the pairs of
+ * offset k with in and out exchanged are exactly the pairs of offset K - 1 - k (a stride-1 map
+ * of one coordinate set onto itself): the map is then used as it stands, group_start included.
+ * Otherwise in_maps_ascend says whether in_maps ascends inside every offset (true for the map of
+ * a transposed convolution, which is a forward map with its lists exchanged); if not the pairs
+ * are re-ordered inside the workspace.  `weight` is the forward weight (K, c_in, c_out).
+ * ------------------------------------------------------------------------------------------- */
+
+int wcn_sparse_conv_dgrad(const void* grad_out, int64_t num_out, int32_t c_out, int32_t dtype,
+                          const void* weight, int32_t weight_dtype, int32_t num_offsets,
+                          int32_t c_in, const int32_t* in_maps, const int32_t* out_maps,
+                          const int64_t* host_offsets, int32_t identity_offset,
+                          int32_t map_is_symmetric, int32_t in_maps_ascend,
+                          const int32_t* group_start_or_null, void* grad_in, int64_t num_in,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/* identity_rows = min(N, M) if identity_offset >= 0, else 0. */
+size_t wcn_conv_wgrad_workspace_bytes(int32_t num_offsets, int32_t c_in, int32_t c_out,
+                                      int64_t num_pairs, int64_t identity_rows);
+
+/* grad_weight is (K, c_in, c_out) in weight_dtype (the feature dtype or fp32). */
+int wcn_sparse_conv_wgrad(const void* features, int64_t num_in, int32_t c_in, const void* grad_out,
+                          int64_t num_out, int32_t c_out, int32_t dtype, const int32_t* in_maps,
+                          const int32_t* out_maps, const int64_t* host_offsets,
+                          int32_t num_offsets, int32_t identity_offset, void* grad_weight,
+                          int32_t weight_dtype, void* workspace, size_t workspace_bytes,
+                          void* stream);
 
 /* Measurement hook (no counterpart in the reference, which times whole calls with CUDA events:
  * warpconvnet/utils/timer.py:41-60).  The two hipEvent_t handles are recorded on the call's

@@ -1,4 +1,4 @@
-"""Torch-CPU restatement of the reference's explicit gather-GEMM-scatter forward.
+"""Torch-CPU restatement of the reference's explicit gather-GEMM-scatter forward and backward.
 
 TEST INFRASTRUCTURE ONLY (parity checker and the benchmark's cpu_baseline leg).
 
@@ -14,6 +14,10 @@ kernel offset) is reproduced by torch itself:
     return out cast back to the dtype X came in with
 
 The bias add and the output container are applied by the caller (sparse_conv.py:1794-1805).
+
+`explicit_gemm_backward` follows sparse_conv.py:314-355 the same way.  It is pinned by torch's
+automatic differentiation of `explicit_gemm_forward` (tests/test_oracle_pins.py), which in turn
+is pinned by the dense-cube conv3d identity and the pairwise brute force.
 """
 from typing import Optional
 
@@ -42,3 +46,37 @@ def explicit_gemm_forward(in_features: torch.Tensor, weight: torch.Tensor, in_ma
         rows_out = out_maps[lo:hi].long()
         out[rows_out] += torch.matmul(x[rows_in], w[k])
     return out.to(dtype=in_features.dtype)
+
+
+def explicit_gemm_backward(grad_output: torch.Tensor, in_features: torch.Tensor,
+                           weight: torch.Tensor, in_maps: torch.Tensor, out_maps: torch.Tensor,
+                           offsets, identity_map_index: Optional[int],
+                           compute_dtype: Optional[torch.dtype] = None):
+    """(grad_in_features, grad_weight):
+        dX = dY @ W[iden]^T, dW[iden] = X^T @ dY     if the map carries an identity index
+        for k != iden, non-empty, in k order:
+            dX[in_map_k] += dY[out_map_k] @ W[k]^T ;  dW[k] += X[in_map_k]^T @ dY[out_map_k]
+    computed in compute_dtype (else the dtype of X), returned in the dtypes of X and W."""
+    dtype = compute_dtype if compute_dtype is not None else in_features.dtype
+    x = in_features.to(dtype)
+    w = weight.to(dtype)
+    gy = grad_output.to(dtype)
+    offs = [int(o) for o in offsets]
+    grad_w = torch.zeros_like(w)
+    if identity_map_index is not None:
+        grad_x = torch.matmul(gy, w[identity_map_index].T)
+        grad_w[identity_map_index] = torch.matmul(x.T, gy)
+    else:
+        grad_x = torch.zeros_like(x)
+    for k in range(len(offs) - 1):
+        if k == identity_map_index:
+            continue
+        lo, hi = offs[k], offs[k + 1]
+        if hi == lo:
+            continue
+        rows_in = in_maps[lo:hi].long()
+        rows_out = out_maps[lo:hi].long()
+        g = gy[rows_out]
+        grad_x[rows_in] += torch.matmul(g, w[k].T)
+        grad_w[k] += torch.matmul(x[rows_in].T, g)
+    return grad_x.to(in_features.dtype), grad_w.to(weight.dtype)

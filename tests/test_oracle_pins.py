@@ -248,3 +248,33 @@ def test_torch_restatement_agrees_with_c_oracle(oracle):
     assert h.dtype == torch.bfloat16
     ref = oracle.explicit_conv_f64(x.to(torch.bfloat16).double().numpy(), w.to(torch.bfloat16).double().numpy(), im, om, off, iden, n)
     assert np.abs(h.double().numpy() - ref).max() / np.abs(ref).max() < 1e-2
+
+
+@pytest.mark.parametrize("case", ["same_coords", "strided", "transposed"])
+def test_backward_restatement_equals_autograd_of_the_forward(oracle, case):
+    """The forward restatement is pinned above (dense-cube conv3d identity, pairwise brute force);
+    torch differentiates it by itself, which pins the hand-written backward formulas (a dropped
+    transpose, exchanged maps or a missed identity branch all fail here)."""
+    from oracle.explicit_conv import explicit_gemm_backward, explicit_gemm_forward
+    coords = synthetic.random_cloud(21, 700, 12, batch_size=2)
+    if case == "same_coords":
+        im, om, off, iden = oracle.kernel_map(coords, coords, (3, 3, 3))
+        n_in = n_out = len(coords)
+    else:
+        coarse = oracle.stride_coords(coords, (2, 2, 2), 2)[0]
+        im, om, off, iden = oracle.kernel_map(coords, coarse, (2, 2, 2), (2, 2, 2))
+        n_in, n_out = len(coords), len(coarse)
+        if case == "transposed":
+            im, om, n_in, n_out = om, im, n_out, n_in
+    K = len(off) - 1
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(n_in, 5, generator=g, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(K, 5, 7, generator=g, dtype=torch.float64, requires_grad=True)
+    gy = torch.randn(n_out, 7, generator=g, dtype=torch.float64)
+    im_t, om_t = torch.as_tensor(im), torch.as_tensor(om)
+    out = explicit_gemm_forward(x, w, im_t, om_t, off, iden, n_out)
+    want_x, want_w = torch.autograd.grad(out, (x, w), gy)
+    got_x, got_w = explicit_gemm_backward(gy, x.detach(), w.detach(), im_t, om_t, off, iden)
+    assert (got_x - want_x).abs().max() < 1e-10
+    assert (got_w - want_w).abs().max() < 1e-10
+    assert want_w.abs().max() > 0 and want_x.abs().max() > 0

@@ -29,6 +29,7 @@ SIGNATURES = {
     "wcn_kmap_read_result": (ctypes.c_int, [_vp, _i64, _i32, _i64p, _vp]),
     "wcn_kmap_fill": (ctypes.c_int, [_vp, _i64, _i64, _vp, _i64, _i32p, _i32p, _vp, _vp, _vp, _vp]),
     "wcn_kmap_group_start": (_vp, [_vp, _i64, _i32]),
+    "wcn_kmap_last_table_flags": (_i32, []),
     "wcn_stride_unique_workspace_bytes": (_sz, [_i64, _i64]),
     "wcn_stride_unique": (ctypes.c_int, [_vp, _i64, _i32p, _vp, _i64, _vp, _vp, _vp]),
     "wcn_stride_unique_read_count": (ctypes.c_int, [_vp, _i64, _i64, _i64p, _vp]),
@@ -36,6 +37,11 @@ SIGNATURES = {
     "wcn_conv_set_timing_events": (ctypes.c_int, [_vp, _vp]),
     "wcn_sparse_conv_fwd": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                            _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
+    "wcn_sparse_conv_dgrad": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
+                                             _i64p, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
+    "wcn_conv_wgrad_workspace_bytes": (_sz, [_i32, _i32, _i32, _i64, _i64]),
+    "wcn_sparse_conv_wgrad": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i32, _i32, _vp, _vp, _i64p,
+                                             _i32, _i32, _vp, _i32, _vp, _sz, _vp]),
 }
 
 _lib = None

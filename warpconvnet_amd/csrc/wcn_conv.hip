@@ -29,15 +29,13 @@
 #include <type_traits>
 
 #include "wcn_common.h"
+#include "wcn_mma.h"
 
 void wcn_scan_rows_launch(int32_t* groups, int64_t G, int rows, int64_t* row_total, hipStream_t s);
 
 namespace {
 
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte piece
+using namespace wcn_mma;
 
 constexpr int ROWS = 256;    // output rows per workgroup
 constexpr int TN = 64;       // output channels per workgroup
@@ -46,63 +44,15 @@ constexpr int NBW = TN / 16 / (THREADS / 256);  // 16-channel blocks per wave
 constexpr int A_ROWS = 128;  // gathered input rows resident in LDS (pairs per batch)
 constexpr int BATCH = 4;     // offsets per batch, at most
 
-__device__ __forceinline__ float to_float(_Float16 v) { return (float)v; }
-__device__ __forceinline__ float to_float(__bf16 v) { return (float)v; }
-__device__ __forceinline__ float to_float(float v) { return v; }
-template <typename T>
-__device__ __forceinline__ T from_float(float v) {
-  return (T)v;
-}
-
-// MFMA operand handling per element type.  16x16x32 (f16/bf16): lane l holds row (l & 15),
-// k = 8 * (l >> 4) .. +7 of A and column (l & 15), same k of B; 16x16x4 (f32): lane l holds
-// A[row l & 15][k = l >> 4], B[k = l >> 4][col l & 15].  The result holds column (l & 15), rows
-// 4 * (l >> 4) .. +3.  Both operands are read from rows of CK contiguous k values.
-template <typename T>
-struct Mma;
-template <>
-struct Mma<_Float16> {
-  typedef f16x8 V;
-  static constexpr int CK = 64, KS = 2;
-  // 8 consecutive k of row `r`: logical part ks * 4 + kgrp, stored at its swizzled position
-  static __device__ __forceinline__ V load(const _Float16* row, int r, int ks, int kgrp) {
-    return *reinterpret_cast<const V*>(row + ((ks * 4 + kgrp) ^ ((r >> 1) & 7)) * 8);
-  }
-  static __device__ __forceinline__ V zero() { return (V){0, 0, 0, 0, 0, 0, 0, 0}; }
-  static __device__ __forceinline__ f32x4 mma(V a, V b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
-  }
-};
-template <>
-struct Mma<__bf16> {
-  typedef bf16x8 V;
-  static constexpr int CK = 64, KS = 2;
-  static __device__ __forceinline__ V load(const __bf16* row, int r, int ks, int kgrp) {
-    return *reinterpret_cast<const V*>(row + ((ks * 4 + kgrp) ^ ((r >> 1) & 7)) * 8);
-  }
-  static __device__ __forceinline__ V zero() { return (V){0, 0, 0, 0, 0, 0, 0, 0}; }
-  static __device__ __forceinline__ f32x4 mma(V a, V b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-  }
-};
-template <>
-struct Mma<float> {
-  typedef float V;
-  static constexpr int CK = 32, KS = 8;
-  // element ks * 4 + kgrp of row `r`: part ks (four floats), swizzled, then the float inside it
-  static __device__ __forceinline__ V load(const float* row, int r, int ks, int kgrp) {
-    return row[(ks ^ ((r >> 1) & 7)) * 4 + kgrp];
-  }
-  static __device__ __forceinline__ V zero() { return 0.f; }
-  static __device__ __forceinline__ f32x4 mma(V a, V b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-  }
-};
-
-// Wt[k][n][c] = W[k][c][n] converted to T, zero padded to (c_out_pad, c_in_pad).
+// The kernels multiply by tiles Wt[k][n][c] (n: channel of the result, c: channel of the gathered
+// rows), converted to T and zero padded to (c_out_pad, c_in_pad).
+//   forward        Wt[k][n][c] = W[k][c][n]            (W is (K, c_in, c_out))
+//   input gradient Wt[k][n][c] = W[k'][n][c], k' = k or K - 1 - k   (W is (K, c_out, c_in) in the
+//                  kernel's terms: the product is dY @ W[k']^T)
 template <typename T, typename WT>
 __global__ void __launch_bounds__(256) conv_prep_weight(const WT* __restrict__ W, int K, int c_in,
                                                         int c_out, int c_in_pad, int c_out_pad,
+                                                        int as_stored, int flip_k,
                                                         T* __restrict__ Wt, uint32_t* __restrict__ zeros) {
   if (blockIdx.x == 0) zeros[threadIdx.x] = 0u;  // 256 threads x 4 bytes
   const int64_t total = (int64_t)K * c_out_pad * c_in_pad;
@@ -111,8 +61,10 @@ __global__ void __launch_bounds__(256) conv_prep_weight(const WT* __restrict__ W
     const int c = (int)(i % c_in_pad);
     const int n = (int)((i / c_in_pad) % c_out_pad);
     const int k = (int)(i / ((int64_t)c_in_pad * c_out_pad));
+    const int ks = flip_k ? K - 1 - k : k;
     float v = 0.f;
-    if (c < c_in && n < c_out) v = to_float(W[((int64_t)k * c_in + c) * c_out + n]);
+    if (c < c_in && n < c_out)
+      v = to_float(as_stored ? W[((int64_t)ks * c_out + n) * c_in + c] : W[((int64_t)ks * c_in + c) * c_out + n]);
     Wt[i] = from_float<T>(v);
   }
 }
@@ -133,11 +85,6 @@ struct ConvArgs {
   int32_t vec_out;  // same for output rows
   int32_t flat_in;  // c_in is a multiple of the staged row and the feature matrix is below 4 GiB
 };
-
-// LDS rows are 128 bytes (eight 16-byte parts) with no padding; part p of row r is stored at
-// part p ^ ((r >> 1) & 7), which makes the 16-byte operand reads of 16 consecutive rows (and of
-// most scattered row sets) hit distinct banks.
-__device__ __forceinline__ int lds_part(int row, int part) { return part ^ ((row >> 1) & 7); }
 
 // One batch = up to BATCH offsets and A_ROWS pairs; the pairs of one offset may be split over
 // consecutive batches.  Packed descriptor of one (batch, offset) entry.
@@ -1074,17 +1021,18 @@ thread_local hipEvent_t g_time_start = nullptr;
 thread_local hipEvent_t g_time_stop = nullptr;
 
 template <typename T>
-int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dtype,
-                hipStream_t s) {
+int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dtype, int as_stored,
+                int flip_k, hipStream_t s) {
   const int64_t total = (int64_t)a.K * a.c_out_pad * a.c_in_pad;
   const int pgrid = (int)std::min<int64_t>(4096, (total + 255) / 256);
   if (weight_dtype == dtype) {
     hipLaunchKernelGGL((conv_prep_weight<T, T>), dim3(pgrid), dim3(256), 0, s, (const T*)weight,
-                       a.K, a.c_in, a.c_out, a.c_in_pad, a.c_out_pad, (T*)a.Wt, (uint32_t*)a.zeros);
+                       a.K, a.c_in, a.c_out, a.c_in_pad, a.c_out_pad, as_stored, flip_k, (T*)a.Wt,
+                       (uint32_t*)a.zeros);
   } else {
     hipLaunchKernelGGL((conv_prep_weight<T, float>), dim3(pgrid), dim3(256), 0, s,
                        (const float*)weight, a.K, a.c_in, a.c_out, a.c_in_pad, a.c_out_pad,
-                       (T*)a.Wt, (uint32_t*)a.zeros);
+                       as_stored, flip_k, (T*)a.Wt, (uint32_t*)a.zeros);
   }
   const dim3 grid((unsigned)((a.num_out + ROWS - 1) / ROWS), (unsigned)(a.c_out_pad / TN));
   constexpr int NC = WCN_RING_NC;  // multiplying waves per workgroup of the ring kernel
@@ -1132,13 +1080,15 @@ size_t wcn_conv_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_
                      out_maps_ascend ? -1 : num_pairs, nullptr);
 }
 
-int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
-                        const void* weight, int32_t weight_dtype, int32_t num_offsets,
-                        int32_t c_out, const void* bias_or_null, const int32_t* in_maps,
-                        const int32_t* out_maps, const int64_t* host_offsets,
-                        int32_t identity_offset, int32_t out_maps_ascend,
-                        const int32_t* group_start_or_null, void* out, int64_t num_out,
-                        void* workspace, size_t workspace_bytes, void* stream) {
+// Shared body of the forward product and the input gradient.  weight_as_stored / flip_offsets
+// choose how the caller's weight becomes the kernels' tiles (see conv_prep_weight).
+static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                    const void* weight, int32_t weight_dtype, int32_t num_offsets, int32_t c_out,
+                    const void* bias_or_null, const int32_t* in_maps, const int32_t* out_maps,
+                    const int64_t* host_offsets, int32_t identity_offset, int32_t out_maps_ascend,
+                    const int32_t* group_start_or_null, void* out, int64_t num_out,
+                    void* workspace, size_t workspace_bytes, int weight_as_stored,
+                    int flip_offsets, void* stream) {
   if (dtype < 0 || dtype > 2 || (weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32))
     return WCN_ERR_INVALID_ARGUMENT;
   if (num_in < 0 || num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || c_in < 1 ||
@@ -1224,10 +1174,48 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
   a.vec_out = (((size_t)c_out * es) % 16 == 0 && ((uintptr_t)out % 16) == 0) ? 1 : 0;
   a.flat_in = (c_in % ck_of(dtype) == 0 && (uint64_t)num_in * c_in * es < (1ull << 32)) ? 1 : 0;
   switch (dtype) {
-    case WCN_DTYPE_F32: return launch_conv<float>(a, weight, weight_dtype, dtype, s);
-    case WCN_DTYPE_F16: return launch_conv<_Float16>(a, weight, weight_dtype, dtype, s);
-    default: return launch_conv<__bf16>(a, weight, weight_dtype, dtype, s);
+    case WCN_DTYPE_F32:
+      return launch_conv<float>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, s);
+    case WCN_DTYPE_F16:
+      return launch_conv<_Float16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, s);
+    default:
+      return launch_conv<__bf16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, s);
   }
+}
+
+int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                        const void* weight, int32_t weight_dtype, int32_t num_offsets,
+                        int32_t c_out, const void* bias_or_null, const int32_t* in_maps,
+                        const int32_t* out_maps, const int64_t* host_offsets,
+                        int32_t identity_offset, int32_t out_maps_ascend,
+                        const int32_t* group_start_or_null, void* out, int64_t num_out,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  return conv_run(features, num_in, c_in, dtype, weight, weight_dtype, num_offsets, c_out,
+                  bias_or_null, in_maps, out_maps, host_offsets, identity_offset, out_maps_ascend,
+                  group_start_or_null, out, num_out, workspace, workspace_bytes, 0, 0, stream);
+}
+
+int wcn_sparse_conv_dgrad(const void* grad_out, int64_t num_out, int32_t c_out, int32_t dtype,
+                          const void* weight, int32_t weight_dtype, int32_t num_offsets,
+                          int32_t c_in, const int32_t* in_maps, const int32_t* out_maps,
+                          const int64_t* host_offsets, int32_t identity_offset,
+                          int32_t map_is_symmetric, int32_t in_maps_ascend,
+                          const int32_t* group_start_or_null, void* grad_in, int64_t num_in,
+                          void* workspace, size_t workspace_bytes, void* stream) {
+  if (map_is_symmetric) {
+    // the pairs of offset k with in and out exchanged are the pairs of offset K - 1 - k: the map
+    // is used as it stands (with its group starts) and the weight tiles are taken in reverse
+    if (num_in != num_out) return WCN_ERR_INVALID_ARGUMENT;
+    return conv_run(grad_out, num_out, c_out, dtype, weight, weight_dtype, num_offsets, c_in,
+                    nullptr, in_maps, out_maps, host_offsets,
+                    identity_offset < 0 ? -1 : num_offsets - 1 - identity_offset, 1,
+                    group_start_or_null, grad_in, num_in, workspace, workspace_bytes, 1, 1, stream);
+  }
+  // in general: the same contraction over the map with in and out exchanged
+  return conv_run(grad_out, num_out, c_out, dtype, weight, weight_dtype, num_offsets, c_in, nullptr,
+                  out_maps, in_maps, host_offsets, identity_offset, in_maps_ascend,
+                  in_maps_ascend ? group_start_or_null : nullptr, grad_in, num_in, workspace,
+                  workspace_bytes, 1, 0, stream);
 }
 
 }  // extern "C"

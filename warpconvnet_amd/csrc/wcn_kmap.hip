@@ -26,7 +26,7 @@ struct KmapGeom {
 };
 
 struct KmapWorkspace {  // host-computed addresses inside a kmap workspace
-  int64_t* result;      // [0..K] offsets, [K+1] = table status bits, [K+2] = occupied slots
+  int64_t* result;      // [0..K] offsets, [K+1] = table status bits, [K+2] = occupied slots | duplicates << 32
   int64_t* row_total;   // [K+1] totals of the rows of `groups`
   int32_t* ticket;      // arrival counter of the scan's workgroups (zeroed by the probe pass)
   int32_t* groups;      // (K+1, G+1): rows 0..K-1 per-offset hit counts of each 64-row group, row K
@@ -316,7 +316,7 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
 __global__ void kmap_zero_ticket(int32_t* ticket) { *ticket = 0; }
 
 struct KmapFinish {  // null `result`: no finishing step
-  int64_t* result;              // [0..K] offsets, [K+1] table status bits, [K+2] occupied slots
+  int64_t* result;              // [0..K] offsets, [K+1] table status bits, [K+2] occupied slots | duplicates << 32
   int32_t* ticket;              // zero before the launch; left at zero
   const WcnTableHeader* hdr;
   int32_t K;
@@ -375,7 +375,7 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
           fin.result[k + 1] = run;
         }
         fin.result[fin.K + 1] = fin.hdr->status;
-        fin.result[fin.K + 2] = fin.hdr->num_blocks;
+        fin.result[fin.K + 2] = (int64_t)fin.hdr->num_blocks | ((int64_t)(fin.hdr->has_duplicates != 0) << 32);
         *fin.ticket = 0;
       }
     }
@@ -532,6 +532,10 @@ void wcn_scan_rows_launch(int32_t* groups, int64_t G, int rows, int64_t* row_tot
   hipLaunchKernelGGL(kmap_scan_rows, dim3(rows), dim3(1024), 0, s, groups, G, row_total, none);
 }
 
+// what the last wcn_kmap_read_result of this host thread learned about the table (bit 0: some
+// key was inserted more than once)
+static thread_local int32_t g_last_table_flags = 0;
+
 extern "C" {
 
 size_t wcn_kmap_workspace_bytes(int64_t num_out, int32_t num_offsets) {
@@ -563,6 +567,8 @@ int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const in
   return WCN_OK;
 }
 
+int32_t wcn_kmap_last_table_flags(void) { return g_last_table_flags; }
+
 int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_offsets,
                          int64_t* host_offsets, void* stream) {
   if (!workspace || !host_offsets || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS)
@@ -573,6 +579,7 @@ int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_off
   const size_t bytes = sizeof(int64_t) * (size_t)(num_offsets + 3);
   if (wcn_read_small(tmp, w.result, bytes, (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
   for (int k = 0; k <= num_offsets; ++k) host_offsets[k] = tmp[k];
+  g_last_table_flags = (int32_t)((tmp[num_offsets + 2] >> 32) & 1);
   const int st = wcn_table_status_from_bits((int32_t)tmp[num_offsets + 1]);
   if (st != WCN_OK) return st;
   if (tmp[num_offsets] > INT32_MAX) return WCN_ERR_TOO_MANY_PAIRS;

@@ -29,6 +29,13 @@ class IntSearchResult:
         # per-64-row group starts.
         self._out_ascend = False
         self._group_start = None
+        # For the gradients: whether in_maps ascends inside every offset (the map of a transposed
+        # convolution: a forward map with its lists exchanged), the group starts that belong to
+        # that order, and whether exchanging in and out turns offset k into offset K - 1 - k
+        # (stride-1 map of a duplicate-free coordinate set onto itself).
+        self._in_ascend = False
+        self._in_group_start = None
+        self._symmetric = False
 
     @torch.no_grad()
     def __getitem__(self, idx: int) -> Tuple[Tensor, Tensor]:

@@ -85,6 +85,7 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     # the workspace (kept alive by the reference below) holds their per-64-row group starts
     result._out_ascend = True
     result._group_start = (ws, L.wcn_kmap_group_start(ptr(ws), M, K), (K, M))
+    result._keys_unique = (L.wcn_kmap_last_table_flags() & 1) == 0
     return result
 
 
@@ -141,6 +142,11 @@ def generate_kernel_map(
     stride = ntuple(in_to_out_stride_ratio, ndim=num_spatial_dims)
     result = _kernel_map_from_table(table, batch_indexed_out_coords, kernel_size, stride,
                                     identity_map_index)
+    same_set = (batch_indexed_in_coords.data_ptr() == batch_indexed_out_coords.data_ptr()
+                and batch_indexed_in_coords.shape == batch_indexed_out_coords.shape
+                and batch_indexed_in_coords.stride() == batch_indexed_out_coords.stride())
+    result._symmetric = bool(same_set and is_odd and all(s == 1 for s in stride)
+                             and getattr(result, "_keys_unique", False))
     if skip_symmetric_kernel_map and is_odd:
         # only the offsets before the centre are kept (torch_discrete.py:286-296)
         half = int(np.prod(kernel_size)) // 2

@@ -8,8 +8,9 @@ sequence for all kernel offsets, fp32 accumulation, one rounding).
 
 There is a single contraction algorithm; the `fwd_algo` / `bwd_algo` / block-size arguments of
 the reference are accepted for call compatibility and do not select anything.  The backward pass
-of the autograd Function is expressed with torch operations over the same kernel map
-(reference: sparse_conv.py:314-355).
+of the autograd Function runs in the same library (`wcn_sparse_conv_dgrad`: the contraction over
+the map with in and out exchanged; `wcn_sparse_conv_wgrad`: per-offset X^T dY over the pairs;
+reference: sparse_conv.py:314-355).
 """
 import ctypes
 import enum
@@ -107,32 +108,72 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
     return out if out.dtype == in_features.dtype else out.to(in_features.dtype)
 
 
-def _explicit_gemm_backward_logic(grad_output: Tensor, in_features: Tensor, weight: Tensor,
-                                  kernel_map: IntSearchResult,
-                                  compute_dtype: Optional[torch.dtype]):
-    """Gradients with torch operations over the kernel map (reference: sparse_conv.py:314-355):
-    dX[in_k] += dY[out_k] @ W[k]^T ;  dW[k] = X[in_k]^T @ dY[out_k]."""
+@torch.no_grad()
+def sparse_conv_backward(grad_output: Tensor, in_features: Tensor, weight: Tensor,
+                         kernel_map: IntSearchResult, compute_dtype: Optional[torch.dtype] = None,
+                         need_input_grad: bool = True, need_weight_grad: bool = True):
+    """Gradients of the contraction on the GPU (replaces the per-offset loops of
+    sparse_conv.py:314-355 / :418-492 / :547-627 and the native GEMMs they call):
+    dX[in_k] += dY[out_k] @ W[k]^T ;  dW[k] = X[in_k]^T @ dY[out_k], fp32 accumulation, one
+    rounding.  Returns (grad_in_features or None, grad_weight or None) in the dtypes of
+    in_features and weight."""
+    require_device(grad_output, "grad_output")
+    require_device(in_features, "in_features")
     dtype = compute_dtype or in_features.dtype
-    x = in_features.to(dtype)
-    w = weight.to(dtype)
-    gy = grad_output.to(dtype)
-    grad_x = torch.zeros_like(x)
-    grad_w = torch.zeros_like(w)
-    iden = kernel_map.identity_map_index
-    if iden is not None:
-        grad_x += gy @ w[iden].T
-        grad_w[iden] = x.T @ gy
-    for k in range(len(kernel_map)):
-        if k == iden:
-            continue
-        in_map, out_map = kernel_map[k]
-        if in_map.numel() == 0:
-            continue
-        in_map, out_map = in_map.long(), out_map.long()
-        g = gy[out_map]
-        grad_x.index_add_(0, in_map, g @ w[k].T)
-        grad_w[k] = x[in_map].T @ g
-    return grad_x.to(in_features.dtype), grad_w.to(weight.dtype)
+    if dtype not in DTYPE_CODE:
+        raise TypeError(f"unsupported feature dtype {dtype}")
+    K, c_in, c_out = weight.shape
+    if len(kernel_map) != K or in_features.shape[1] != c_in or grad_output.shape[1] != c_out:
+        raise ValueError(f"shape mismatch: features {tuple(in_features.shape)}, grad_output "
+                         f"{tuple(grad_output.shape)}, weight {tuple(weight.shape)}, "
+                         f"{len(kernel_map)} offsets")
+    x = in_features.detach().to(dtype).contiguous()
+    gy = grad_output.detach().to(dtype).contiguous()
+    w = weight.detach()
+    if w.dtype != dtype and w.dtype != torch.float32:
+        w = w.to(dtype)
+    w = w.contiguous()
+    km = kernel_map
+    n_in, n_out = x.shape[0], gy.shape[0]
+    device = x.device
+    L = lib()
+    num_pairs = int(km.offsets[-1])
+    host_offsets = (ctypes.c_int64 * (K + 1))(*[int(v) for v in km.offsets.tolist()])
+    iden = -1 if km.identity_map_index is None else int(km.identity_map_index)
+    code = DTYPE_CODE[dtype]
+    grad_x = grad_w = None
+
+    if need_input_grad:
+        if n_in == 0 or n_out == 0:
+            grad_x = torch.zeros_like(x)
+        else:
+            symmetric = 1 if (km._symmetric and km._out_ascend and n_in == n_out) else 0
+            ascend = 1 if (symmetric or km._in_ascend) else 0
+            gs = km._group_start if symmetric else km._in_group_start
+            group_start = None
+            if ascend and gs is not None and gs[2] == (K, n_in):
+                group_start = ctypes.c_void_p(gs[1])
+            ws = workspace(L.wcn_conv_workspace_bytes(n_in, K, c_out, c_in, code, num_pairs, ascend),
+                           device)
+            grad_x = torch.empty((n_in, c_in), dtype=dtype, device=device)
+            check(L.wcn_sparse_conv_dgrad(ptr(gy), n_out, c_out, code, ptr(w), DTYPE_CODE[w.dtype], K,
+                                          c_in, ptr(km.in_maps), ptr(km.out_maps), host_offsets, iden,
+                                          symmetric, 1 if km._in_ascend else 0, group_start,
+                                          ptr(grad_x), n_in, ptr(ws), ws.numel(), stream_ptr(device)),
+                  "wcn_sparse_conv_dgrad")
+        grad_x = grad_x.to(in_features.dtype)
+
+    if need_weight_grad:
+        grad_w = torch.empty((K, c_in, c_out), dtype=w.dtype, device=device)
+        identity_rows = min(n_in, n_out) if iden >= 0 else 0
+        ws = workspace(L.wcn_conv_wgrad_workspace_bytes(K, c_in, c_out, num_pairs, identity_rows),
+                       device)
+        check(L.wcn_sparse_conv_wgrad(ptr(x), n_in, c_in, ptr(gy), n_out, c_out, code,
+                                      ptr(km.in_maps), ptr(km.out_maps), host_offsets, K, iden,
+                                      ptr(grad_w), DTYPE_CODE[w.dtype], ptr(ws), ws.numel(),
+                                      stream_ptr(device)), "wcn_sparse_conv_wgrad")
+        grad_w = grad_w.to(weight.dtype)
+    return grad_x, grad_w
 
 
 class UnifiedSpatiallySparseConvFunction(Function):
@@ -156,12 +197,10 @@ class UnifiedSpatiallySparseConvFunction(Function):
     @staticmethod
     def backward(ctx, grad_output):
         in_features, weight = ctx.saved_tensors
-        grad_x, grad_w = _explicit_gemm_backward_logic(grad_output, in_features, weight,
-                                                       ctx.kernel_map, ctx.compute_dtype)
-        if not ctx.needs_input_grad[0]:
-            grad_x = None
-        if not ctx.needs_input_grad[1]:
-            grad_w = None
+        grad_x, grad_w = sparse_conv_backward(grad_output, in_features, weight, ctx.kernel_map,
+                                              ctx.compute_dtype,
+                                              need_input_grad=ctx.needs_input_grad[0],
+                                              need_weight_grad=ctx.needs_input_grad[1])
         return grad_x, grad_w, None, None, None, None, None, None, None
 
 
@@ -224,6 +263,8 @@ def generate_output_coords_and_kernel_map(
                                               kernel_dilation, skip_symmetric_kernel_map=False)
         kernel_map = IntSearchResult(in_maps=forward_map.out_maps, out_maps=forward_map.in_maps,
                                      offsets=forward_map.offsets)
+        kernel_map._in_ascend = forward_map._out_ascend
+        kernel_map._in_group_start = forward_map._group_start
     else:
         kernel_map = generate_kernel_map(in_coords, out_coords, stride, kernel_size,
                                          kernel_dilation, skip_symmetric_kernel_map=False)
