@@ -83,6 +83,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time the gradients of the same convolution (reported under config.backward; "
+                         "the headline value stays the forward path)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -194,6 +197,33 @@ def main():
             "algorithmic_bytes": conv_bytes,
         },
     }
+
+    if args.backward:
+        from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_backward
+        gy = torch.randn(n, c_out, device=dev).to(torch.float16)
+        w32 = weight_d.float()  # parameters are fp32 in training; the weight gradient comes back in fp32
+        times = {}
+        for name, kw in (("dgrad", dict(need_weight_grad=False)), ("wgrad", dict(need_input_grad=False))):
+            for _ in range(args.warmup):
+                sparse_conv_backward(gy, feats_d, w32, km, **kw)
+            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            a0.record()
+            for _ in range(args.steps):
+                sparse_conv_backward(gy, feats_d, w32, km, **kw)
+            a1.record()
+            torch.cuda.synchronize()
+            times[name] = a0.elapsed_time(a1) / args.steps
+        wgrad_bytes = s * (n * c_in + n * c_out) + 8 * num_pairs + 4 * K * c_in * c_out
+        wgrad_flops = 2.0 * (num_pairs + n) * c_in * c_out  # the identity offset runs over all rows
+        result["config"]["backward"] = {
+            "dgrad_call_ms": times["dgrad"],
+            "wgrad_call_ms": times["wgrad"],
+            "dgrad_algorithmic_GBps": conv_bytes / (times["dgrad"] * 1e-3) / 1e9,
+            "wgrad_algorithmic_GBps": wgrad_bytes / (times["wgrad"] * 1e-3) / 1e9,
+            "wgrad_TFLOPs": wgrad_flops / (times["wgrad"] * 1e-3) / 1e12,
+            "note": "warm kernel map (the forward's), fp32 weights, whole calls incl. weight preparation",
+        }
 
     if not args.no_cpu_baseline:
         base, ref_out, _ = cpu_baseline(bcoords, feats, weight)

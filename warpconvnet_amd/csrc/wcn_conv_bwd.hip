@@ -13,9 +13,11 @@
 // order (no atomics: the result is bitwise reproducible) and rounds once to the weight dtype.
 //
 // The MFMA operands want, per lane, consecutive *pairs* of one channel, while a gathered feature
-// row holds consecutive channels of one pair.  The transposition happens on the way into LDS:
-// lane l of a wave fetches 16 bytes of the row of pair l and writes its elements to the LDS rows
-// of their channels, at position l: the 64 lanes of one such write fill 128 contiguous bytes.
+// row holds consecutive channels of one pair.  The transposition happens on the way into LDS: a
+// lane fetches 16 bytes of a gathered row and writes its elements to the LDS rows of their
+// channels, at the pair's position.  Four adjacent lanes fetch 64 contiguous bytes of one row (one
+// request to the vector cache instead of four), sixteen rows per load instruction; a transposing
+// write of the wave then covers 32 contiguous bytes in each of four LDS rows.
 #include <algorithm>
 
 #include "wcn_common.h"
@@ -27,6 +29,9 @@ using namespace wcn_mma;
 
 constexpr int WG_THREADS = 256;
 constexpr int TILE = 64;  // channels of X and of dY per workgroup
+#ifndef WCN_WGRAD_LPR
+#define WCN_WGRAD_LPR 4
+#endif
 
 struct WgradArgs {
   const void* X;
@@ -57,37 +62,51 @@ __global__ void __launch_bounds__(64) wgrad_plan(const int64_t* __restrict__ off
 }
 
 // 16 bytes (VEC elements) of row `row` starting at channel ch0, zeros where there is nothing.
-template <typename T>
+// With VECIO (rows are whole 16-byte vectors) every call is exactly one load, so the number of
+// loads in flight is known when the code is compiled and a wait for the oldest ones does not
+// wait for the newest; pieces that do not exist read the first bytes of the matrix instead and
+// are replaced by zeros afterwards.
+template <typename T, bool VECIO>
 __device__ __forceinline__ u32x4 load_piece(const T* __restrict__ base, int64_t row, int64_t num_rows,
-                                            int channels, int ch0, bool vec) {
+                                            int channels, int ch0) {
   constexpr int VEC = 16 / sizeof(T);
-  u32x4 r = (u32x4){0u, 0u, 0u, 0u};
-  if (row < 0 || row >= num_rows || ch0 >= channels) return r;
+  const u32x4 zero = (u32x4){0u, 0u, 0u, 0u};
+  const bool valid = row >= 0 && row < num_rows && ch0 < channels;
+  if (VECIO) {
+    const T* src = base + (valid ? row * channels + ch0 : 0);
+    const u32x4 got = *reinterpret_cast<const u32x4*>(src);
+    return valid ? got : zero;
+  }
+  if (!valid) return zero;
   const T* src = base + row * channels + ch0;
-  if (vec) return *reinterpret_cast<const u32x4*>(src);  // channels is a multiple of VEC here
   T tmp[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) tmp[j] = ch0 + j < channels ? src[j] : from_float<T>(0.f);
   return *reinterpret_cast<const u32x4*>(tmp);
 }
 
-template <typename T>
+// IDENT: the workgroups of this launch are the chunks of the identity offset (pair p is row p of
+// both matrices, no map is read); otherwise the launch covers every chunk and the workgroups of
+// the identity offset leave at once.  Two instances keep the hot loop free of branches.
+template <typename T, bool VECIO, bool IDENT>
 __global__ void __launch_bounds__(WG_THREADS) conv_wgrad(WgradArgs a) {
   typedef Mma<T> M;
   typedef typename M::V V;
   constexpr int CK = M::CK, KS = M::KS;      // pairs per step (one LDS row), MFMA k-steps per step
   constexpr int VEC = 16 / sizeof(T);
   constexpr int PARTS = TILE / VEC;           // 16-byte pieces of a 64-channel row
-  constexpr int PSEL = 64 / CK;               // lanes per pair in one load instruction
-  constexpr int NPI = PARTS / 2 / PSEL;       // pieces per thread and step
-  static_assert(NPI * PSEL * 2 == PARTS && CK * sizeof(T) == 128, "a step fills 128-byte LDS rows");
+  constexpr int NPI = CK * PARTS / 128;       // pieces per thread and step (two waves per operand)
+  constexpr int LPR = WCN_WGRAD_LPR;          // adjacent lanes on one gathered row
+  constexpr int RPI = 64 / LPR;               // rows per load instruction
+  constexpr int GROUPS = PARTS / LPR;         // groups of LPR pieces in a 64-channel row
+  static_assert(CK * sizeof(T) == 128 && NPI * RPI * 2 * LPR == CK * PARTS, "a step fills 128-byte LDS rows");
   // [buffer][operand][channel][pair]
   __shared__ __attribute__((aligned(16))) T tiles[2][2][TILE * CK];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kgrp = lane >> 4;
-  const int chunk = blockIdx.x;
+  const int chunk = IDENT ? a.chunk_first[a.identity] + (int)blockIdx.x : (int)blockIdx.x;
   const int ci0 = blockIdx.y * TILE, co0 = blockIdx.z * TILE;
 
   // which offset this chunk belongs to: the last k with chunk_first[k] <= chunk
@@ -97,36 +116,55 @@ __global__ void __launch_bounds__(WG_THREADS) conv_wgrad(WgradArgs a) {
     if (a.chunk_first[mid] <= chunk) lo = mid; else hi = mid;
   }
   const int k = lo;
-  const bool ident = k == a.identity;
-  const int64_t n_k = ident ? a.identity_rows : a.offsets[k + 1] - a.offsets[k];
+  if ((k == a.identity) != IDENT) return;  // the same for the whole workgroup
+  const int64_t n_k = IDENT ? a.identity_rows : a.offsets[k + 1] - a.offsets[k];
   const int64_t first = (int64_t)(chunk - a.chunk_first[k]) * a.pairs_per_chunk;  // inside the offset
   const int64_t left = n_k - first;
   const int count = (int)(left < a.pairs_per_chunk ? left : a.pairs_per_chunk);
   const int64_t pbase = a.offsets[k] + first;
   const int steps = (count + CK - 1) / CK;
 
-  // this thread's share of a step: operand (wave & 1), pair (lane % CK), NPI pieces
+  // this thread's share of a step: operand (wave & 1); piece i is 16 bytes of the row of pair
+  // pair_of(i), channels part_of(i) * VEC .. of the tile.  The wave pair (wave >> 1 = 0, 1) covers
+  // the step's CK pairs x PARTS pieces as 2 * NPI instructions of RPI rows x LPR pieces.
   const int operand = wave & 1;
-  const int pr = lane % CK, psel = lane / CK;
+  auto pair_of = [&](int i) { return (((wave >> 1) * NPI + i) / GROUPS) * RPI + lane / LPR; };
+  auto part_of = [&](int i) { return (((wave >> 1) * NPI + i) % GROUPS) * LPR + lane % LPR; };
+  constexpr int NROW = (NPI + GROUPS - 1) / GROUPS;  // distinct pairs among a thread's pieces
   const T* const src = (const T*)(operand ? a.dY : a.X);
   const int32_t* const map = operand ? a.out_maps : a.in_maps;
   const int64_t src_rows = operand ? a.num_out : a.num_in;
   const int src_ch = operand ? a.c_out : a.c_in;
   const int ch_base = operand ? co0 : ci0;
-  const bool vec = operand ? a.vec_out != 0 : a.vec_in != 0;
 
-  auto row_of = [&](int s) -> int64_t {  // source row of this thread's pair in step s, or -1
-    const int p = s * CK + pr;
-    if (s >= steps || p >= count) return -1;
-    return ident ? first + p : (int64_t)map[pbase + p];
+  // The map entry of piece i's pair in step s: always exactly one load, and the value is not
+  // touched until the rows are requested DEPTH steps later (a use right here would make the wave
+  // wait for the load at once).  Pairs past the chunk's end read its last entry; row_from sorts
+  // that out at the time of use.
+  auto raw_of = [&](int s, int i) -> int32_t {
+    if (IDENT) return 0;
+    const int p = s * CK + pair_of(i);
+    return map[pbase + (p < count ? p : count - 1)];  // count >= 1 in every launched chunk
   };
-  u32x4 piece[NPI];
-  auto fetch = [&](int64_t row) {
+  auto row_from = [&](int32_t raw, int s, int i) -> int64_t {  // source row, or -1
+    const int p = s * CK + pair_of(i);
+    const int64_t row = IDENT ? first + p : (int64_t)raw;
+    return p < count ? row : -1;
+  };
+  // the rows of DEPTH steps are in flight at any time (a step multiplies for a few hundred
+  // cycles, a gathered row takes a few thousand to arrive)
+  constexpr int DEPTH = 3;
+  u32x4 piece[DEPTH][NPI];
+  int32_t row_ahead[DEPTH][NROW];  // pieces i with the same i / GROUPS share a pair
+  auto rows_of = [&](int s, int32_t* raw) {
 #pragma unroll
-    for (int i = 0; i < NPI; ++i) {
-      const int part = (wave >> 1) * (PARTS / 2) + i * PSEL + psel;
-      piece[i] = load_piece<T>(src, row, src_rows, src_ch, ch_base + part * VEC, vec);
-    }
+    for (int g = 0; g < NROW; ++g) raw[g] = raw_of(s, g * GROUPS);
+  };
+  auto fetch = [&](const int32_t* raw, int s, u32x4* dst) {
+#pragma unroll
+    for (int i = 0; i < NPI; ++i)
+      dst[i] = load_piece<T, VECIO>(src, row_from(raw[i / GROUPS], s, i), src_rows, src_ch,
+                                    ch_base + part_of(i) * VEC);
   };
 
   // the wave's quadrant of the tile: 32 channels of X by 32 channels of dY
@@ -137,43 +175,55 @@ __global__ void __launch_bounds__(WG_THREADS) conv_wgrad(WgradArgs a) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  int64_t row_next = row_of(0);
-  fetch(row_next);
-  row_next = row_of(1);
-  for (int s = 0; s < steps; ++s) {
-    // transpose into LDS: element j of piece i goes to row (channel) part * VEC + j, position pr
-    T* const dst = tiles[s & 1][operand];
 #pragma unroll
-    for (int i = 0; i < NPI; ++i) {
-      const int part = (wave >> 1) * (PARTS / 2) + i * PSEL + psel;
-      const T* v = reinterpret_cast<const T*>(&piece[i]);
+  for (int u = 0; u < DEPTH; ++u) rows_of(u, row_ahead[u]);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const int ch = part * VEC + j;
-        dst[ch * CK + lds_part(ch, pr / VEC) * VEC + pr % VEC] = v[j];
+  for (int u = 0; u < DEPTH; ++u) {
+    fetch(row_ahead[u], u, piece[u]);
+    rows_of(DEPTH + u, row_ahead[u]);
+  }
+  // the step count is rounded up to a multiple of DEPTH (the extra steps multiply zeros), which
+  // keeps the loop free of exits in the middle
+  for (int s0 = 0; s0 < steps; s0 += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      const int s = s0 + u;
+      // transpose into LDS: element j of piece i goes to row (channel) part * VEC + j, position pr
+      T* const dst = tiles[s & 1][operand];
+#pragma unroll
+      for (int i = 0; i < NPI; ++i) {
+        const int part = part_of(i), pr = pair_of(i);
+        const T* v = reinterpret_cast<const T*>(&piece[u][i]);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const int ch = part * VEC + j;
+          dst[ch * CK + lds_part(ch, pr / VEC) * VEC + pr % VEC] = v[j];
+        }
       }
-    }
-    __syncthreads();  // step s is in LDS; everyone is done reading the other buffer
-    fetch(row_next);  // rows of step s + 1 travel while step s is multiplied
-    row_next = row_of(s + 2);
-    const T* const xt = tiles[s & 1][0];
-    const T* const yt = tiles[s & 1][1];
-    V xf[2][KS], yf[2][KS];
+      // step s is in LDS; everyone is done reading the other buffer.  (Written out because
+      // __syncthreads would also wait for the global loads in flight.)
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      fetch(row_ahead[u], s + DEPTH, piece[u]);  // rows of step s + DEPTH
+      rows_of(s + 2 * DEPTH, row_ahead[u]);
+      const T* const xt = tiles[s & 1][0];
+      const T* const yt = tiles[s & 1][1];
+      V xf[2][KS], yf[2][KS];
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      const int rx = qi + b * 16 + (lane & 15), ry = qo + b * 16 + (lane & 15);
+      for (int b = 0; b < 2; ++b) {
+        const int rx = qi + b * 16 + (lane & 15), ry = qo + b * 16 + (lane & 15);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        xf[b][ks] = M::load(xt + rx * CK, rx, ks, kgrp);
-        yf[b][ks] = M::load(yt + ry * CK, ry, ks, kgrp);
+        for (int ks = 0; ks < KS; ++ks) {
+          xf[b][ks] = M::load(xt + rx * CK, rx, ks, kgrp);
+          yf[b][ks] = M::load(yt + ry * CK, ry, ks, kgrp);
+        }
       }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) acc[i][j] = M::mma(xf[i][ks], yf[j][ks], acc[i][j]);
     }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = M::mma(xf[i][ks], yf[j][ks], acc[i][j]);
   }
 
   // a lane holds column (lane & 15) = channel of dY, rows 4 * kgrp .. + 3 = channels of X
@@ -190,22 +240,36 @@ __global__ void __launch_bounds__(WG_THREADS) conv_wgrad(WgradArgs a) {
       }
 }
 
-// dW[k][ci][co] = sum of the offset's chunks, in chunk order, rounded once.
+// dW[k][ci][co] = sum of the offset's chunks, rounded once.  A workgroup owns 256 consecutive
+// elements of one offset's padded (ci, co) plane; thread (j, e) adds the chunks c = j, j + 4, ...
+// of four adjacent elements, and the four partial sums are combined as (0 + 1) + (2 + 3): the
+// order of the additions is fixed, so the result is bitwise reproducible.
 template <typename WT>
 __global__ void __launch_bounds__(256) wgrad_reduce(const float* __restrict__ partial,
                                                     const int32_t* __restrict__ chunk_first, int K,
                                                     int c_in, int c_out, int c_in_pad, int c_out_pad,
                                                     WT* __restrict__ dW) {
-  const int64_t total = (int64_t)K * c_in * c_out;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    const int co = (int)(i % c_out);
-    const int ci = (int)((i / c_out) % c_in);
-    const int k = (int)(i / ((int64_t)c_in * c_out));
-    float sum = 0.f;
-    for (int c = chunk_first[k]; c < chunk_first[k + 1]; ++c)
-      sum += partial[((int64_t)c * c_in_pad + ci) * c_out_pad + co];
-    dW[i] = from_float<WT>(sum);
+  __shared__ f32x4 part[4][64];
+  const int plane = c_in_pad * c_out_pad;
+  const int slices = plane / 256;
+  const int k = blockIdx.x / slices, slice = blockIdx.x % slices;
+  const int j = threadIdx.x >> 6, e = threadIdx.x & 63;
+  const int elem = slice * 256 + e * 4;  // first of this thread's four elements in the plane
+  const int c0 = chunk_first[k], c1 = chunk_first[k + 1];
+  f32x4 sum = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int c = c0 + j; c < c1; c += 4)
+    sum += *reinterpret_cast<const f32x4*>(partial + (int64_t)c * plane + elem);
+  part[j][e] = sum;
+  __syncthreads();
+  if (j == 0) {
+    const f32x4 total = (part[0][e] + part[1][e]) + (part[2][e] + part[3][e]);
+    const int ci = elem / c_out_pad, co = elem % c_out_pad;
+    if (ci < c_in) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (co + r < c_out) dW[((int64_t)k * c_in + ci) * c_out + co + r] = from_float<WT>(total[r]);
+    }
   }
 }
 
@@ -241,10 +305,21 @@ inline size_t wgrad_layout(void* base, int K, int c_in, int c_out, int64_t pairs
   return off;
 }
 
-template <typename T>
-void launch_wgrad(const WgradArgs& a, int chunks, hipStream_t s) {
+template <typename T, bool VECIO>
+void launch_wgrad_io(const WgradArgs& a, int chunks, int identity_chunks, bool have_pairs, hipStream_t s) {
   const dim3 grid((unsigned)chunks, (unsigned)(a.c_in_pad / TILE), (unsigned)(a.c_out_pad / TILE));
-  hipLaunchKernelGGL(conv_wgrad<T>, grid, dim3(WG_THREADS), 0, s, a);
+  if (have_pairs) hipLaunchKernelGGL((conv_wgrad<T, VECIO, false>), grid, dim3(WG_THREADS), 0, s, a);
+  if (identity_chunks > 0) {
+    const dim3 igrid((unsigned)identity_chunks, grid.y, grid.z);
+    hipLaunchKernelGGL((conv_wgrad<T, VECIO, true>), igrid, dim3(WG_THREADS), 0, s, a);
+  }
+}
+template <typename T>
+void launch_wgrad(const WgradArgs& a, int chunks, int identity_chunks, bool have_pairs, hipStream_t s) {
+  if (a.vec_in && a.vec_out)
+    launch_wgrad_io<T, true>(a, chunks, identity_chunks, have_pairs, s);
+  else
+    launch_wgrad_io<T, false>(a, chunks, identity_chunks, have_pairs, s);
 }
 
 }  // namespace
@@ -318,14 +393,15 @@ int wcn_sparse_conv_wgrad(const void* features, int64_t num_in, int32_t c_in, co
   a.vec_in = (((size_t)c_in * es) % 16 == 0 && ((uintptr_t)features % 16) == 0) ? 1 : 0;
   a.vec_out = (((size_t)c_out * es) % 16 == 0 && ((uintptr_t)grad_out % 16) == 0) ? 1 : 0;
   if (chunks > 0) {
+    const int ichunks = (int)((identity_rows + ppc - 1) / ppc);
+    const bool have_pairs = chunks > ichunks && L > 0;  // the map is only read if it is not empty
     switch (dtype) {
-      case WCN_DTYPE_F32: launch_wgrad<float>(a, (int)chunks, s); break;
-      case WCN_DTYPE_F16: launch_wgrad<_Float16>(a, (int)chunks, s); break;
-      default: launch_wgrad<__bf16>(a, (int)chunks, s); break;
+      case WCN_DTYPE_F32: launch_wgrad<float>(a, (int)chunks, ichunks, have_pairs, s); break;
+      case WCN_DTYPE_F16: launch_wgrad<_Float16>(a, (int)chunks, ichunks, have_pairs, s); break;
+      default: launch_wgrad<__bf16>(a, (int)chunks, ichunks, have_pairs, s); break;
     }
   }
-  const int64_t total = (int64_t)num_offsets * c_in * c_out;
-  const unsigned rgrid = (unsigned)std::min<int64_t>(4096, (total + 255) / 256);
+  const unsigned rgrid = (unsigned)((int64_t)num_offsets * (a.c_in_pad * a.c_out_pad / 256));
   if (weight_dtype == WCN_DTYPE_F32) {
     hipLaunchKernelGGL(wgrad_reduce<float>, dim3(rgrid), dim3(256), 0, s, (const float*)w.partial,
                        (const int32_t*)w.chunk_first, num_offsets, c_in, c_out, a.c_in_pad,
