@@ -77,6 +77,163 @@ def cpu_baseline(bcoords, feats, weight):
     }, out, (im, om, off)
 
 
+def secondary_configs(dev, steps, warmup):
+    """The other single-layer configurations (parity-test cases; reported under config.other_configs
+    with --all-configs, never as the headline value): cold map build + contraction per step."""
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.search_results import IntSearchResult
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    from warpconvnet_amd.utils import synthetic
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(steps):
+            r = fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps, r
+
+    def weights(K, ci, co, dtype, seed):
+        g = torch.Generator().manual_seed(seed)
+        return (torch.randn(K, ci, co, generator=g) * (2.0 / (ci * K)) ** 0.5).to(dtype).to(dev)
+
+    def single(name, bc, ksize, ci, co, dtype, out):
+        c = torch.as_tensor(bc, device=dev)
+        n = len(bc)
+        K = int(np.prod(ksize))
+        x = torch.randn(n, ci, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
+        w = weights(K, ci, co, dtype, 2)
+        t_map, km = timed(lambda: generate_kernel_map(c, c, (1, 1, 1), ksize))
+        t_conv, _ = timed(lambda: sparse_conv_forward(x, w, km, n))
+        L = int(km.offsets[-1])
+        out[name] = {"num_voxels": n, "num_pairs": L, "kernel_map_build_ms": t_map,
+                     "contraction_call_ms": t_conv, "voxels_per_s": n / ((t_map + t_conv) * 1e-3),
+                     "contraction_TFLOPs": 2.0 * L * ci * co / (t_conv * 1e-3) / 1e12}
+
+    out = {}
+    single("configs[0]: 3x3x3 32->32 fp32, 100k voxels on 3 spheres",
+           synthetic.batch_indexed([synthetic.spheres_scene(0, 100_000, 0.01)]), (3, 3, 3), 32, 32,
+           torch.float32, out)
+    items, _ = synthetic.indoor_batch(4, 250_000, 0.02, seed=0)
+    bc = synthetic.batch_indexed(items)
+    single("configs[4a]: 5x5x5 16->16 fp16, 1M voxels", bc, (5, 5, 5), 16, 16, torch.float16, out)
+    coarse_items = [synthetic.indoor_scene(b, None, 0.16) for b in range(4)]
+    single("configs[4b]: 3x3x3 256->256 fp16, 16 cm voxels", synthetic.batch_indexed(coarse_items),
+           (3, 3, 3), 256, 256, torch.float16, out)
+    # configs[2]: 2x2x2 stride-2 96 -> 128 and its transposed 128 -> 96, bf16, 1M fine voxels
+    c = torch.as_tensor(bc, device=dev)
+    n = len(bc)
+    x = torch.randn(n, 96, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(dev)
+    wd, wu = weights(8, 96, 128, torch.bfloat16, 4), weights(8, 128, 96, torch.bfloat16, 5)
+
+    def build():
+        coarse, _ = stride_coords(c, (2, 2, 2))
+        return coarse, generate_kernel_map(c, coarse, (2, 2, 2), (2, 2, 2))
+
+    t_map, (coarse, km) = timed(build)
+    m = len(coarse)
+    t_down, y = timed(lambda: sparse_conv_forward(x, wd, km, m))
+    up = IntSearchResult(km.out_maps, km.in_maps, km.offsets)
+    up._in_ascend, up._in_group_start = km._out_ascend, km._group_start
+    t_up, _ = timed(lambda: sparse_conv_forward(y, wu, up, n))
+    out["configs[2]: 2x2x2 s2 96->128 + transposed 128->96 bf16, 1M fine voxels"] = {
+        "num_voxels": n, "num_coarse": m, "num_pairs": int(km.offsets[-1]),
+        "coords_and_kernel_map_build_ms": t_map, "down_contraction_call_ms": t_down,
+        "up_contraction_call_ms": t_up, "voxels_per_s": n / ((t_map + t_down + t_up) * 1e-3)}
+    return out
+
+
+class _UNet:
+    """configs[3]: MinkUNet18-style encoder-decoder for inference: 3x3x3 stem (C = 32), four down
+    stages (32, 64, 128, 256: 2x2x2 stride-2 convolution + two residual blocks of two 3x3x3
+    convolutions) and four up stages (transposed 2x2x2 stride-2 convolution, skip concatenation,
+    two residual blocks, 1x1 shortcut where the channel count changes).  Batch norm is folded into
+    the convolutions' weight and bias; ReLU and the residual adds are torch elementwise ops."""
+
+    def __init__(self, dev, dtype, seed=0):
+        from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d
+        torch.manual_seed(seed)
+        mk = lambda *a, **k: SparseConv3d(*a, bias=True, **k).to(dev).to(dtype)  # noqa: E731
+        enc = (32, 64, 128, 256)
+        self.stem = mk(3, 32, 3)
+        self.down, self.enc_blocks = [], []
+        prev = 32
+        for ch in enc:
+            self.down.append(mk(prev, ch, 2, stride=2))
+            self.enc_blocks.append([(mk(ch, ch, 3), mk(ch, ch, 3), None) for _ in range(2)])
+            prev = ch
+        skips = (128, 64, 32, 32)  # channels of the encoder level each up stage lands on
+        self.up, self.dec_blocks = [], []
+        for ch in skips:
+            self.up.append(mk(prev, ch, 2, stride=2, transposed=True))
+            self.dec_blocks.append([(mk(2 * ch, ch, 3), mk(ch, ch, 3), mk(2 * ch, ch, 1)),
+                                    (mk(ch, ch, 3), mk(ch, ch, 3), None)])
+            prev = ch
+
+    @staticmethod
+    def _relu(x):
+        return x.replace(batched_features=torch.relu(x.feature_tensor))
+
+    def _block(self, x, blk):
+        a, b, shortcut = blk
+        y = b(self._relu(a(x)))
+        skip = x if shortcut is None else shortcut(x)
+        return self._relu(y.replace(batched_features=y.feature_tensor + skip.feature_tensor))
+
+    @torch.no_grad()
+    def __call__(self, x):
+        levels = [self._relu(self.stem(x))]
+        for down, blocks in zip(self.down, self.enc_blocks):
+            y = self._relu(down(levels[-1]))
+            for blk in blocks:
+                y = self._block(y, blk)
+            levels.append(y)
+        y = levels.pop()
+        for up, blocks in zip(self.up, self.dec_blocks):
+            skip = levels.pop()
+            y = self._relu(up(y, skip))
+            y = y.replace(batched_features=torch.cat([y.feature_tensor, skip.feature_tensor], dim=1))
+            for blk in blocks:
+                y = self._block(y, blk)
+        return y
+
+
+def unet_config(dev, steps, warmup):
+    """One inference pass per step over a fresh Voxels (every kernel map is rebuilt, as for a new
+    input): 4 x 250k voxels, 3-channel features, bf16, random-init weights."""
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    from warpconvnet_amd.utils import synthetic
+    items, offsets = synthetic.indoor_batch(4, 250_000, 0.02, seed=0)
+    coords = torch.as_tensor(np.concatenate(items), dtype=torch.int32, device=dev)
+    n = coords.shape[0]
+    feats = torch.randn(n, 3, generator=torch.Generator().manual_seed(11)).to(torch.bfloat16).to(dev)
+    net = _UNet(dev, torch.bfloat16)
+
+    def run():
+        return net(Voxels(coords, feats, offsets=torch.as_tensor(np.asarray(offsets))))
+
+    for _ in range(warmup):
+        out = run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = run()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    assert out.feature_tensor.shape == (n, 32) and bool(torch.isfinite(out.feature_tensor).all())
+    convs = [net.stem] + net.down + net.up + [m for stage in net.enc_blocks + net.dec_blocks
+                                             for blk in stage for m in blk if m is not None]
+    sparse = sum(1 for m in convs if int(np.prod(m.kernel_size)) > 1)
+    return {"num_voxels": n, "sparse_convolutions": sparse, "pointwise_convolutions": len(convs) - sparse,
+            "ms_per_pass": ms,
+            "voxels_per_s": n / (ms * 1e-3)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -86,6 +243,8 @@ def main():
     ap.add_argument("--backward", action="store_true",
                     help="also time the gradients of the same convolution (reported under config.backward; "
                          "the headline value stays the forward path)")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also time the other single-layer configurations (config.other_configs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -224,6 +383,11 @@ def main():
             "wgrad_TFLOPs": wgrad_flops / (times["wgrad"] * 1e-3) / 1e12,
             "note": "warm kernel map (the forward's), fp32 weights, whole calls incl. weight preparation",
         }
+
+    if args.all_configs:
+        result["config"]["other_configs"] = secondary_configs(dev, max(3, args.steps // 2), 2)
+        result["config"]["other_configs"]["configs[3]: MinkUNet18-style encoder-decoder, bf16, 1M voxels"] = \
+            unet_config(dev, max(3, args.steps // 4), 2)
 
     if not args.no_cpu_baseline:
         base, ref_out, _ = cpu_baseline(bcoords, feats, weight)

@@ -206,3 +206,29 @@ def test_module_autocast_and_backward():
     ref.square().sum().backward()
     assert rel_err(xg.grad.cpu().numpy(), xc.grad.numpy()) <= 1e-4
     assert rel_err(conv.weight.grad.cpu().numpy(), wc.grad.numpy()) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype,c_in,c_out", [(torch.float32, 7, 13), (torch.float16, 3, 32),
+                                               (torch.bfloat16, 13, 7)])
+def test_c_abi_with_rows_that_are_not_16_byte_vectors(oracle, dtype, c_in, c_out):
+    """wcn_sparse_conv_fwd called directly with channel counts whose rows are not whole 16-byte
+    vectors: the library's general kernel (the Python entry points pad such inputs instead)."""
+    import ctypes
+    from warpconvnet_amd._lib import DTYPE_CODE, check, lib, ptr, stream_ptr, workspace
+    bc = synthetic.random_cloud(70, 4000, 22, batch_size=2)
+    n = len(bc)
+    im, om, off, iden = oracle.kernel_map(bc, bc, (3, 3, 3))
+    x = normal_features(n, c_in, seed=1, dtype=dtype)
+    w = kaiming_weight(27, c_in, c_out, seed=2, dtype=dtype)
+    L = lib()
+    code = DTYPE_CODE[dtype]
+    ws = workspace(L.wcn_conv_workspace_bytes(n, 27, c_in, c_out, code, len(im), 1), DEV)
+    out = torch.empty(n, c_out, dtype=dtype, device=DEV)
+    xd, wd = x.to(DEV), w.to(DEV)
+    imd, omd = _dev_i32(im), _dev_i32(om)
+    offs = (ctypes.c_int64 * 28)(*[int(v) for v in off])
+    check(L.wcn_sparse_conv_fwd(ptr(xd), n, c_in, code, ptr(wd), code, 27, c_out, None, ptr(imd),
+                                ptr(omd), offs, iden, 1, None, ptr(out), n, ptr(ws), ws.numel(),
+                                stream_ptr(torch.device(DEV))), "wcn_sparse_conv_fwd")
+    want = oracle.explicit_conv_f64(x.double().numpy(), w.double().numpy(), im, om, off, iden, n)
+    assert rel_err(out.float().cpu().numpy(), want) <= TOL[dtype]

@@ -14,8 +14,19 @@ def batch_index_from_offset(offsets: Tensor) -> Tensor:
 @torch.no_grad()
 def batch_indexed_coordinates(batched_coords: Tensor, offsets: Tensor) -> Tensor:
     """(N, D) coordinates -> (N, D+1) rows [batch, ...] in the coordinate dtype and device
-    (reference: batch_index.py:110-117)."""
-    batch_index = batch_index_from_offset(offsets).to(batched_coords)
+    (reference: batch_index.py:110-117).  For coordinates on a GPU the batch column is made on
+    the device from the B + 1 offsets (sent through pinned memory without waiting for the stream)
+    instead of being expanded on the host and copied."""
+    if batched_coords.is_cuda:
+        n = batched_coords.shape[0]
+        bounds = offsets[1:].to(dtype=torch.int64, device="cpu")
+        staged = torch.empty(bounds.shape, dtype=torch.int64, pin_memory=True)
+        staged.copy_(bounds)
+        bounds_dev = staged.to(batched_coords.device, non_blocking=True)
+        rows = torch.arange(n, device=batched_coords.device, dtype=torch.int64)
+        batch_index = torch.searchsorted(bounds_dev, rows, right=True).to(batched_coords.dtype)
+    else:
+        batch_index = batch_index_from_offset(offsets).to(batched_coords)
     return torch.cat([batch_index.unsqueeze(1), batched_coords], dim=1)
 
 

@@ -56,6 +56,11 @@ class POINT_ORDERING(enum.Enum):
     MORTON_XYZ = "morton_xyz"
 
 
+def in_coords_of(voxels: Voxels):
+    """The cached (N, D+1) batch-indexed rows of a tensor (the same object on every access)."""
+    return voxels.batched_coordinates.batch_indexed_coordinates
+
+
 def _is_random_order(order) -> bool:
     return str(getattr(order, "value", order)).lower() == "random"
 
@@ -85,6 +90,14 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
         w = w.to(x.dtype)
     w = w.contiguous()
     b = None if bias is None else bias.detach().to(x.dtype).contiguous()
+    # Feature rows that are not whole 16-byte vectors (the 3-channel input of a network's stem)
+    # would take the library's slow general kernel: zero-pad the channels instead (the matching
+    # weight rows are zero, the result is unchanged).
+    vec = 16 // x.element_size()
+    if x.shape[1] % vec != 0 and x.shape[0] > 0:
+        pad = vec - x.shape[1] % vec
+        x = torch.nn.functional.pad(x, (0, pad))
+        w = torch.nn.functional.pad(w, (0, 0, 0, pad))
     km = kernel_map
     K, c_in, c_out = w.shape
     device = x.device
@@ -367,8 +380,20 @@ def spatially_sparse_conv(
         out_features = sparse_conv_forward(features, weight, kernel_map, num_out_coords, bias=bias,
                                            compute_dtype=effective_compute_dtype)
 
+    # The output's coordinate object.  Where the output rows are an existing tensor's (stride 1,
+    # or a given output tensor) that tensor's coordinate object is reused, and a newly made one is
+    # seeded with the (M, D+1) rows already at hand: either way the batch-indexed rows are not
+    # rebuilt by the next layer (the reference rebuilds them in every call, geometry.py:141-142).
+    if out_coords is in_coords_of(input_sparse_tensor):
+        new_coords = input_sparse_tensor.batched_coordinates
+    elif output_spatially_sparse_tensor is not None and \
+            out_coords is in_coords_of(output_spatially_sparse_tensor):
+        new_coords = output_spatially_sparse_tensor.batched_coordinates
+    else:
+        new_coords = IntCoords(out_coords[:, 1:], offsets=out_offsets.cpu().int())
+        new_coords._batch_indexed = out_coords
     return input_sparse_tensor.replace(
-        batched_coordinates=IntCoords(out_coords[:, 1:], offsets=out_offsets.cpu().int()),
+        batched_coordinates=new_coords,
         batched_features=out_features,
         tensor_stride=out_tensor_stride,
     )
