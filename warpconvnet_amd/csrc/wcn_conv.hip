@@ -84,6 +84,11 @@ struct ConvArgs {
   int32_t vec_in;   // feature rows are 16-byte aligned and a whole number of 16-byte vectors
   int32_t vec_out;  // same for output rows
   int32_t flat_in;  // c_in is a multiple of the staged row and the feature matrix is below 4 GiB
+  // Few output tiles and several slices of input channels (small maps with wide features): the
+  // slices go to different workgroups (blockIdx.z), each writes its fp32 sums to
+  // partial[slice][row][c_out_pad] and conv_split_reduce adds them in slice order.
+  int32_t split;
+  float* partial;
 };
 
 // One batch = up to BATCH offsets and A_ROWS pairs; the pairs of one offset may be split over
@@ -511,7 +516,7 @@ __device__ __forceinline__ int step_num(uint32_t w0) { return (int)((w0 >> 8) & 
 __device__ __forceinline__ int step_first(uint32_t w0) { return (int)((w0 >> 16) & 0x1FFu); }
 __device__ __forceinline__ bool step_identity(uint32_t w0) { return (w0 >> 31) != 0u; }
 
-template <typename T, int NC>
+template <typename T, int NC, bool SPLIT>
 __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
   typedef Mma<T> M;
   typedef typename M::V V;
@@ -548,7 +553,9 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
   if (tid < 32) ((uint32_t*)(smem + C::ZERO_OFF))[tid] = 0u;
   T* __restrict__ out = (T*)a.out;
   T* const stage = (T*)ring;  // output tile staged for 16-byte stores: RROWS x 128 bytes (the rings are contiguous)
-  const bool staged = sizeof(T) == 2 && a.vec_out;
+  const bool staged = sizeof(T) == 2 && a.vec_out && !SPLIT;
+  const int c0_begin = SPLIT ? (int)blockIdx.z * CK : 0;       // this workgroup's input-channel slices
+  const int c0_end = SPLIT ? c0_begin + CK : a.c_in_pad;
 
   // Start of a chunk (up to 32 offsets of one slice of input channels): the step plan and clean
   // slot tables.  Every wave runs it; returns the number of steps.
@@ -611,7 +618,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
     for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) acc[rb][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    for (int c0 = 0; c0 < a.c_in_pad; c0 += CK) {
+    for (int c0 = c0_begin; c0 < c0_end; c0 += CK) {
       for (int kbase = 0; kbase < a.K; kbase += 32) {
         const int S = begin_chunk(kbase);
         if (S == 0) continue;
@@ -682,10 +689,23 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int col = n0 + nb * 16 + kgrp * 4 + r;
-        bias_v[nb][r] = (bias && col < a.c_out) ? to_float(bias[col]) : 0.f;
+        bias_v[nb][r] = (bias && !SPLIT && col < a.c_out) ? to_float(bias[col]) : 0.f;
       }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // every wave is done with the rings, every load has landed
+    if (SPLIT) {  // fp32 sums of this slice, 16 bytes per lane and block; bias and rounding come later
+      float* const slice = a.partial + (int64_t)blockIdx.z * a.num_out * a.c_out_pad;
+#pragma unroll
+      for (int rb = 0; rb < 4; ++rb) {
+        const int lr = (rb * NC + wave) * 16 + (lane & 15);
+        if (m0 + lr < a.num_out) {
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+            *reinterpret_cast<f32x4*>(slice + (m0 + lr) * a.c_out_pad + n0 + nb * 16 + kgrp * 4) = acc[rb][nb];
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
       const int lr = (rb * NC + wave) * 16 + (lane & 15);
@@ -711,7 +731,7 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
       }
     }
   } else {
-    for (int c0 = 0; c0 < a.c_in_pad; c0 += CK) {
+    for (int c0 = c0_begin; c0 < c0_end; c0 += CK) {
       for (int kbase = 0; kbase < a.K; kbase += 32) {
         const int S = begin_chunk(kbase);
         if (S == 0) continue;
@@ -831,6 +851,27 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
             *reinterpret_cast<const u32x4*>(&stage[r * CK + lds_part(r, part) * VEC]);
     }
   }
+}
+
+// out[m][c] = bias[c] + the slices' partial sums added in slice order, rounded once (one thread per
+// four channels).
+template <typename T>
+__global__ void __launch_bounds__(256) conv_split_reduce(const float* __restrict__ partial, int slices,
+                                                         int64_t num_out, int c_out, int c_out_pad,
+                                                         const T* __restrict__ bias, T* __restrict__ out) {
+  const int quads = c_out_pad / 4;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= num_out * quads) return;
+  const int64_t m = i / quads;
+  const int col = (int)(i % quads) * 4;
+  if (col >= c_out) return;
+  f32x4 sum = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int z = 0; z < slices; ++z)
+    sum += *reinterpret_cast<const f32x4*>(partial + ((int64_t)z * num_out + m) * c_out_pad + col);
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (col + r < c_out)
+      out[m * c_out + col + r] = from_float<T>(sum[r] + (bias ? to_float(bias[col + r]) : 0.f));
 }
 
 // group_start[k][g] = number of pairs of offset k with out_maps < 64 * g (binary search; needs
@@ -959,6 +1000,13 @@ inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
 inline size_t elem_size(int dtype) { return dtype == WCN_DTYPE_F32 ? 4 : 2; }
 inline int ck_of(int dtype) { return dtype == WCN_DTYPE_F32 ? Mma<float>::CK : Mma<_Float16>::CK; }
 
+// Slices of input channels go to separate workgroups when the output tiles alone would leave most
+// of the 256 CUs (two workgroups each) idle.
+inline bool conv_wants_split(int64_t num_out, int c_in_pad, int c_out_pad, int ck) {
+  const int64_t tiles = (num_out + 64 * WCN_RING_NC - 1) / (64 * WCN_RING_NC) * (c_out_pad / TN);
+  return c_in_pad / ck > 1 && tiles <= 256;
+}
+
 struct ConvWorkspace {
   int64_t* offsets;      // K+1 (device copy of the host offsets)
   void* Wt;              // K * c_out_pad * c_in_pad elements
@@ -971,6 +1019,7 @@ struct ConvWorkspace {
   int32_t* groups;
   int32_t* in_sorted;
   int32_t* out_sorted;
+  float* partial;        // (slices, num_out, c_out_pad) when the input-channel slices are split
   int c_in_pad, c_out_pad, words;
   int64_t G;
 };
@@ -992,6 +1041,11 @@ inline size_t conv_layout(void* base, int64_t num_out, int K, int c_in, int c_ou
   off += wcn_align256(sizeof(int32_t) * (size_t)K * (size_t)(G + 1));
   if (w) w->row_total = (int64_t*)(p + off);
   off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
+  if (w) w->partial = nullptr;
+  if (conv_wants_split(num_out, cip, cop, ck_of(dtype))) {
+    if (w) w->partial = (float*)(p + off);
+    off += wcn_align256(sizeof(float) * (size_t)(cip / ck_of(dtype)) * (size_t)num_out * cop);
+  }
   if (resort_pairs >= 0) {
     if (w) w->row_mask = (uint32_t*)(p + off);
     off += wcn_align256(sizeof(uint32_t) * (size_t)num_out * words);
@@ -1042,7 +1096,9 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) return WCN_ERR_LAUNCH;
     if (allowed_device != device) {
-      if (hipFuncSetAttribute((const void*)conv_fwd_ring<T, NC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+      if (hipFuncSetAttribute((const void*)conv_fwd_ring<T, NC, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              RingCfg<NC>::LDS_BYTES) != hipSuccess ||
+          hipFuncSetAttribute((const void*)conv_fwd_ring<T, NC, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               RingCfg<NC>::LDS_BYTES) != hipSuccess)
         return WCN_ERR_LAUNCH;
       allowed_device = device;
@@ -1050,8 +1106,18 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
   }
   if (g_time_start) (void)hipEventRecord(g_time_start, s);
   if (a.vec_in) {
-    const dim3 rgrid((unsigned)((a.num_out + RingCfg<NC>::RROWS - 1) / RingCfg<NC>::RROWS), grid.y);
-    hipLaunchKernelGGL((conv_fwd_ring<T, NC>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
+    const unsigned slices = a.split ? (unsigned)(a.c_in_pad / Mma<T>::CK) : 1u;
+    const dim3 rgrid((unsigned)((a.num_out + RingCfg<NC>::RROWS - 1) / RingCfg<NC>::RROWS), grid.y, slices);
+    if (a.split)
+      hipLaunchKernelGGL((conv_fwd_ring<T, NC, true>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
+    else
+      hipLaunchKernelGGL((conv_fwd_ring<T, NC, false>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
+    if (a.split) {
+      const int64_t items = a.num_out * (a.c_out_pad / 4);
+      hipLaunchKernelGGL(conv_split_reduce<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
+                         (const float*)a.partial, (int)slices, a.num_out, a.c_out, a.c_out_pad,
+                         (const T*)a.bias, (T*)a.out);
+    }
   } else {
     hipLaunchKernelGGL(conv_fwd<T>, grid, dim3(THREADS), 0, s, a);
   }
@@ -1173,6 +1239,8 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   a.vec_in = (((size_t)c_in * es) % 16 == 0 && ((uintptr_t)features % 16) == 0) ? 1 : 0;
   a.vec_out = (((size_t)c_out * es) % 16 == 0 && ((uintptr_t)out % 16) == 0) ? 1 : 0;
   a.flat_in = (c_in % ck_of(dtype) == 0 && (uint64_t)num_in * c_in * es < (1ull << 32)) ? 1 : 0;
+  a.partial = w.partial;
+  a.split = (a.vec_in && w.partial != nullptr) ? 1 : 0;
   switch (dtype) {
     case WCN_DTYPE_F32:
       return launch_conv<float>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, s);
