@@ -516,14 +516,17 @@ __device__ __forceinline__ int step_num(uint32_t w0) { return (int)((w0 >> 8) & 
 __device__ __forceinline__ int step_first(uint32_t w0) { return (int)((w0 >> 16) & 0x1FFu); }
 __device__ __forceinline__ bool step_identity(uint32_t w0) { return (w0 >> 31) != 0u; }
 
-template <typename T, int NC, bool SPLIT>
+// NARROW: bit 0 = at most TN / 2 output channels, bit 1 = at most CK / 2 input channels.  The
+// multiplying waves then leave out the half of the channel blocks / k-steps that is padding (the
+// requests and the LDS layout stay as they are).
+template <typename T, int NC, bool SPLIT, int NARROW>
 __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
   typedef Mma<T> M;
   typedef typename M::V V;
   typedef RingCfg<NC> C;
-  constexpr int CK = M::CK, KS = M::KS;
+  constexpr int CK = M::CK, KS = (NARROW & 2) ? M::KS / 2 : M::KS;
   constexpr int VEC = 16 / sizeof(T);
-  constexpr int NB = TN / 16;
+  constexpr int NB = (NARROW & 1) ? TN / 32 : TN / 16;
   constexpr int RROWS = C::RROWS, NP = C::NP, PER = C::PER;
   static_assert(CK * sizeof(T) == 128, "ring rows are 128 bytes");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -1096,11 +1099,12 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) return WCN_ERR_LAUNCH;
     if (allowed_device != device) {
-      if (hipFuncSetAttribute((const void*)conv_fwd_ring<T, NC, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              RingCfg<NC>::LDS_BYTES) != hipSuccess ||
-          hipFuncSetAttribute((const void*)conv_fwd_ring<T, NC, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              RingCfg<NC>::LDS_BYTES) != hipSuccess)
-        return WCN_ERR_LAUNCH;
+      const void* instances[5] = {(const void*)conv_fwd_ring<T, NC, false, 0>, (const void*)conv_fwd_ring<T, NC, false, 1>,
+                                  (const void*)conv_fwd_ring<T, NC, false, 2>, (const void*)conv_fwd_ring<T, NC, false, 3>,
+                                  (const void*)conv_fwd_ring<T, NC, true, 0>};
+      for (const void* f : instances)
+        if (hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, RingCfg<NC>::LDS_BYTES) != hipSuccess)
+          return WCN_ERR_LAUNCH;
       allowed_device = device;
     }
   }
@@ -1108,10 +1112,18 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
   if (a.vec_in) {
     const unsigned slices = a.split ? (unsigned)(a.c_in_pad / Mma<T>::CK) : 1u;
     const dim3 rgrid((unsigned)((a.num_out + RingCfg<NC>::RROWS - 1) / RingCfg<NC>::RROWS), grid.y, slices);
+    // channel counts of at most half a tile leave out the padding half of the multiplications
+    const int narrow = (a.c_out <= TN / 2 ? 1 : 0) | (a.c_in <= Mma<T>::CK / 2 ? 2 : 0);
     if (a.split)
-      hipLaunchKernelGGL((conv_fwd_ring<T, NC, true>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
+      hipLaunchKernelGGL((conv_fwd_ring<T, NC, true, 0>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
+    else if (narrow == 0)
+      hipLaunchKernelGGL((conv_fwd_ring<T, NC, false, 0>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
+    else if (narrow == 1)
+      hipLaunchKernelGGL((conv_fwd_ring<T, NC, false, 1>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
+    else if (narrow == 2)
+      hipLaunchKernelGGL((conv_fwd_ring<T, NC, false, 2>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
     else
-      hipLaunchKernelGGL((conv_fwd_ring<T, NC, false>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
+      hipLaunchKernelGGL((conv_fwd_ring<T, NC, false, 3>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
     if (a.split) {
       const int64_t items = a.num_out * (a.c_out_pad / 4);
       hipLaunchKernelGGL(conv_split_reduce<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
