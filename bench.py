@@ -108,7 +108,11 @@ def secondary_configs(dev, steps, warmup):
         K = int(np.prod(ksize))
         x = torch.randn(n, ci, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
         w = weights(K, ci, co, dtype, 2)
-        t_map, km = timed(lambda: generate_kernel_map(c, c, (1, 1, 1), ksize))
+        def cold_map():
+            cold = c.view(-1, 4)  # a new tensor object: the coordinate table is built again
+            return generate_kernel_map(cold, cold, (1, 1, 1), ksize)
+
+        t_map, km = timed(cold_map)
         t_conv, _ = timed(lambda: sparse_conv_forward(x, w, km, n))
         L = int(km.offsets[-1])
         out[name] = {"num_voxels": n, "num_pairs": L, "kernel_map_build_ms": t_map,
@@ -132,8 +136,9 @@ def secondary_configs(dev, steps, warmup):
     wd, wu = weights(8, 96, 128, torch.bfloat16, 4), weights(8, 128, 96, torch.bfloat16, 5)
 
     def build():
-        coarse, _ = stride_coords(c, (2, 2, 2))
-        return coarse, generate_kernel_map(c, coarse, (2, 2, 2), (2, 2, 2))
+        cold = c.view(-1, 4)
+        coarse, _ = stride_coords(cold, (2, 2, 2))
+        return coarse, generate_kernel_map(cold, coarse, (2, 2, 2), (2, 2, 2))
 
     t_map, (coarse, km) = timed(build)
     m = len(coarse)
@@ -266,7 +271,8 @@ def main():
     L = lib()
 
     def step(time_kernel=None):
-        km = generate_kernel_map(coords_d, coords_d, (1, 1, 1), (3, 3, 3))
+        cold = coords_d.view(-1, 4)  # a new tensor object: no coordinate table is kept on it yet
+        km = generate_kernel_map(cold, cold, (1, 1, 1), (3, 3, 3))
         mid = torch.cuda.Event(enable_timing=True)
         mid.record()
         if time_kernel is not None:

@@ -206,3 +206,28 @@ def test_golden_fixtures_on_gpu():
         out = sparse_conv_forward(torch.as_tensor(g["features"], device=DEV),
                                   torch.as_tensor(g["weight"], device=DEV), km, len(g["out_coords"]))
         assert rel_err(out.cpu().numpy(), g["out_features_f64"]) <= 1e-5, path
+
+
+def test_maps_over_one_tensor_share_its_table(oracle):
+    """The coordinate table is kept on the input tensor object: a second map over the same rows
+    reuses it, an in-place change of the rows rebuilds it, and the maps are the oracle's either way."""
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    bc = synthetic.random_cloud(90, 5000, 24, batch_size=2)
+    c = torch.as_tensor(bc, device=DEV)
+    km3 = generate_kernel_map(c, c, (1, 1, 1), (3, 3, 3))
+    table = c._wcn_table[1]
+    coarse, _ = stride_coords(c, (2, 2, 2))
+    km2 = generate_kernel_map(c, coarse, (2, 2, 2), (2, 2, 2))
+    assert c._wcn_table[1] is table
+    for km, out, ks, st in ((km3, bc, (3, 3, 3), (1, 1, 1)), (km2, coarse.cpu().numpy(), (2, 2, 2), (2, 2, 2))):
+        im, om, off, _ = oracle.kernel_map(bc, out, ks, st)
+        assert np.array_equal(km.in_maps.cpu().numpy(), im) and np.array_equal(km.out_maps.cpu().numpy(), om)
+        assert np.array_equal(km.offsets.numpy(), off)
+    c[:, 1] += 3  # in place: the kept table no longer describes the rows
+    km3b = generate_kernel_map(c, c, (1, 1, 1), (3, 3, 3))
+    assert c._wcn_table[1] is not table
+    assert torch.equal(km3b.in_maps, km3.in_maps) and torch.equal(km3b.offsets, km3.offsets)  # a pure shift
+    q = torch.as_tensor(bc[:50], device=DEV)
+    q[:, 1] += 3
+    assert torch.equal(c._wcn_table[1].search(q).cpu(), torch.arange(50, dtype=torch.int32))

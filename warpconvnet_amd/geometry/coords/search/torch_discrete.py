@@ -89,6 +89,27 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     return result
 
 
+def _table_of(coords: Tensor, hash_method: HashMethod, device) -> TorchHashTable:
+    """The coordinate table of an input tensor, built once per tensor object: the maps of
+    different kernels over the same input rows (the 3x3x3 and the strided 2x2x2 map of one
+    resolution of a network) share it.  It is kept on the tensor object together with the
+    tensor's version counter, so an in-place change of the coordinates rebuilds it.  (The
+    reference builds a new table in every call, torch_discrete.py:398-401.)"""
+    kept = getattr(coords, "_wcn_table", None)
+    if kept is not None and kept[0] == coords._version:
+        return kept[1]
+    # built from an alias of the tensor (same storage, another Python object): the table keeps its
+    # keys alive, and keeping the table on `coords` itself would otherwise close a reference
+    # cycle that only the garbage collector could free
+    table = TorchHashTable.from_keys(coords.detach(), hash_method=hash_method, device=device,
+                                     _defer_check=True)
+    try:
+        coords._wcn_table = (coords._version, table)
+    except AttributeError:
+        pass
+    return table
+
+
 @torch.no_grad()
 def generate_kernel_map(
     batch_indexed_in_coords: Tensor,
@@ -132,8 +153,7 @@ def generate_kernel_map(
     if num_spatial_dims > 3:
         raise NotImplementedError("more than 3 spatial dimensions are not supported")
 
-    table = TorchHashTable.from_keys(batch_indexed_in_coords, hash_method=hash_method,
-                                     device=device, _defer_check=True)
+    table = _table_of(batch_indexed_in_coords, hash_method, device)
 
     is_odd = all(k % 2 == 1 for k in kernel_size)
     same_count = batch_indexed_in_coords.shape[0] == batch_indexed_out_coords.shape[0]
