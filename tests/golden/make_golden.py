@@ -15,7 +15,10 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
+import torch  # noqa: E402
+
 from oracle import cpu_oracle  # noqa: E402
+from oracle.explicit_conv import explicit_gemm_backward  # noqa: E402
 from warpconvnet_amd.utils import synthetic  # noqa: E402
 
 
@@ -32,11 +35,18 @@ def case(name, coords, ksize, stride, c_in, c_out, seed):
     x = rng.normal(size=(len(coords), c_in)).astype(np.float32)
     w = (rng.normal(size=(K, c_in, c_out)) * np.sqrt(2.0 / (c_in * K))).astype(np.float32)
     out = cpu_oracle.explicit_conv_f64(x, w, im, om, off, iden, len(out_coords))
+    # gradients of sum(out * grad_out): the torch restatement of the reference's explicit backward
+    # (sparse_conv.py:314-355) in float64
+    gy = rng.normal(size=(len(out_coords), c_out)).astype(np.float32)
+    gx, gw = explicit_gemm_backward(torch.from_numpy(gy).double(), torch.from_numpy(x).double(),
+                                    torch.from_numpy(w).double(), torch.from_numpy(im),
+                                    torch.from_numpy(om), off, iden)
     np.savez_compressed(os.path.join(HERE, name + ".npz"), in_coords=coords, kernel_size=np.array(ksize),
                         stride=np.array(stride), out_coords=out_coords, out_first_index=first,
                         out_offsets=np.asarray(out_offsets, np.int64), in_maps=im, out_maps=om,
                         offsets=off, identity=np.array(-1 if iden is None else iden),
-                        features=x, weight=w, out_features_f64=out)
+                        features=x, weight=w, out_features_f64=out, grad_out=gy,
+                        grad_features_f64=gx.numpy(), grad_weight_f64=gw.numpy())
 
 
 if __name__ == "__main__":

@@ -179,13 +179,13 @@ def test_empty_and_tiny_inputs():
 
 
 def test_golden_fixtures_on_gpu():
-    """Committed fixtures: strided coordinates, kernel map (bit-exact) and fp32 features."""
+    """Committed fixtures: strided coordinates, kernel map (bit-exact), fp32 features and gradients."""
     import glob
     import os
     from helpers import rel_err
     from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
     from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
-    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_backward, sparse_conv_forward
     paths = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
     assert len(paths) >= 4
     for path in paths:
@@ -206,6 +206,11 @@ def test_golden_fixtures_on_gpu():
         out = sparse_conv_forward(torch.as_tensor(g["features"], device=DEV),
                                   torch.as_tensor(g["weight"], device=DEV), km, len(g["out_coords"]))
         assert rel_err(out.cpu().numpy(), g["out_features_f64"]) <= 1e-5, path
+        gx, gw = sparse_conv_backward(torch.as_tensor(g["grad_out"], device=DEV),
+                                      torch.as_tensor(g["features"], device=DEV),
+                                      torch.as_tensor(g["weight"], device=DEV), km)
+        assert rel_err(gx.cpu().numpy(), g["grad_features_f64"]) <= 1e-5, path
+        assert rel_err(gw.cpu().numpy(), g["grad_weight_f64"]) <= 1e-5, path
 
 
 def test_maps_over_one_tensor_share_its_table(oracle):

@@ -1,26 +1,30 @@
-// Feature contraction of the sparse convolution forward (gfx950, MFMA).
+// Feature contraction of the sparse convolution (gfx950, MFMA): forward product and, through the
+// same kernels, the input gradient.
 //
 //   out[m, :] = bias + sum_k sum_{p in offset k, out_maps[p] == m} X[in_maps[p], :] @ W[k]
 //
-// Output-stationary, atomic-free, accumulators in registers.  A workgroup of four waves owns 256
-// consecutive output rows x 64 output channels; each wave keeps the fp32 accumulators of its 64
-// rows in MFMA result layout for the whole kernel, so the result is bitwise reproducible.
+// Output-stationary, atomic-free, fp32 accumulators in registers in MFMA result layout for the
+// whole kernel, one rounding at the end: the result is bitwise reproducible.
 //
 // The map is consumed as the reference's pair lists, which ascend in output row inside every
-// offset: the pairs of one offset that touch the workgroup's rows are one contiguous run, found
-// with the group_start table (pairs of offset k below output row 64 * g).
+// offset: the pairs of one offset that touch a tile's rows are one contiguous run, found with the
+// group_start table (pairs of offset k below output row 64 * g).  Lists that do not ascend (the
+// exchanged lists of a transposed convolution or of an input gradient) are first re-ordered
+// inside the workspace (rows_* kernels below).
 //
-// The loop over offsets is cut into batches (up to 4 offsets, up to 128 pairs; the pairs of one
-// offset may continue in the next batch).  The batches run as a software pipeline: while batch b
-// is multiplied, the gathered input rows and the W[k]^T tiles of batch b + 1 are in flight into
-// registers and the pairs of batch b + 2 are being read, so no global load is waited for right
-// after it is issued.  Per batch every thread fetches at most one pair, the pairs become slots of
-// the gathered-row buffer, and a slot table maps (offset of the batch, output row) to its slot.
-// In the multiply, lane l of a 16-row block reads the gathered row of output row (l & 15) through
-// the slot table, or a row of zeros if that output row has no pair for this offset, so the
-// product lands in the accumulator rows directly (v_mfma_f32_16x16x32_{f16,bf16},
-// v_mfma_f32_16x16x4_f32).  16-row blocks without any pair skip their MFMAs.  One rounding to the
-// feature dtype when the tile is written.
+// Two kernels:
+//   conv_fwd_ring  feature rows that are whole 16-byte vectors (every case the Python entry points
+//                  produce): rows, weight tiles and pairs go from memory straight into LDS rings,
+//                  eight waves in two roles; described where it is defined.
+//   conv_fwd       any channel count: a workgroup of four waves owns 256 output rows x 64 output
+//                  channels; the offsets are cut into batches (up to 4 offsets, up to 128 pairs)
+//                  that run as a software pipeline through registers: while batch b is multiplied,
+//                  the gathered rows and W[k]^T tiles of batch b + 1 are in flight and the pairs
+//                  of batch b + 2 are being read.
+// In both, lane l of a 16-row block reads the gathered row of output row (l & 15) through a slot
+// table, or a row of zeros if that output row has no pair for the offset, so the product lands in
+// the accumulator rows directly (v_mfma_f32_16x16x32_{f16,bf16}, v_mfma_f32_16x16x4_f32); 16-row
+// blocks without any pair skip their MFMAs.
 //
 // Compulsory HBM bytes: every gathered input row once (L * C_in * s; revisits are served by the
 // L2 / Infinity Cache when the voxel order has locality), the map once (8 L), the output once
