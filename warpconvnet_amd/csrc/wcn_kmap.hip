@@ -141,7 +141,7 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
                                                        int32_t* __restrict__ groups, int64_t G,
                                                        KmapProbe o) {
   constexpr int K = KX * KY * KZ;
-  static_assert(K <= 32 && KX <= 5 && KY <= 5 && KZ <= 5, "fixed kernel covers small kernels");
+  static_assert(KX <= 5 && KY <= 5 && KZ <= 5, "a kernel of up to five voxels spans at most two blocks per dimension");
   __shared__ unsigned long long s_mask[8][256];
   __shared__ int32_t s_base[8][256];
   const int tid = threadIdx.x;
@@ -213,45 +213,54 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
   }
   // no barrier: every thread reads back only its own column
 
-  uint32_t hm = 0;
-  int32_t pos[K];
-  {
-    int k = 0;
+  // Offsets are handled NI planes (values of the slowest kernel index) at a time: all of a small
+  // kernel at once, one plane of KY x KZ offsets at a time for 4x4x4 and 5x5x5 (the per-offset
+  // positions and rows live in registers).
+  constexpr int NI = K <= 32 ? KX : 1, PER = NI * KY * KZ;
+  static_assert(PER <= 32, "one plane fits a 32-bit hit mask");
+  int group_hits = 0;
+#pragma nounroll
+  for (int i0 = 0; i0 < KX; i0 += NI) {
+    uint32_t hm = 0;
+    int32_t pos[PER];
+    {
+      int q = 0;
 #pragma unroll
-    for (int i = 0; i < KX; ++i) {
+      for (int di = 0; di < NI; ++di) {
 #pragma unroll
-      for (int j = 0; j < KY; ++j) {
+        for (int j = 0; j < KY; ++j) {
 #pragma unroll
-        for (int kk = 0; kk < KZ; ++kk, ++k) {
-          const uint32_t ax = (r0[0] & 3u) + i, ay = (r0[1] & 3u) + j, az = (r0[2] & 3u) + kk;
-          const int e = (int)(((ax >> 2) << 2) | ((ay >> 2) << 1) | (az >> 2));
-          const uint32_t bit = ((ax & 3u) << 4) | ((ay & 3u) << 2) | (az & 3u);
-          const unsigned long long mk = s_mask[e][tid];
-          const uint32_t hit = (uint32_t)((mk >> bit) & 1ull);
-          hm |= hit << k;
-          pos[k] = s_base[e][tid] + wcn_rank_below(mk, bit);
+          for (int kk = 0; kk < KZ; ++kk, ++q) {
+            const uint32_t ax = (r0[0] & 3u) + (uint32_t)(i0 + di), ay = (r0[1] & 3u) + j, az = (r0[2] & 3u) + kk;
+            const int e = (int)(((ax >> 2) << 2) | ((ay >> 2) << 1) | (az >> 2));
+            const uint32_t bit = ((ax & 3u) << 4) | ((ay & 3u) << 2) | (az & 3u);
+            const unsigned long long mk = s_mask[e][tid];
+            const uint32_t hit = (uint32_t)((mk >> bit) & 1ull);
+            hm |= hit << q;
+            pos[q] = s_base[e][tid] + wcn_rank_below(mk, bit);
+          }
         }
       }
     }
-  }
 
-  int32_t found[K];
+    int32_t found[PER];
 #pragma unroll
-  for (int k = 0; k < K; ++k) found[k] = ((hm >> k) & 1u) ? perm[pos[k]] : -1;
+    for (int q = 0; q < PER; ++q) found[q] = ((hm >> q) & 1u) ? perm[pos[q]] : -1;
 
-  int group_hits = 0;
 #pragma unroll
-  for (int k = 0; k < K; ++k) {
-    const bool hit = (hm >> k) & 1u;
-    const unsigned long long hits = __ballot(hit);
-    const int cnt = __popcll(hits);
-    group_hits += cnt;
-    if (lane == 0) {
-      groups[(int64_t)k * (G + 1) + group] = cnt;
-      o.hits[group * K + k] = hits;
+    for (int q = 0; q < PER; ++q) {
+      const int k = i0 * KY * KZ + q;
+      const bool hit = (hm >> q) & 1u;
+      const unsigned long long hits = __ballot(hit);
+      const int cnt = __popcll(hits);
+      group_hits += cnt;
+      if (lane == 0) {
+        groups[(int64_t)k * (G + 1) + group] = cnt;
+        o.hits[group * K + k] = hits;
+      }
+      if (hit)  // hits of a group are parked contiguously, in lane order
+        o.found[(int64_t)k * (G * 64) + group * 64 + __popcll(hits & ((1ull << lane) - 1ull))] = found[q];
     }
-    if (hit)  // hits of a group are parked contiguously, in lane order
-      o.found[(int64_t)k * (G * 64) + group * 64 + __popcll(hits & ((1ull << lane) - 1ull))] = found[k];
   }
   if (lane == 0) groups[(int64_t)K * (G + 1) + group] = group_hits;
 }
@@ -415,6 +424,9 @@ void launch_probe(const WcnTableView& v, const int32_t* out_coords, int64_t num_
                        v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G, o);
   } else if (is_fixed_size(g, 2, 2, 2)) {
     hipLaunchKernelGGL((kmap_pass_fixed<2, 2, 2>), grid, block, 0, s, v.hdr, v.slots, cap_mask,
+                       v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G, o);
+  } else if (is_fixed_size(g, 5, 5, 5)) {
+    hipLaunchKernelGGL((kmap_pass_fixed<5, 5, 5>), grid, block, 0, s, v.hdr, v.slots, cap_mask,
                        v.perm, (const int4*)out_coords, num_out, g, w.groups, w.G, o);
   } else {
     hipLaunchKernelGGL(kmap_pass, grid, block, 0, s, v.hdr, v.slots, cap_mask, v.perm,
