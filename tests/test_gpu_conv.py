@@ -232,3 +232,48 @@ def test_c_abi_with_rows_that_are_not_16_byte_vectors(oracle, dtype, c_in, c_out
                                 stream_ptr(torch.device(DEV))), "wcn_sparse_conv_fwd")
     want = oracle.explicit_conv_f64(x.double().numpy(), w.double().numpy(), im, om, off, iden, n)
     assert rel_err(out.float().cpu().numpy(), want) <= TOL[dtype]
+
+
+def test_two_dimensional_convolution(oracle):
+    """SparseConv2d on (N, 2) coordinates, forward and gradients: the device kernels run it as a
+    3-D problem with a size-1 third dimension; the oracle sees the same rows with z = 0."""
+    from oracle.explicit_conv import explicit_gemm_backward
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    from warpconvnet_amd.nn.modules.sparse_conv import SparseConv2d
+    rng = np.random.default_rng(7)
+    xy = np.unique(rng.integers(-40, 40, size=(5000, 2)), axis=0).astype(np.int32)
+    rng.shuffle(xy)
+    n = len(xy)
+    offsets = torch.tensor([0, n // 3, n])
+    x = normal_features(n, 16, seed=4)
+    torch.manual_seed(1)
+    down = SparseConv2d(16, 24, 3, stride=2, bias=False).to(DEV)
+    same = SparseConv2d(16, 24, 3, bias=False).to(DEV)
+    xd = x.to(DEV).requires_grad_(True)
+    vox = Voxels(torch.as_tensor(xy, device=DEV), xd, offsets=offsets)
+    batch = np.repeat([0, 1], [n // 3, n - n // 3]).astype(np.int32)
+    bc = np.concatenate([batch[:, None], xy, np.zeros((n, 1), np.int32)], axis=1)
+
+    y = same(vox)
+    assert y.coordinate_tensor.shape == (n, 2)
+    im, om, off, iden = oracle.kernel_map(bc, bc, (3, 3, 1))
+    w = same.weight.detach().cpu()
+    want = oracle.explicit_conv_f64(x.double().numpy(), w.double().numpy(), im, om, off, iden, n)
+    assert rel_err(y.feature_tensor.detach().cpu().numpy(), want) <= 1e-5
+    gy = normal_features(n, 24, seed=5)
+    y.feature_tensor.backward(gy.to(DEV))
+    want_x, want_w = explicit_gemm_backward(gy.double(), x.double(), w.double(), torch.as_tensor(im),
+                                            torch.as_tensor(om), off, iden)
+    assert rel_err(xd.grad.cpu().numpy(), want_x.numpy()) <= 1e-5
+    assert rel_err(same.weight.grad.cpu().numpy(), want_w.numpy()) <= 1e-5
+
+    z = down(vox)
+    out_bc = z.batch_indexed_coordinates.cpu().numpy()
+    assert out_bc.shape[1] == 3 and z.tensor_stride == (2, 2)
+    out4 = np.concatenate([out_bc, np.zeros((len(out_bc), 1), np.int32)], axis=1)
+    want_set, _, _ = oracle.stride_coords(bc, (2, 2, 1), 2)
+    assert np.array_equal(out4[np.lexsort(out4.T[::-1])], want_set[np.lexsort(want_set.T[::-1])])
+    im, om, off, iden = oracle.kernel_map(bc, out4, (3, 3, 1), (2, 2, 1))
+    want = oracle.explicit_conv_f64(x.double().numpy(), down.weight.detach().double().cpu().numpy(), im, om,
+                                    off, iden, len(out4))
+    assert rel_err(z.feature_tensor.detach().cpu().numpy(), want) <= 1e-5
