@@ -146,6 +146,14 @@ def secondary_configs(dev, steps, warmup):
     up = IntSearchResult(km.out_maps, km.in_maps, km.offsets)
     up._in_ascend, up._in_group_start = km._out_ascend, km._group_start
     t_up, _ = timed(lambda: sparse_conv_forward(y, wu, up, n))
+    # a consumer of the same strided map: 2x2x2 stride-2 max pooling of 64 fp16 channels
+    from warpconvnet_amd.nn.functional.sparse_pool import _SparsePoolFunction
+    xp = torch.randn(n, 64, generator=torch.Generator().manual_seed(6)).to(torch.float16).to(dev)
+    t_pool, _ = timed(lambda: _SparsePoolFunction.apply(xp, km, m, 2))
+    pool_bytes = 2 * 64 * (n + m) + 4 * (n + m)
+    out["max pooling 2x2x2 s2 over the configs[2] map, 64 channels fp16 (warm map)"] = {
+        "num_voxels": n, "num_coarse": m, "call_ms": t_pool,
+        "algorithmic_GBps": pool_bytes / (t_pool * 1e-3) / 1e9}
     out["configs[2]: 2x2x2 s2 96->128 + transposed 128->96 bf16, 1M fine voxels"] = {
         "num_voxels": n, "num_coarse": m, "num_pairs": int(km.offsets[-1]),
         "coords_and_kernel_map_build_ms": t_map, "down_contraction_call_ms": t_down,

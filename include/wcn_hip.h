@@ -213,6 +213,39 @@ int wcn_sparse_conv_wgrad(const void* features, int64_t num_in, int32_t c_in, co
                           int32_t weight_dtype, void* workspace, size_t workspace_bytes,
                           void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Pooling over a kernel map.  Replaces the torch sort + torch_scatter.segment_csr reduction of
+ * sparse_reduce (warpconvnet/nn/functional/sparse_pool.py:84-104, ops/reductions.py:38-56) and
+ * its autograd:
+ *
+ *   out[m, :] = reduce over the pairs p with out_maps[p] == m of X[in_maps[p], :]
+ *
+ * mode 0 = sum, 1 = mean, 2 = max, 3 = min; output rows without pairs become 0.  fp32
+ * accumulation, one rounding.  The pairs are first grouped by row: wcn_map_rows_build(gathered_rows = in_maps,
+ * grouping_rows = out_maps, ..., num_rows = M) for the forward pass, and with the two lists
+ * exchanged (num_rows = N) for the gradient, each into a workspace of
+ * wcn_map_rows_workspace_bytes(num_rows, K, L) bytes that the pooling calls then read.
+ * For max / min, argmax (M, C) int32 receives the input row that supplied each extremum (-1 where
+ * there is none) and must be passed to the gradient.  rows_by_out may be NULL in the gradient of
+ * sum, max and min.
+ * ------------------------------------------------------------------------------------------- */
+
+size_t wcn_map_rows_workspace_bytes(int64_t num_rows, int32_t num_offsets, int64_t num_pairs);
+
+int wcn_map_rows_build(const int32_t* gathered_rows, const int32_t* grouping_rows,
+                       const int64_t* host_offsets, int32_t num_offsets, int64_t num_rows,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+int wcn_sparse_pool_fwd(const void* features, int64_t num_in, int32_t channels, int32_t dtype,
+                        const void* rows_by_out, int64_t num_out, int32_t num_offsets,
+                        int64_t num_pairs, int32_t mode, void* out, int32_t* argmax_or_null,
+                        void* stream);
+
+int wcn_sparse_pool_bwd(const void* grad_out, int64_t num_out, int32_t channels, int32_t dtype,
+                        const void* rows_by_in, const void* rows_by_out, int64_t num_in,
+                        int32_t num_offsets, int64_t num_pairs, int32_t mode,
+                        const int32_t* argmax_or_null, void* grad_in, void* stream);
+
 /* Measurement hook (no counterpart in the reference, which times whole calls with CUDA events:
  * warpconvnet/utils/timer.py:41-60).  The two hipEvent_t handles are recorded on the call's
  * stream immediately before and after the contraction kernel of the NEXT wcn_sparse_conv_fwd

@@ -278,3 +278,43 @@ def test_backward_restatement_equals_autograd_of_the_forward(oracle, case):
     assert (got_x - want_x).abs().max() < 1e-10
     assert (got_w - want_w).abs().max() < 1e-10
     assert want_w.abs().max() > 0 and want_x.abs().max() > 0
+
+
+# ---- pooling over a kernel map ----------------------------------------------------------------
+
+def test_pool_dense_cube_equals_torch_pooling(oracle):
+    """kernel = stride = 2 over a full 8^3 cube: the sparse pooling of the voxel list is
+    max_pool3d / avg_pool3d of the dense tensor."""
+    from oracle.pool import pool_over_map
+    S, C = 8, 5
+    g = torch.Generator().manual_seed(2)
+    dense = torch.randn(1, C, S, S, S, generator=g, dtype=torch.float64)
+    grid = torch.stack(torch.meshgrid(torch.arange(S), torch.arange(S), torch.arange(S), indexing="ij"), -1)
+    xyz = grid.reshape(-1, 3)[torch.randperm(S**3, generator=g)]
+    coords = np.concatenate([np.zeros((S**3, 1), np.int32), xyz.numpy().astype(np.int32)], 1)
+    feats = dense[0, :, xyz[:, 0], xyz[:, 1], xyz[:, 2]].T.contiguous()
+    coarse = oracle.stride_coords(coords, (2, 2, 2), 1)[0]
+    im, om, off, _ = oracle.kernel_map(coords, coarse, (2, 2, 2), (2, 2, 2))
+    cx, cy, cz = coarse[:, 1], coarse[:, 2], coarse[:, 3]
+    for name, fn in (("max", torch.nn.functional.max_pool3d), ("mean", torch.nn.functional.avg_pool3d)):
+        got = pool_over_map(feats, torch.as_tensor(im), torch.as_tensor(om), len(coarse), name)
+        want = fn(dense, 2)[0][:, cx, cy, cz].T
+        assert (got - want).abs().max() < 1e-12, name
+
+
+def test_pool_equals_row_by_row_brute_force(oracle):
+    from oracle.pool import pool_over_map
+    coords = synthetic.random_cloud(31, 400, 9, batch_size=2)
+    coarse = oracle.stride_coords(coords, (2, 2, 2), 2)[0]
+    im, om, off, _ = oracle.kernel_map(coords, coarse, (3, 3, 3), (2, 2, 2))  # overlapping windows
+    x = torch.randn(len(coords), 3, generator=torch.Generator().manual_seed(4), dtype=torch.float64)
+    rows = [[] for _ in range(len(coarse))]
+    for i, m in zip(im, om):
+        rows[m].append(int(i))
+    assert any(len(r) > 4 for r in rows)
+    ops = {"sum": lambda t: t.sum(0), "mean": lambda t: t.mean(0), "max": lambda t: t.max(0).values,
+           "min": lambda t: t.min(0).values}
+    for name, op in ops.items():
+        want = torch.stack([op(x[r]) if r else torch.zeros(3, dtype=torch.float64) for r in rows])
+        got = pool_over_map(x, torch.as_tensor(im), torch.as_tensor(om), len(coarse), name)
+        assert (got - want).abs().max() < 1e-12, name

@@ -39,6 +39,12 @@ SIGNATURES = {
                                            _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
     "wcn_sparse_conv_dgrad": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                              _i64p, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
+    "wcn_map_rows_workspace_bytes": (_sz, [_i64, _i32, _i64]),
+    "wcn_map_rows_build": (ctypes.c_int, [_vp, _vp, _i64p, _i32, _i64, _vp, _sz, _vp]),
+    "wcn_sparse_pool_fwd": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i64, _i32, _i64, _i32, _vp,
+                                           _vp, _vp]),
+    "wcn_sparse_pool_bwd": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, _i64, _i32, _i64, _i32,
+                                           _vp, _vp, _vp]),
     "wcn_conv_wgrad_workspace_bytes": (_sz, [_i32, _i32, _i32, _i64, _i64]),
     "wcn_sparse_conv_wgrad": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i32, _i32, _vp, _vp, _i64p,
                                              _i32, _i32, _vp, _i32, _vp, _sz, _vp]),

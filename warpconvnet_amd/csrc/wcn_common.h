@@ -181,6 +181,26 @@ __device__ __forceinline__ int wcn_wave_inclusive_sum(int v) {
 // and one event per host thread, created on first use and kept until the process ends.
 int wcn_read_small(void* host_dst, const void* device_src, size_t bytes, hipStream_t stream);
 
+// Output-row form of a pair list (rows of the map grouped by output row, inside a row ascending
+// in kernel offset): row_mask[m] has bit k set if offset k has a pair for output row m,
+// row_in[row_ptr[m] .. row_ptr[m + 1]) are the input rows of those pairs.  Built by
+// wcn_rows_build (wcn_conv.hip) inside a caller-provided workspace; used by the contraction to
+// re-order lists that do not ascend and by the pooling kernels.
+struct WcnRowsView {
+  int64_t* offsets;    // K + 1, device copy of the host offsets
+  uint32_t* row_mask;  // num_out * words
+  int32_t* row_ptr;    // num_out + 1
+  int32_t* row_in;     // pairs
+  int32_t* groups;     // G + 1 (scan scratch)
+  int64_t* row_total;  // 1 (scan scratch)
+  int32_t words;       // ceil(K / 32)
+  int64_t G;           // ceil(num_out / 64)
+};
+size_t wcn_rows_layout(void* base, int64_t num_out, int num_offsets, int64_t pairs, WcnRowsView* v);
+// `v.offsets` must already hold the offsets; pairs whose output row is out of range are dropped.
+int wcn_rows_build(const int32_t* in_maps, const int32_t* out_maps, int num_offsets, int64_t num_out,
+                   int64_t pairs, const WcnRowsView& v, hipStream_t stream);
+
 #ifdef __HIPCC__
 
 #define WCN_LAUNCH_CHECK()                      \

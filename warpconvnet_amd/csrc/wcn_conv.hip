@@ -1145,6 +1145,52 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
 
 }  // namespace
 
+size_t wcn_rows_layout(void* base, int64_t num_out, int num_offsets, int64_t pairs, WcnRowsView* v) {
+  char* p = (char*)base;
+  size_t off = 0;
+  const int64_t G = (num_out + 63) / 64;
+  const int words = (num_offsets + 31) / 32;
+  if (v) v->offsets = (int64_t*)(p + off);
+  off += wcn_align256(sizeof(int64_t) * (size_t)(num_offsets + 1));
+  if (v) v->row_mask = (uint32_t*)(p + off);
+  off += wcn_align256(sizeof(uint32_t) * (size_t)num_out * words);
+  if (v) v->row_ptr = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)(num_out + 1));
+  if (v) v->row_in = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)pairs);
+  if (v) v->groups = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)(G + 1));
+  if (v) v->row_total = (int64_t*)(p + off);
+  off += 256;
+  if (v) {
+    v->words = words;
+    v->G = G;
+  }
+  return off;
+}
+
+int wcn_rows_build(const int32_t* in_maps, const int32_t* out_maps, int num_offsets, int64_t num_out,
+                   int64_t pairs, const WcnRowsView& v, hipStream_t s) {
+  const unsigned rows_grid = (unsigned)((num_out + 255) / 256);
+  const int64_t mask_words = num_out * v.words;
+  hipLaunchKernelGGL(rows_clear, dim3((unsigned)std::min<int64_t>(4096, (mask_words + 255) / 256)),
+                     dim3(256), 0, s, v.row_mask, mask_words);
+  if (pairs > 0)
+    hipLaunchKernelGGL(rows_mark, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, s, out_maps,
+                       (const int64_t*)v.offsets, num_offsets, v.words, num_out, v.row_mask);
+  hipLaunchKernelGGL(rows_count<false>, dim3(rows_grid), dim3(256), 0, s,
+                     (const uint32_t*)v.row_mask, v.words, num_out, v.groups, v.row_ptr);
+  wcn_scan_rows_launch(v.groups, v.G, 1, v.row_total, s);
+  hipLaunchKernelGGL(rows_count<true>, dim3(rows_grid), dim3(256), 0, s,
+                     (const uint32_t*)v.row_mask, v.words, num_out, v.groups, v.row_ptr);
+  if (pairs > 0)
+    hipLaunchKernelGGL(rows_fill, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, s, in_maps,
+                       out_maps, (const int64_t*)v.offsets, num_offsets, v.words, num_out,
+                       (const uint32_t*)v.row_mask, (const int32_t*)v.row_ptr, v.row_in);
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
 extern "C" {
 
 int wcn_conv_set_timing_events(void* start_event, void* stop_event) {

@@ -1,0 +1,291 @@
+// Pooling over a kernel map (gfx950): every output row is the sum / mean / maximum of the input
+// rows its pairs name (reference: warpconvnet/nn/functional/sparse_pool.py:25-120, which sorts
+// the pairs by output row with torch and reduces the segments with torch_scatter.segment_csr).
+//
+// The pairs are first put in output-row form (wcn_rows_build: row_ptr / row_in, the kernels the
+// contraction uses to re-order lists), then one thread per (output row, 16 bytes of channels)
+// walks the row's input rows with fp32 accumulators and writes its piece once: no atomics, every
+// feature row read in whole 16-byte pieces, the output written once.  HBM-bound:
+// s * C * (L + M) + 4 (L + M) bytes.
+//
+// The gradient runs the same walk over the map with in and out exchanged: the gradient of an
+// input row is the sum over its pairs of the output row's gradient (divided by the output row's
+// pair count for the mean; only where the input row was the maximum for max).
+#include <algorithm>
+
+#include "wcn_common.h"
+#include "wcn_mma.h"
+
+namespace {
+
+using namespace wcn_mma;
+
+enum { POOL_SUM = 0, POOL_MEAN = 1, POOL_MAX = 2, POOL_MIN = 3 };
+
+template <typename T>
+struct Piece {  // 16 bytes of channels
+  static constexpr int N = 16 / sizeof(T);
+  T v[N];
+};
+
+// One 16-byte piece of row `row`, channels c0 .. c0 + N - 1 (zeros past the last channel; rows
+// whose byte length is not a multiple of 16 are read element by element).
+template <typename T>
+__device__ __forceinline__ void load_piece(const T* __restrict__ base, int64_t row, int channels, int c0,
+                                           bool vec, float* out) {
+  constexpr int N = Piece<T>::N;
+  const T* src = base + row * channels + c0;
+  if (vec) {
+    const u32x4 raw = *reinterpret_cast<const u32x4*>(src);
+    const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int j = 0; j < N; ++j) out[j] = to_float(e[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) out[j] = c0 + j < channels ? to_float(src[j]) : 0.f;
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void store_piece(T* __restrict__ base, int64_t row, int channels, int c0,
+                                            bool vec, const float* val) {
+  constexpr int N = Piece<T>::N;
+  T* dst = base + row * channels + c0;
+  if (vec) {
+    Piece<T> p;
+#pragma unroll
+    for (int j = 0; j < N; ++j) p.v[j] = from_float<T>(val[j]);
+    *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(&p);
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+      if (c0 + j < channels) dst[j] = from_float<T>(val[j]);
+  }
+}
+
+// out[m] = reduce over row_in[row_ptr[m] .. row_ptr[m+1]) of X[.]; rows without pairs become 0
+// (sparse_pool.py:92-104).  For the maximum / minimum, arg[m][c] is the input row that supplied it
+// (the first one in the row's order among equals), -1 for rows without pairs.
+template <typename T>
+__global__ void __launch_bounds__(256) pool_fwd(const T* __restrict__ X, int64_t num_in, int channels,
+                                                const int32_t* __restrict__ row_ptr,
+                                                const int32_t* __restrict__ row_in, int64_t num_out,
+                                                int mode, bool vec, T* __restrict__ out,
+                                                int32_t* __restrict__ arg) {
+  constexpr int N = Piece<T>::N;
+  const int pieces = (channels + N - 1) / N;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= num_out * pieces) return;
+  const int64_t m = i / pieces;
+  const int c0 = (int)(i % pieces) * N;
+  const int begin = row_ptr[m], end = row_ptr[m + 1];
+  float acc[N];
+  int32_t who[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    acc[j] = 0.f;
+    who[j] = -1;
+  }
+  for (int e = begin; e < end; ++e) {
+    const int32_t r = row_in[e];
+    if ((uint32_t)r >= (uint64_t)num_in) continue;
+    float x[N];
+    load_piece<T>(X, r, channels, c0, vec, x);
+    if (mode >= POOL_MAX) {
+      const float sign = mode == POOL_MAX ? 1.f : -1.f;  // the minimum is the maximum of -x
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        const bool better = who[j] < 0 || sign * x[j] > sign * acc[j];
+        acc[j] = better ? x[j] : acc[j];
+        who[j] = better ? r : who[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) acc[j] += x[j];
+    }
+  }
+  if (mode == POOL_MEAN && end > begin) {
+    const float inv = 1.f / (float)(end - begin);
+#pragma unroll
+    for (int j = 0; j < N; ++j) acc[j] *= inv;
+  }
+  store_piece<T>(out, m, channels, c0, vec, acc);
+  if (mode >= POOL_MAX && arg) {
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+      if (c0 + j < channels) arg[m * channels + c0 + j] = who[j];
+  }
+}
+
+// dX[n] = sum over the pairs (n, m) of input row n of dY[m] (sum), dY[m] / count[m] (mean), or
+// dY[m] where arg[m][c] == n (max).  `row_ptr` / `row_in` are the rows form of the exchanged map
+// (rows = input rows, entries = output rows); out_ptr is the row_ptr of the forward rows form
+// (pair count of every output row), used by the mean.
+template <typename T>
+__global__ void __launch_bounds__(256) pool_bwd(const T* __restrict__ dY, int64_t num_out, int channels,
+                                                const int32_t* __restrict__ row_ptr,
+                                                const int32_t* __restrict__ row_in, int64_t num_in,
+                                                int mode, bool vec, const int32_t* __restrict__ out_ptr,
+                                                const int32_t* __restrict__ arg, T* __restrict__ dX) {
+  constexpr int N = Piece<T>::N;
+  const int pieces = (channels + N - 1) / N;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= num_in * pieces) return;
+  const int64_t n = i / pieces;
+  const int c0 = (int)(i % pieces) * N;
+  float acc[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) acc[j] = 0.f;
+  for (int e = row_ptr[n]; e < row_ptr[n + 1]; ++e) {
+    const int32_t m = row_in[e];
+    if ((uint32_t)m >= (uint64_t)num_out) continue;
+    float g[N];
+    load_piece<T>(dY, m, channels, c0, vec, g);
+    if (mode == POOL_MEAN) {
+      const int cnt = out_ptr[m + 1] - out_ptr[m];
+      const float inv = cnt > 0 ? 1.f / (float)cnt : 0.f;
+#pragma unroll
+      for (int j = 0; j < N; ++j) acc[j] += g[j] * inv;
+    } else if (mode >= POOL_MAX) {
+#pragma unroll
+      for (int j = 0; j < N; ++j)
+        if (c0 + j < channels && arg[(int64_t)m * channels + c0 + j] == (int32_t)n) acc[j] += g[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) acc[j] += g[j];
+    }
+  }
+  store_piece<T>(dX, n, channels, c0, vec, acc);
+}
+
+inline bool rows_are_vectors(const void* p, int channels, int dtype) {
+  const size_t es = dtype == WCN_DTYPE_F32 ? 4 : 2;
+  return ((size_t)channels * es) % 16 == 0 && ((uintptr_t)p % 16) == 0;
+}
+
+template <typename T>
+void launch_pool_fwd(const void* X, int64_t num_in, int channels, const WcnRowsView& v, int64_t num_out,
+                     int mode, bool vec, void* out, int32_t* arg, hipStream_t s) {
+  const int pieces = (channels + Piece<T>::N - 1) / Piece<T>::N;
+  const int64_t items = num_out * pieces;
+  hipLaunchKernelGGL(pool_fwd<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, (const T*)X,
+                     num_in, channels, (const int32_t*)v.row_ptr, (const int32_t*)v.row_in, num_out, mode,
+                     vec, (T*)out, arg);
+}
+
+template <typename T>
+void launch_pool_bwd(const void* dY, int64_t num_out, int channels, const WcnRowsView& v, int64_t num_in,
+                     int mode, bool vec, const int32_t* out_ptr, const int32_t* arg, void* dX,
+                     hipStream_t s) {
+  const int pieces = (channels + Piece<T>::N - 1) / Piece<T>::N;
+  const int64_t items = num_in * pieces;
+  hipLaunchKernelGGL(pool_bwd<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, (const T*)dY,
+                     num_out, channels, (const int32_t*)v.row_ptr, (const int32_t*)v.row_in, num_in, mode,
+                     vec, out_ptr, arg, (T*)dX);
+}
+
+bool map_args_ok(const int64_t* host_offsets, int K, const int32_t* in_maps, const int32_t* out_maps,
+                 int64_t* pairs) {
+  if (!host_offsets || K < 1 || K > WCN_MAX_OFFSETS || host_offsets[0] != 0) return false;
+  for (int k = 0; k < K; ++k)
+    if (host_offsets[k + 1] < host_offsets[k]) return false;
+  *pairs = host_offsets[K];
+  if (*pairs > INT32_MAX) return false;
+  return *pairs == 0 || (in_maps && out_maps);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t wcn_map_rows_workspace_bytes(int64_t num_rows, int32_t num_offsets, int64_t num_pairs) {
+  if (num_rows < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || num_pairs < 0) return 0;
+  return wcn_rows_layout(nullptr, num_rows, num_offsets, num_pairs, nullptr);
+}
+
+int wcn_map_rows_build(const int32_t* gathered_rows, const int32_t* grouping_rows,
+                       const int64_t* host_offsets, int32_t num_offsets, int64_t num_rows,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+  int64_t pairs = 0;
+  if (!map_args_ok(host_offsets, num_offsets, gathered_rows, grouping_rows, &pairs) || num_rows < 0 ||
+      num_rows >= (1ll << 31) || !workspace)
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (workspace_bytes < wcn_map_rows_workspace_bytes(num_rows, num_offsets, pairs))
+    return WCN_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  WcnRowsView v;
+  wcn_rows_layout(workspace, num_rows, num_offsets, pairs, &v);
+  if (hipMemcpyAsync(v.offsets, host_offsets, sizeof(int64_t) * (size_t)(num_offsets + 1),
+                     hipMemcpyHostToDevice, s) != hipSuccess)
+    return WCN_ERR_LAUNCH;
+  if (num_rows == 0) return WCN_OK;
+  return wcn_rows_build(gathered_rows, grouping_rows, num_offsets, num_rows, pairs, v, s);
+}
+
+int wcn_sparse_pool_fwd(const void* features, int64_t num_in, int32_t channels, int32_t dtype,
+                        const void* rows_by_out, int64_t num_out, int32_t num_offsets,
+                        int64_t num_pairs, int32_t mode, void* out, int32_t* argmax_or_null,
+                        void* stream) {
+  if (dtype < 0 || dtype > 2 || mode < POOL_SUM || mode > POOL_MIN || channels < 1 || num_in < 0 ||
+      num_out < 0 || num_pairs < 0 || !rows_by_out || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS)
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (num_out == 0) return WCN_OK;
+  if (!out || (num_in > 0 && !features)) return WCN_ERR_INVALID_ARGUMENT;
+  WcnRowsView v;
+  wcn_rows_layout(const_cast<void*>(rows_by_out), num_out, num_offsets, num_pairs, &v);
+  const bool vec = rows_are_vectors(features, channels, dtype) && rows_are_vectors(out, channels, dtype);
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case WCN_DTYPE_F32:
+      launch_pool_fwd<float>(features, num_in, channels, v, num_out, mode, vec, out, argmax_or_null, s);
+      break;
+    case WCN_DTYPE_F16:
+      launch_pool_fwd<_Float16>(features, num_in, channels, v, num_out, mode, vec, out, argmax_or_null, s);
+      break;
+    default:
+      launch_pool_fwd<__bf16>(features, num_in, channels, v, num_out, mode, vec, out, argmax_or_null, s);
+      break;
+  }
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+int wcn_sparse_pool_bwd(const void* grad_out, int64_t num_out, int32_t channels, int32_t dtype,
+                        const void* rows_by_in, const void* rows_by_out, int64_t num_in,
+                        int32_t num_offsets, int64_t num_pairs, int32_t mode,
+                        const int32_t* argmax_or_null, void* grad_in, void* stream) {
+  if (dtype < 0 || dtype > 2 || mode < POOL_SUM || mode > POOL_MIN || channels < 1 || num_in < 0 ||
+      num_out < 0 || num_pairs < 0 || !rows_by_in || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS)
+    return WCN_ERR_INVALID_ARGUMENT;
+  if ((mode >= POOL_MAX && !argmax_or_null) || (mode == POOL_MEAN && !rows_by_out))
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (num_in == 0) return WCN_OK;
+  if (!grad_in || (num_out > 0 && !grad_out)) return WCN_ERR_INVALID_ARGUMENT;
+  WcnRowsView v, vo;
+  wcn_rows_layout(const_cast<void*>(rows_by_in), num_in, num_offsets, num_pairs, &v);
+  const int32_t* out_ptr = nullptr;
+  if (rows_by_out) {
+    wcn_rows_layout(const_cast<void*>(rows_by_out), num_out, num_offsets, num_pairs, &vo);
+    out_ptr = vo.row_ptr;
+  }
+  const bool vec = rows_are_vectors(grad_out, channels, dtype) && rows_are_vectors(grad_in, channels, dtype);
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case WCN_DTYPE_F32:
+      launch_pool_bwd<float>(grad_out, num_out, channels, v, num_in, mode, vec, out_ptr, argmax_or_null,
+                             grad_in, s);
+      break;
+    case WCN_DTYPE_F16:
+      launch_pool_bwd<_Float16>(grad_out, num_out, channels, v, num_in, mode, vec, out_ptr,
+                                argmax_or_null, grad_in, s);
+      break;
+    default:
+      launch_pool_bwd<__bf16>(grad_out, num_out, channels, v, num_in, mode, vec, out_ptr, argmax_or_null,
+                              grad_in, s);
+      break;
+  }
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+}  // extern "C"
