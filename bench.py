@@ -146,6 +146,18 @@ def secondary_configs(dev, steps, warmup):
     up = IntSearchResult(km.out_maps, km.in_maps, km.offsets)
     up._in_ascend, up._in_group_start = km._out_ascend, km._group_start
     t_up, _ = timed(lambda: sparse_conv_forward(y, wu, up, n))
+    # consumers of the same maps: depthwise 3x3x3 over the 1M-voxel map, 2x2x2 stride-2 max pooling
+    from warpconvnet_amd.nn.functional.sparse_conv_depth import spatially_sparse_depthwise_conv
+    km3 = generate_kernel_map(c, c, (1, 1, 1), (3, 3, 3))
+    xdw = torch.randn(n, 64, generator=torch.Generator().manual_seed(7)).to(torch.float16).to(dev)
+    wdw = (torch.randn(27, 64, generator=torch.Generator().manual_seed(8)) * 0.2).to(torch.float16).to(dev)
+    with torch.no_grad():
+        t_dw, _ = timed(lambda: spatially_sparse_depthwise_conv(xdw, wdw, km3, n))
+    L3 = int(km3.offsets[-1])
+    out["depthwise 3x3x3 over the configs[1] map, 64 channels fp16 (warm map)"] = {
+        "num_voxels": n, "num_pairs": L3, "call_ms": t_dw,
+        "gathered_GBps": 2 * 64 * (L3 + n) / (t_dw * 1e-3) / 1e9}
+    del km3
     # a consumer of the same strided map: 2x2x2 stride-2 max pooling of 64 fp16 channels
     from warpconvnet_amd.nn.functional.sparse_pool import _SparsePoolFunction
     xp = torch.randn(n, 64, generator=torch.Generator().manual_seed(6)).to(torch.float16).to(dev)

@@ -246,6 +246,36 @@ int wcn_sparse_pool_bwd(const void* grad_out, int64_t num_out, int32_t channels,
                         int32_t num_offsets, int64_t num_pairs, int32_t mode,
                         const int32_t* argmax_or_null, void* grad_in, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Depthwise convolution over a kernel map.  Replaces the per-offset loops of
+ * warpconvnet/nn/functional/sparse_conv_depth.py:151-231 (explicit) / :233-345 (implicit, native
+ * _C.fma.implicit_fma / implicit_reduction calls):
+ *
+ *   out[m, c]         = sum_k sum_{pairs p of offset k with out_maps[p] == m} X[in_maps[p], c] * W[k, c]
+ *   grad_in[n, c]     = the same over the exchanged map with grad_out in place of X
+ *   grad_weight[k, c] = sum_{pairs p of offset k} X[in_maps[p], c] * grad_out[out_maps[p], c]
+ *
+ * weight is (K, C) in the feature dtype or fp32.  identity_offset >= 0: that offset is taken over
+ * the rows m < min(N, M) with in = out = m and its pairs are ignored (sparse_conv_depth.py:163-165).
+ * Forward and input gradient read a rows form built by wcn_map_rows_build (by output row, resp.
+ * with the lists exchanged, by input row).
+ * ------------------------------------------------------------------------------------------- */
+
+int wcn_sparse_depthwise_fwd(const void* features, int64_t num_in, int32_t channels, int32_t dtype,
+                             const void* weight, int32_t weight_dtype, const void* rows_by_out,
+                             int64_t num_out, int32_t num_offsets, int64_t num_pairs,
+                             int32_t identity_offset, void* out, void* stream);
+
+size_t wcn_depthwise_wgrad_workspace_bytes(int32_t num_offsets, int32_t channels, int64_t num_pairs,
+                                           int64_t identity_rows);
+
+int wcn_sparse_depthwise_wgrad(const void* features, int64_t num_in, const void* grad_out,
+                               int64_t num_out, int32_t channels, int32_t dtype,
+                               const int32_t* in_maps, const int32_t* out_maps,
+                               const int64_t* host_offsets, int32_t num_offsets,
+                               int32_t identity_offset, void* grad_weight, int32_t weight_dtype,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
 /* Measurement hook (no counterpart in the reference, which times whole calls with CUDA events:
  * warpconvnet/utils/timer.py:41-60).  The two hipEvent_t handles are recorded on the call's
  * stream immediately before and after the contraction kernel of the NEXT wcn_sparse_conv_fwd

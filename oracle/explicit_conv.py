@@ -80,3 +80,30 @@ def explicit_gemm_backward(grad_output: torch.Tensor, in_features: torch.Tensor,
         grad_x[rows_in] += torch.matmul(g, w[k].T)
         grad_w[k] += torch.matmul(x[rows_in].T, g)
     return grad_x.to(in_features.dtype), grad_w.to(weight.dtype)
+
+
+def explicit_depthwise_forward(in_features: torch.Tensor, weight: torch.Tensor, in_maps: torch.Tensor,
+                               out_maps: torch.Tensor, offsets, identity_map_index: Optional[int],
+                               num_out_coords: int,
+                               compute_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Depthwise convolution, weight (K, C), following
+    warpconvnet/nn/functional/sparse_conv_depth.py:151-182 operation by operation:
+        out = X * W[iden]                       if the map carries an identity index, else zeros
+        for k != iden, non-empty, in k order:   out[out_map_k] += X[in_map_k] * W[k]
+    Written with differentiable torch operations: the gradients the parity tests compare against
+    are autograd's.  Pinned in tests/test_oracle_pins.py by conv3d with groups = C on a dense cube."""
+    x = in_features if compute_dtype is None else in_features.to(compute_dtype)
+    w = weight if compute_dtype is None else weight.to(compute_dtype)
+    offs = [int(o) for o in offsets]
+    if identity_map_index is not None:
+        out = x * w[identity_map_index].unsqueeze(0)
+    else:
+        out = torch.zeros(num_out_coords, w.shape[-1], dtype=x.dtype, device=x.device)
+    for k in range(len(offs) - 1):
+        if k == identity_map_index:
+            continue
+        lo, hi = offs[k], offs[k + 1]
+        if hi == lo:
+            continue
+        out = out.index_add(0, out_maps[lo:hi].long(), x[in_maps[lo:hi].long()] * w[k].unsqueeze(0))
+    return out.to(dtype=in_features.dtype)

@@ -318,3 +318,22 @@ def test_pool_equals_row_by_row_brute_force(oracle):
         want = torch.stack([op(x[r]) if r else torch.zeros(3, dtype=torch.float64) for r in rows])
         got = pool_over_map(x, torch.as_tensor(im), torch.as_tensor(om), len(coarse), name)
         assert (got - want).abs().max() < 1e-12, name
+
+
+def test_depthwise_dense_cube_equals_grouped_conv3d(oracle):
+    from oracle.explicit_conv import explicit_depthwise_forward
+    S, C = 6, 5
+    g = torch.Generator().manual_seed(8)
+    dense = torch.randn(1, C, S, S, S, generator=g, dtype=torch.float64)
+    w = torch.randn(27, C, generator=g, dtype=torch.float64)
+    grid = torch.stack(torch.meshgrid(torch.arange(S), torch.arange(S), torch.arange(S), indexing="ij"), -1)
+    xyz = grid.reshape(-1, 3)[torch.randperm(S**3, generator=g)]
+    coords = np.concatenate([np.zeros((S**3, 1), np.int32), xyz.numpy().astype(np.int32)], 1)
+    feats = dense[0, :, xyz[:, 0], xyz[:, 1], xyz[:, 2]].T.contiguous()
+    im, om, off, iden = oracle.kernel_map(coords, coords, (3, 3, 3))
+    w5 = w.reshape(3, 3, 3, C).permute(3, 0, 1, 2).unsqueeze(1).contiguous()  # (C, 1, 3, 3, 3)
+    want = torch.nn.functional.conv3d(dense, w5, padding=1, groups=C)[0][:, xyz[:, 0], xyz[:, 1], xyz[:, 2]].T
+    for use_iden in (iden, None):  # with and without the identity shortcut
+        got = explicit_depthwise_forward(feats, w, torch.as_tensor(im), torch.as_tensor(om), off,
+                                         use_iden, len(coords))
+        assert (got - want).abs().max() < 1e-12
