@@ -41,7 +41,17 @@ _MODE = {REDUCTIONS.SUM: 0, REDUCTIONS.MEAN: 1, REDUCTIONS.MAX: 2, REDUCTIONS.MI
 
 
 def _rows_form(gathered: Tensor, grouping: Tensor, km: IntSearchResult, num_rows: int) -> Tensor:
-    """Workspace holding the pairs grouped by `grouping` row (row_ptr / row_in)."""
+    """Workspace holding the pairs grouped by `grouping` row (row_ptr / row_in).  It depends on
+    the map alone, so it is kept on the map object: the layers and the backward passes that share
+    a map share it."""
+    kept = km.__dict__.setdefault("_rows_forms", {})
+    key = (grouping.data_ptr(), gathered.data_ptr(), num_rows)
+    if key not in kept:
+        kept[key] = _build_rows_form(gathered, grouping, km, num_rows)
+    return kept[key]
+
+
+def _build_rows_form(gathered: Tensor, grouping: Tensor, km: IntSearchResult, num_rows: int) -> Tensor:
     L = lib()
     K = len(km)
     pairs = int(km.offsets[-1])
