@@ -251,3 +251,41 @@ def test_synthetic_scenes_are_seeded_and_unique():
     assert len(np.unique(s, axis=0)) == 3000
     bc = synthetic.batch_indexed([a, s])
     assert bc.shape == (8000, 4) and (np.diff(bc[:, 0]) >= 0).all()
+
+
+def test_voxels_dense_round_trip():
+    """from_dense / to_dense (reference: tests/types/test_voxels.py:241-267 round trip)."""
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    g = torch.Generator().manual_seed(0)
+    dense = torch.randn(2, 3, 5, 6, 4, generator=g)
+    dense = dense * (torch.rand(2, 1, 5, 6, 4, generator=g) < 0.3)  # ~30 % occupied
+    vox = Voxels.from_dense(dense)
+    occupied = int((dense.abs().sum(1) > 0).sum())
+    assert len(vox) == occupied and vox.num_channels == 3 and vox.batch_size == 2
+    assert vox.offsets.tolist() == [0, int((dense[0].abs().sum(0) > 0).sum()), occupied]
+    bc = vox.batch_indexed_coordinates
+    assert torch.equal(dense[bc[:, 0].long(), :, bc[:, 1].long(), bc[:, 2].long(), bc[:, 3].long()],
+                       vox.feature_tensor)
+    # back onto the same grid
+    back = vox.to_dense(channel_dim=1, min_coords=(0, 0, 0), max_coords=(4, 5, 3))
+    assert torch.equal(back, dense)
+    assert torch.equal(vox.to_dense(channel_dim=1, spatial_shape=(5, 6, 4)), dense)
+    # bounding-box form: the grid starts at the minimum coordinate
+    lo = vox.coordinate_tensor.min(0).values.tolist()
+    hi = vox.coordinate_tensor.max(0).values.tolist()
+    box = vox.to_dense(channel_dim=-1)
+    assert box.shape == (2, hi[0] - lo[0] + 1, hi[1] - lo[1] + 1, hi[2] - lo[2] + 1, 3)
+    assert torch.equal(box.movedim(-1, 1), dense[:, :, lo[0]:hi[0] + 1, lo[1]:hi[1] + 1, lo[2]:hi[2] + 1])
+    # a window drops what lies outside
+    win = vox.to_dense(channel_dim=1, min_coords=(1, 1, 1), spatial_shape=(3, 3, 2))
+    assert torch.equal(win, dense[:, :, 1:4, 1:4, 1:3])
+    # dense values read back at a target tensor's coordinates (shifted to its minimum)
+    other = torch.randn(2, 7, 5, 6, 4, generator=g)
+    shifted = torch.zeros_like(other)
+    shifted[:, :, :5 - lo[0], :6 - lo[1], :4 - lo[2]] = other[:, :, lo[0]:, lo[1]:, lo[2]:]
+    picked = Voxels.from_dense(shifted, target_spatial_sparse_tensor=vox)
+    assert torch.equal(picked.feature_tensor,
+                       other[bc[:, 0].long(), :, bc[:, 1].long(), bc[:, 2].long(), bc[:, 3].long()])
+    # two spatial dimensions
+    d2 = torch.randn(1, 2, 4, 4, generator=g) * (torch.rand(1, 1, 4, 4, generator=g) < 0.5)
+    assert torch.equal(Voxels.from_dense(d2).to_dense(spatial_shape=(4, 4)), d2)
