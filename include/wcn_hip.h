@@ -276,6 +276,23 @@ int wcn_sparse_depthwise_wgrad(const void* features, int64_t num_in, const void*
                                int32_t identity_offset, void* grad_weight, int32_t weight_dtype,
                                void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Morton (Z-order) codes of voxel coordinates.  Replaces the CuPy launch of
+ * assign_order_discrete_20bit_kernel_4points (warpconvnet/csrc/morton_code.cu:60-84) behind
+ * morton_code() (geometry/coords/ops/serialization.py:181-254):
+ *
+ *   codes[i] = spread(c[a2] - o[a2]) << 2 | spread(c[a1] - o[a1]) << 1 | spread(c[a0] - o[a0])
+ *
+ * c = the three spatial columns of row i starting at column first_spatial of a (n, columns) int32
+ * array, o = device_origin[3] (the per-column minimum, on the device), (a0, a1, a2) = host_axes
+ * (a permutation of 0, 1, 2: the ordering's axis order), spread() = two zero bits between
+ * consecutive bits, 21 bits kept.
+ * ------------------------------------------------------------------------------------------- */
+
+int wcn_morton_codes(const int32_t* coords, int64_t n, int32_t columns, int32_t first_spatial,
+                     const int32_t* device_origin, const int32_t host_axes[3], int64_t* codes,
+                     void* stream);
+
 /* Measurement hook (no counterpart in the reference, which times whole calls with CUDA events:
  * warpconvnet/utils/timer.py:41-60).  The two hipEvent_t handles are recorded on the call's
  * stream immediately before and after the contraction kernel of the NEXT wcn_sparse_conv_fwd

@@ -236,3 +236,45 @@ def test_maps_over_one_tensor_share_its_table(oracle):
     q = torch.as_tensor(bc[:50], device=DEV)
     q[:, 1] += 3
     assert torch.equal(c._wcn_table[1].search(q).cpu(), torch.arange(50, dtype=torch.int32))
+
+
+def _morton_numpy(xyz, axes):
+    """Bit-by-bit restatement: bit i of the axis in position p goes to bit 3 i + p."""
+    rel = (xyz - xyz.min(0)).astype(np.uint64)
+    code = np.zeros(len(xyz), dtype=np.uint64)
+    for pos, axis in enumerate(axes):
+        for bit in range(21):
+            code |= ((rel[:, axis] >> np.uint64(bit)) & np.uint64(1)) << np.uint64(3 * bit + pos)
+    return code.astype(np.int64)
+
+
+def test_morton_codes_and_sort():
+    """encode / morton_code / Voxels.sort (reference: serialization.py:85-254, voxels.py:246-267):
+    codes against a bit-by-bit restatement for every axis order, the permutation sorts by code
+    inside every batch item, the inverse restores the order, features travel with their voxels."""
+    from warpconvnet_amd.geometry.coords.ops.serialization import (POINT_ORDERING,
+                                                                   POINT_ORDERING_TO_MORTON_PERMUTATIONS,
+                                                                   encode, morton_code)
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    rng = np.random.default_rng(3)
+    xyz = np.unique(rng.integers(-3000, 900_000, size=(20_000, 3)), axis=0).astype(np.int32)
+    rng.shuffle(xyz)
+    dev = torch.as_tensor(xyz, device=DEV)
+    for order, axes in POINT_ORDERING_TO_MORTON_PERMUTATIONS.items():
+        assert np.array_equal(morton_code(dev, order=order).cpu().numpy(), _morton_numpy(xyz, axes)), order
+    n = len(xyz)
+    offsets = torch.tensor([0, n // 4, n // 2, n])
+    res = encode(dev, batch_offsets=offsets, order="morton_xyz", return_perm=True, return_inverse=True)
+    codes, perm = res.codes.cpu().numpy(), res.perm.cpu().numpy()
+    assert np.array_equal(np.sort(perm), np.arange(n))
+    for lo, hi in zip(offsets[:-1].tolist(), offsets[1:].tolist()):
+        seg = perm[lo:hi]
+        assert seg.min() >= lo and seg.max() < hi              # rows stay in their batch item
+        assert (np.diff(codes[seg]) > 0).all()                 # ascending (codes of distinct voxels differ)
+    assert np.array_equal(perm[res.inverse_perm.cpu().numpy()], np.arange(n))
+    feats = torch.arange(n, dtype=torch.float32, device=DEV).unsqueeze(1)
+    vox = Voxels(dev, feats, offsets=offsets)
+    s = vox.sort(POINT_ORDERING.MORTON_XYZ)
+    assert s.ordering == POINT_ORDERING.MORTON_XYZ and s.sort(POINT_ORDERING.MORTON_XYZ) is s
+    assert torch.equal(s.coordinate_tensor, dev[res.perm]) and torch.equal(s.feature_tensor[:, 0].long(), res.perm)
+    assert encode(torch.empty(0, 3, dtype=torch.int32), return_perm=True).perm.numel() == 0

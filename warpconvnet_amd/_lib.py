@@ -50,6 +50,7 @@ SIGNATURES = {
     "wcn_depthwise_wgrad_workspace_bytes": (_sz, [_i32, _i32, _i64, _i64]),
     "wcn_sparse_depthwise_wgrad": (ctypes.c_int, [_vp, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _i64p, _i32,
                                                   _i32, _vp, _i32, _vp, _sz, _vp]),
+    "wcn_morton_codes": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32p, _vp, _vp]),
     "wcn_conv_wgrad_workspace_bytes": (_sz, [_i32, _i32, _i32, _i64, _i64]),
     "wcn_sparse_conv_wgrad": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i32, _i32, _vp, _vp, _i64p,
                                              _i32, _i32, _vp, _i32, _vp, _sz, _vp]),

@@ -28,7 +28,7 @@ def stride_coords(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
     assert len(stride) == num_spatial_dims, \
         (f"Stride must match the number of spatial dimensions. Got {len(stride)} spatial "
          f"dimensions for but coordinates with {num_spatial_dims} spatial dimensions.")
-    if str(getattr(order, "value", order)).lower() != "random":
+    if str(getattr(order, "name", order)).lower() != "random":
         raise NotImplementedError("only the default (unordered) output ordering is built")
     if all(s == 1 for s in stride):
         return batch_indexed_coords, offsets_from_batch_index(batch_indexed_coords[:, 0])

@@ -147,6 +147,23 @@ class Voxels(Geometry):
             dense.view(-1, self.num_channels)[self._flat_index(rows, (self.batch_size, *spatial_shape))] = feats
         return dense if channel_dim == -1 else dense.movedim(-1, channel_dim)
 
+    def sort(self, ordering=None) -> "Voxels":
+        """Rows re-ordered along a Morton curve inside every batch item (voxels.py:246-267)."""
+        from ..coords.ops.serialization import POINT_ORDERING, encode
+        if ordering is None:
+            ordering = POINT_ORDERING.MORTON_XYZ
+        if ordering == self.ordering:
+            return self
+        assert isinstance(self.batched_features, CatFeatures), "Features must be a CatFeatures to sort."
+        result = encode(self.coordinate_tensor, batch_offsets=self.offsets, order=ordering,
+                        return_perm=True)
+        kwargs = self.extra_attributes
+        kwargs["ordering"] = ordering
+        kwargs["code"] = result.codes
+        kwargs.pop("_cache", None)  # kernel maps index rows: they do not survive a re-ordering
+        return self.__class__(IntCoords(self.coordinate_tensor[result.perm], self.offsets),
+                              CatFeatures(self.feature_tensor[result.perm], self.offsets), **kwargs)
+
     def unique(self) -> "Voxels":
         """Drop duplicate voxels, keeping the lowest row of each (voxels.py:278-287)."""
         idx, batch_offsets = voxel_downsample_random_indices(self.coordinate_tensor, self.offsets)

@@ -24,6 +24,7 @@ from torch.autograd import Function
 
 from ..._lib import DTYPE_CODE, check, lib, ptr, require_device, stream_ptr, workspace
 from ...geometry.coords.integer import IntCoords
+from ...geometry.coords.ops.serialization import POINT_ORDERING
 from ...geometry.coords.ops.stride import stride_coords
 from ...geometry.coords.search.cache import IntSearchCache, IntSearchCacheKey
 from ...geometry.coords.search.search_results import IntSearchResult
@@ -51,18 +52,14 @@ class SPARSE_CONV_BWD_ALGO_MODE(enum.Enum):
     AUTO = "auto"
 
 
-class POINT_ORDERING(enum.Enum):
-    RANDOM = "random"
-    MORTON_XYZ = "morton_xyz"
-
-
 def in_coords_of(voxels: Voxels):
     """The cached (N, D+1) batch-indexed rows of a tensor (the same object on every access)."""
     return voxels.batched_coordinates.batch_indexed_coordinates
 
 
 def _is_random_order(order) -> bool:
-    return str(getattr(order, "value", order)).lower() == "random"
+    name = getattr(order, "name", order)
+    return str(name).lower() in ("random", "point_ordering.random")
 
 
 # ------------------------------------------------------------------------------------------------
