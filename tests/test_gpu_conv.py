@@ -277,3 +277,52 @@ def test_two_dimensional_convolution(oracle):
     want = oracle.explicit_conv_f64(x.double().numpy(), down.weight.detach().double().cpu().numpy(), im, om,
                                     off, iden, len(out4))
     assert rel_err(z.feature_tensor.detach().cpu().numpy(), want) <= 1e-5
+
+
+def test_generative_convolution_expands_the_coordinates(oracle):
+    """generative=True: the output voxels are the inputs plus everything a kernel offset reaches
+    (reference: coords/ops/expand.py:17-64, sparse_conv.py:1852-1870), as a set equal to numpy's
+    unique over all shifted rows; features against the oracle over those output rows."""
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    items = [synthetic.random_cloud(120 + b, 1500, 30)[:, 1:] for b in range(2)]
+    bc = synthetic.batch_indexed(items)
+    x = normal_features(len(bc), 16, seed=1)
+    w = kaiming_weight(27, 16, 24, seed=2)
+    out = spatially_sparse_conv(_voxels(items, x), w.to(DEV), 3, generative=True)
+    out_bc = out.batch_indexed_coordinates.cpu().numpy()
+    offs = oracle.kernel_offsets((3, 3, 3))
+    want_set = np.unique((bc[None, :, :] + offs[:, None, :]).reshape(-1, 4), axis=0)
+    assert len(out_bc) == len(want_set) > len(bc)
+    assert np.array_equal(out_bc[np.lexsort(out_bc.T[::-1])], want_set)
+    assert (np.diff(out_bc[:, 0]) >= 0).all()                      # batch items stay contiguous
+    assert out.offsets.tolist() == [0, int((out_bc[:, 0] == 0).sum()), len(out_bc)]
+    want, _ = _oracle_out(oracle, x, w, bc, out_bc, (3, 3, 3), (1, 1, 1))
+    assert rel_err(out.feature_tensor.cpu().numpy(), want) <= 1e-5
+    # strided and generative: the strided voxels are expanded
+    out2 = spatially_sparse_conv(_voxels(items, x), w.to(DEV), 3, stride=2, generative=True)
+    out2_bc = out2.batch_indexed_coordinates.cpu().numpy()
+    coarse = oracle.stride_coords(bc, (2, 2, 2), 2)[0]
+    want_set2 = np.unique((coarse[None, :, :] + offs[:, None, :]).reshape(-1, 4), axis=0)
+    assert np.array_equal(out2_bc[np.lexsort(out2_bc.T[::-1])], want_set2)
+    want2, _ = _oracle_out(oracle, x, w, bc, out2_bc, (3, 3, 3), (2, 2, 2))
+    assert rel_err(out2.feature_tensor.cpu().numpy(), want2) <= 1e-5
+
+
+def test_morton_ordered_output(oracle):
+    """order=MORTON_XYZ: the output rows of a strided convolution are sorted along the curve inside
+    every batch item (sparse_conv.py:1888-1896); features follow their voxels."""
+    from warpconvnet_amd.geometry.coords.ops.serialization import POINT_ORDERING, morton_code
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    items = [synthetic.random_cloud(130 + b, 3000, 30)[:, 1:] for b in range(2)]
+    bc = synthetic.batch_indexed(items)
+    x = normal_features(len(bc), 8, seed=3)
+    w = kaiming_weight(8, 8, 8, seed=4)
+    out = spatially_sparse_conv(_voxels(items, x), w.to(DEV), 2, stride=2, order=POINT_ORDERING.MORTON_XYZ)
+    out_bc = out.batch_indexed_coordinates
+    codes = morton_code(out_bc[:, 1:].contiguous()).cpu().numpy()
+    b = out_bc[:, 0].cpu().numpy()
+    assert (np.diff(b) >= 0).all()
+    for item in (0, 1):
+        assert (np.diff(codes[b == item]) > 0).all()
+    want, _ = _oracle_out(oracle, x, w, bc, out_bc.cpu().numpy(), (2, 2, 2), (2, 2, 2))
+    assert rel_err(out.feature_tensor.cpu().numpy(), want) <= 1e-5

@@ -32,7 +32,19 @@ def stride_coords(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
         raise NotImplementedError("only the default (unordered) output ordering is built")
     if all(s == 1 for s in stride):
         return batch_indexed_coords, offsets_from_batch_index(batch_indexed_coords[:, 0])
+    out, count = unique_floor_div_rows(batch_indexed_coords, stride)
+    unique_coords = out[:count, : num_spatial_dims + 1]
+    if num_spatial_dims != 3:
+        unique_coords = unique_coords.contiguous()
+    return unique_coords, offsets_from_batch_index(unique_coords[:, 0])
+
+
+@torch.no_grad()
+def unique_floor_div_rows(batch_indexed_coords: Tensor, stride: Tuple[int, ...]):
+    """((n, 4) buffer, M): the distinct rows of floor(coords / [1, *stride]) in its first M rows,
+    ascending in the first source row of each (one library call and one host read)."""
     assert batch_indexed_coords.dtype == torch.int32
+    num_spatial_dims = batch_indexed_coords.shape[1] - 1
     device = batch_indexed_coords.device
     coords = _four_columns(batch_indexed_coords)
     n = coords.shape[0]
@@ -53,7 +65,4 @@ def stride_coords(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
             continue
         check(status, "wcn_stride_unique")
         break
-    unique_coords = out[: count.value, : num_spatial_dims + 1]
-    if num_spatial_dims != 3:
-        unique_coords = unique_coords.contiguous()
-    return unique_coords, offsets_from_batch_index(unique_coords[:, 0])
+    return out, int(count.value)

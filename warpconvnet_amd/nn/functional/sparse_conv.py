@@ -24,7 +24,8 @@ from torch.autograd import Function
 
 from ..._lib import DTYPE_CODE, check, lib, ptr, require_device, stream_ptr, workspace
 from ...geometry.coords.integer import IntCoords
-from ...geometry.coords.ops.serialization import POINT_ORDERING
+from ...geometry.coords.ops.expand import expand_coords
+from ...geometry.coords.ops.serialization import POINT_ORDERING, encode
 from ...geometry.coords.ops.stride import stride_coords
 from ...geometry.coords.search.cache import IntSearchCache, IntSearchCacheKey
 from ...geometry.coords.search.search_results import IntSearchResult
@@ -235,21 +236,33 @@ def generate_output_coords_and_kernel_map(
     """Output coordinates (given / strided / same as input), then the kernel map, through the
     cache on the input tensor (reference: sparse_conv.py:1808-1996).  A transposed convolution
     reuses the cached forward map of the matching strided convolution with in/out exchanged."""
-    if generative:
-        raise NotImplementedError("generative convolutions (coordinate expansion) are not built")
     if stride_mode != STRIDED_CONV_MODE.STRIDE_ONLY:
         raise NotImplementedError("only STRIDED_CONV_MODE.STRIDE_ONLY is built")
-    if not _is_random_order(order):
-        raise NotImplementedError("only the default (unordered) output ordering is built")
     in_coords = input_sparse_tensor.batch_indexed_coordinates
 
+    # output coordinates: given, expanded (generative), strided, or the input's (sparse_conv.py:1843-1886)
     if output_spatially_sparse_tensor is not None:
+        assert not generative, \
+            "Output spatially sparse tensor is not supported with generative convolution"
         out_coords = output_spatially_sparse_tensor.batch_indexed_coordinates
         out_offsets = output_spatially_sparse_tensor.offsets
+    elif generative and all(s == 1 for s in stride):
+        assert not transposed, "Transposed and generative convolution is not supported yet"
+        out_coords, out_offsets = expand_coords(in_coords, kernel_size=kernel_size,
+                                                kernel_dilation=kernel_dilation)
     elif any(s != 1 for s in stride):
         out_coords, out_offsets = stride_coords(in_coords, stride)
+        if generative:  # the strided voxels are expanded in addition
+            out_coords, out_offsets = expand_coords(out_coords, kernel_size=kernel_size,
+                                                    kernel_dilation=kernel_dilation)
     else:
         out_coords, out_offsets = in_coords, input_sparse_tensor.offsets
+
+    # optional ordering of the output rows along a space-filling curve (sparse_conv.py:1888-1896)
+    if not _is_random_order(order):
+        code = encode(out_coords[:, 1:].contiguous(), batch_offsets=out_offsets, order=order,
+                      return_perm=True)
+        out_coords = out_coords[code.perm].contiguous()
 
     def make_key(is_transposed, in_off, out_off):
         return IntSearchCacheKey(kernel_size=kernel_size, kernel_dilation=kernel_dilation,
