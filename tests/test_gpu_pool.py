@@ -116,3 +116,30 @@ def test_pool_at_benchmark_size():
                        torch.ones_like(sparse_reduce(vox, 2, 2, "max").feature_tensor))
     counts = sparse_reduce(vox, 2, 2, "sum").feature_tensor
     assert int(counts[:, 0].float().sum()) == n and float(counts.max()) <= 8 and float(counts.min()) >= 1
+
+
+def test_reduce_and_stride_convolution(oracle):
+    """stride_mode=REDUCE_AND_STRIDE: max pooling over stride-sized windows, then the convolution
+    with stride 1 over the pooled voxels (reference: sparse_conv.py:1753-1766)."""
+    from helpers import kaiming_weight
+    from warpconvnet_amd.nn.functional.sparse_conv import STRIDED_CONV_MODE, spatially_sparse_conv
+    from warpconvnet_amd.nn.functional.sparse_pool import sparse_max_pool
+    items = [synthetic.random_cloud(140 + b, 3000, 24)[:, 1:] for b in range(2)]
+    x = normal_features(sum(len(i) for i in items), 16, seed=5)
+    w = kaiming_weight(27, 16, 24, seed=6).to(DEV)
+    fine = _voxels(items, x.to(DEV))
+    got = spatially_sparse_conv(fine, w, 3, stride=2, stride_mode=STRIDED_CONV_MODE.REDUCE_AND_STRIDE)
+    pooled = sparse_max_pool(_voxels(items, x.to(DEV)), 2, 2)
+    want = spatially_sparse_conv(pooled, w, 3)
+    assert got.tensor_stride == (2, 2, 2)
+    assert torch.equal(got.coordinate_tensor, want.coordinate_tensor)
+    assert torch.equal(got.feature_tensor, want.feature_tensor)
+    # and against the oracle chain
+    from oracle.pool import pool_over_map
+    bc = synthetic.batch_indexed(items)
+    pc = pooled.batch_indexed_coordinates.cpu().numpy()
+    im, om, off, _ = oracle.kernel_map(bc, pc, (2, 2, 2), (2, 2, 2))
+    px = pool_over_map(x.double(), torch.as_tensor(im), torch.as_tensor(om), len(pc), "max")
+    im, om, off, iden = oracle.kernel_map(pc, pc, (3, 3, 3))
+    ref = oracle.explicit_conv_f64(px.numpy(), w.double().cpu().numpy(), im, om, off, iden, len(pc))
+    assert rel_err(got.feature_tensor.cpu().numpy(), ref) <= 1e-5

@@ -35,7 +35,7 @@ from ...utils.ntuple import ntuple
 
 
 class STRIDED_CONV_MODE(enum.Enum):
-    REDUCE_AND_STRIDE = "reduce_and_stride"  # pooling before the convolution: not built
+    REDUCE_AND_STRIDE = "reduce_and_stride"  # the input is pooled by the stride, then convolved
     STRIDE_ONLY = "stride_only"
 
 
@@ -236,8 +236,9 @@ def generate_output_coords_and_kernel_map(
     """Output coordinates (given / strided / same as input), then the kernel map, through the
     cache on the input tensor (reference: sparse_conv.py:1808-1996).  A transposed convolution
     reuses the cached forward map of the matching strided convolution with in/out exchanged."""
-    if stride_mode != STRIDED_CONV_MODE.STRIDE_ONLY:
-        raise NotImplementedError("only STRIDED_CONV_MODE.STRIDE_ONLY is built")
+    if stride_mode == STRIDED_CONV_MODE.REDUCE_AND_STRIDE and any(s != 1 for s in stride):
+        raise ValueError("REDUCE_AND_STRIDE reaches the map builder with stride 1 (the functional "
+                         "entry point pools the input by the stride first)")
     in_coords = input_sparse_tensor.batch_indexed_coordinates
 
     # output coordinates: given, expanded (generative), strided, or the input's (sparse_conv.py:1843-1886)
@@ -361,6 +362,14 @@ def spatially_sparse_conv(
             out_tensor_stride = ntuple(1, ndim=ndim)
         assert any(o < i for o, i in zip(out_tensor_stride, in_tensor_stride)), \
             "Output stride is larger than input stride"
+
+    if stride_mode == STRIDED_CONV_MODE.REDUCE_AND_STRIDE and any(s != 1 for s in _stride):
+        # the input is pooled over stride-sized windows first, the convolution then runs with
+        # stride 1 over the pooled voxels (sparse_conv.py:1753-1766)
+        from .sparse_pool import sparse_reduce
+        input_sparse_tensor = sparse_reduce(input_sparse_tensor, kernel_size=_stride, stride=_stride,
+                                            reduction=stride_reduce)
+        _stride = ntuple(1, ndim=ndim)
 
     features = input_sparse_tensor.feature_tensor
     effective_compute_dtype = compute_dtype if compute_dtype is not None else features.dtype
