@@ -110,9 +110,16 @@ int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_off
  * No counterpart in the reference. */
 int32_t wcn_kmap_last_table_flags(void);
 
+/* in_maps / out_maps have room for pair_capacity pairs.  The pass reads the pair count and the
+ * table status from the workspace itself and writes nothing if there are more pairs than that or
+ * the table reported a problem, so it may be enqueued into buffers of assumed size right after
+ * wcn_kmap_count, before wcn_kmap_read_result has told the host the count (the result's copy to
+ * the host is enqueued by wcn_kmap_count and therefore runs ahead of this pass); the caller then
+ * checks host_offsets[K] <= pair_capacity and calls again with larger buffers if not. */
 int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
                   int64_t num_out, const int32_t host_kernel_size[3], const int32_t host_stride[3],
-                  const void* workspace, int32_t* in_maps, int32_t* out_maps, void* stream);
+                  const void* workspace, int64_t pair_capacity, int32_t* in_maps,
+                  int32_t* out_maps, void* stream);
 
 /* Device address, inside a kmap workspace, of the (K, ceil(num_out/64)+1) int32 table
  * group_start[k][g] = number of pairs of offset k whose output row is below 64*g (valid after

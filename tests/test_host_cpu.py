@@ -64,8 +64,9 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert L.wcn_kmap_count(fake, 10, 1024, fake, 5, three, three, null, null) == -1
     big = (ctypes.c_int32 * 3)(11, 11, 11)                             # 1331 offsets > 1024
     assert L.wcn_kmap_count(fake, 10, 1024, fake, 5, big, three, fake, null) == -1
-    assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, bad, three, fake, fake, fake, null) == -1
-    assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, three, three, fake, null, null, null) == -1
+    assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, bad, three, fake, 100, fake, fake, null) == -1
+    assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, three, three, fake, 100, null, null, null) == -1
+    assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, three, three, fake, -1, fake, fake, null) == -1
     assert L.wcn_stride_unique(fake, 10, bad, fake, 1024, fake, fake, null) == -1
     offs = (ctypes.c_int64 * 28)(*([0] * 28))
 

@@ -180,6 +180,10 @@ __device__ __forceinline__ int wcn_wave_inclusive_sum(int v) {
 // blocking stream synchronisation wakes the host tens of microseconds later).  One staging buffer
 // and one event per host thread, created on first use and kept until the process ends.
 int wcn_read_small(void* host_dst, const void* device_src, size_t bytes, hipStream_t stream);
+// The same read split in two: begin enqueues the copy (before whatever is enqueued next), end waits
+// for it; an end without a matching begin on this thread does the whole read.
+int wcn_read_early_begin(const void* device_src, size_t bytes, hipStream_t stream);
+int wcn_read_early_end(void* host_dst, const void* device_src, size_t bytes, hipStream_t stream);
 
 // Output-row form of a pair list (rows of the map grouped by output row, inside a row ascending
 // in kernel offset): row_mask[m] has bit k set if offset k has a pair for output row m,

@@ -273,12 +273,16 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
                                                  const int32_t* __restrict__ found,
                                                  const int32_t* __restrict__ groups,
                                                  const int64_t* __restrict__ offsets, int K_runtime,
-                                                 int64_t G, int32_t* __restrict__ in_maps,
+                                                 int64_t G, int64_t pair_capacity,
+                                                 int32_t* __restrict__ in_maps,
                                                  int32_t* __restrict__ out_maps) {
   const int K = KFIX > 0 ? KFIX : K_runtime;
   const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t group = m >> 6;  // wave-uniform
   if (group >= G) return;
+  // offsets[K] = number of pairs, offsets[K + 1] = table status bits (written by the scan): the
+  // pass may have been enqueued before the host has seen either, so it checks them itself
+  if (offsets[K] > pair_capacity || offsets[K + 1] != 0) return;
   const int lane = wcn_lane();
   const unsigned long long below = (1ull << lane) - 1ull;
   for (int k0 = 0; k0 < K; k0 += 64) {
@@ -434,19 +438,19 @@ void launch_probe(const WcnTableView& v, const int32_t* out_coords, int64_t num_
   }
 }
 
-void launch_emit(int64_t num_out, const KmapGeom& g, const KmapWorkspace& w, int32_t* in_maps,
-                 int32_t* out_maps, hipStream_t s) {
+void launch_emit(int64_t num_out, const KmapGeom& g, const KmapWorkspace& w, int64_t pair_capacity,
+                 int32_t* in_maps, int32_t* out_maps, hipStream_t s) {
   const dim3 grid(grid_for(num_out, 256)), block(256);
   const int64_t* offsets = (const int64_t*)w.result;
   if (g.K == 27) {
     hipLaunchKernelGGL(kmap_emit<27>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
-                       w.G, in_maps, out_maps);
+                       w.G, pair_capacity, in_maps, out_maps);
   } else if (g.K == 8) {
     hipLaunchKernelGGL(kmap_emit<8>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
-                       w.G, in_maps, out_maps);
+                       w.G, pair_capacity, in_maps, out_maps);
   } else {
     hipLaunchKernelGGL(kmap_emit<0>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
-                       w.G, in_maps, out_maps);
+                       w.G, pair_capacity, in_maps, out_maps);
   }
 }
 
@@ -576,6 +580,9 @@ int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const in
   const KmapFinish fin = {w.result, w.ticket, v.hdr, g.K};
   hipLaunchKernelGGL(kmap_scan_rows, dim3(g.K + 1), dim3(1024), 0, s, w.groups, w.G, w.row_total, fin);
   WCN_LAUNCH_CHECK();
+  // the result's trip to the host starts here, ahead of anything the caller enqueues next (an emit
+  // pass into buffers of assumed size, say); wcn_kmap_read_result collects it
+  if (wcn_read_early_begin(w.result, sizeof(int64_t) * (size_t)(g.K + 3), s) != WCN_OK) return WCN_ERR_LAUNCH;
   return WCN_OK;
 }
 
@@ -589,7 +596,7 @@ int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_off
   kmap_layout(const_cast<void*>(workspace), num_out, num_offsets, &w);
   int64_t tmp[WCN_MAX_OFFSETS + 3];
   const size_t bytes = sizeof(int64_t) * (size_t)(num_offsets + 3);
-  if (wcn_read_small(tmp, w.result, bytes, (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
+  if (wcn_read_early_end(tmp, w.result, bytes, (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
   for (int k = 0; k <= num_offsets; ++k) host_offsets[k] = tmp[k];
   g_last_table_flags = (int32_t)((tmp[num_offsets + 2] >> 32) & 1);
   const int st = wcn_table_status_from_bits((int32_t)tmp[num_offsets + 1]);
@@ -600,19 +607,20 @@ int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_off
 
 int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
                   int64_t num_out, const int32_t host_kernel_size[3], const int32_t host_stride[3],
-                  const void* workspace, int32_t* in_maps, int32_t* out_maps, void* stream) {
+                  const void* workspace, int64_t pair_capacity, int32_t* in_maps, int32_t* out_maps,
+                  void* stream) {
   KmapGeom g;
   if (!make_geom(host_kernel_size, host_stride, &g)) return WCN_ERR_INVALID_ARGUMENT;
   if (!table_args_ok(table, n_keys, capacity) || !workspace || num_out < 0 ||
-      num_out >= (1ll << 31) || (num_out > 0 && !out_coords))
+      num_out >= (1ll << 31) || (num_out > 0 && !out_coords) || pair_capacity < 0)
     return WCN_ERR_INVALID_ARGUMENT;
-  if (num_out == 0) return WCN_OK;
+  if (num_out == 0 || pair_capacity == 0) return WCN_OK;
   if (!in_maps || !out_maps) return WCN_ERR_INVALID_ARGUMENT;
   WcnTableView v;
   wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
   KmapWorkspace w;
   kmap_layout(const_cast<void*>(workspace), num_out, g.K, &w);
-  launch_emit(num_out, g, w, in_maps, out_maps, (hipStream_t)stream);
+  launch_emit(num_out, g, w, pair_capacity, in_maps, out_maps, (hipStream_t)stream);
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }

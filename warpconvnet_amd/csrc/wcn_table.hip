@@ -276,6 +276,58 @@ int wcn_read_small(void* host_dst, const void* device_src, size_t bytes, hipStre
   return WCN_OK;
 }
 
+// A read that is requested where the data is produced and collected later: the copy into the
+// thread's second staging buffer is enqueued at once (so that it runs before whatever the caller
+// enqueues next), the wait happens in wcn_read_early_end.  One pending read per host thread; an
+// end without a matching begin is a plain wcn_read_small.
+namespace {
+constexpr size_t kEarlyStaging = 16384;
+thread_local void* g_early_staging = nullptr;
+thread_local hipEvent_t g_early_done = nullptr;
+thread_local int g_early_device = -1;
+thread_local const void* g_early_src = nullptr;
+thread_local size_t g_early_bytes = 0;
+}  // namespace
+
+int wcn_read_early_begin(const void* device_src, size_t bytes, hipStream_t stream) {
+  g_early_src = nullptr;
+  if (bytes > kEarlyStaging) return WCN_ERR_INVALID_ARGUMENT;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return WCN_ERR_LAUNCH;
+  if (!g_early_staging &&
+      hipHostMalloc(&g_early_staging, kEarlyStaging, hipHostMallocDefault) != hipSuccess) {
+    g_early_staging = nullptr;
+    return WCN_ERR_LAUNCH;
+  }
+  if (!g_early_done || g_early_device != device) {
+    if (g_early_done) (void)hipEventDestroy(g_early_done);
+    if (hipEventCreateWithFlags(&g_early_done, hipEventDisableTiming) != hipSuccess) {
+      g_early_done = nullptr;
+      return WCN_ERR_LAUNCH;
+    }
+    g_early_device = device;
+  }
+  if (hipMemcpyAsync(g_early_staging, device_src, bytes, hipMemcpyDeviceToHost, stream) != hipSuccess)
+    return WCN_ERR_LAUNCH;
+  if (hipEventRecord(g_early_done, stream) != hipSuccess) return WCN_ERR_LAUNCH;
+  g_early_src = device_src;
+  g_early_bytes = bytes;
+  return WCN_OK;
+}
+
+int wcn_read_early_end(void* host_dst, const void* device_src, size_t bytes, hipStream_t stream) {
+  if (g_early_src != device_src || g_early_bytes != bytes)
+    return wcn_read_small(host_dst, device_src, bytes, stream);
+  g_early_src = nullptr;
+  for (;;) {
+    const hipError_t e = hipEventQuery(g_early_done);
+    if (e == hipSuccess) break;
+    if (e != hipErrorNotReady) return WCN_ERR_LAUNCH;
+  }
+  memcpy(host_dst, g_early_staging, bytes);
+  return WCN_OK;
+}
+
 int wcn_table_status_from_bits(int32_t bits) {
   if (bits & WCN_DEV_RANGE) return WCN_ERR_COORD_RANGE;
   if (bits & WCN_DEV_OVERFLOW) return WCN_ERR_TABLE_OVERFLOW;

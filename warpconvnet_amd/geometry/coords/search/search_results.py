@@ -18,7 +18,7 @@ class IntSearchResult:
     def __init__(self, in_maps: Tensor, out_maps: Tensor, offsets: Tensor,
                  identity_map_index: Optional[int] = None):
         offsets = offsets.cpu()
-        assert len(in_maps) == len(out_maps) == int(offsets[-1])
+        assert in_maps.shape[0] == out_maps.shape[0] == int(offsets[-1])
         self.in_maps = in_maps
         self.out_maps = out_maps
         self.offsets = offsets
@@ -33,6 +33,7 @@ class IntSearchResult:
         # convolution: a forward map with its lists exchanged), the group starts that belong to
         # that order, and whether exchanging in and out turns offset k into offset K - 1 - k
         # (stride-1 map of a duplicate-free coordinate set onto itself).
+        self._host_offsets = None  # (K + 1) ctypes int64 array of `offsets`, when the builder left one
         self._in_ascend = False
         self._in_group_start = None
         self._symmetric = False

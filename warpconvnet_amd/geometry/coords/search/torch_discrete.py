@@ -63,10 +63,19 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     M = out4.shape[0]
     ws = workspace(L.wcn_kmap_workspace_bytes(M, K), device)
     host_offsets = (ctypes.c_int64 * (K + 1))()
+    # The pairs are emitted into buffers of assumed size while the pair count is still on its way
+    # to the host (a voxel of a surface-like scene has a handful of neighbours, far from K); the
+    # lists handed out are views of these buffers.  More pairs than assumed: the emit pass has
+    # written nothing and runs again with exact buffers.
+    assumed = min(K * M, max(8 * M, 1 << 16))
+    in_buf = torch.empty(assumed, dtype=torch.int32, device=device)
+    out_buf = torch.empty(assumed, dtype=torch.int32, device=device)
     while True:
         raw, n_keys, slots = table._raw()
         check(L.wcn_kmap_count(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws),
                                stream_ptr(device)), "wcn_kmap_count")
+        check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), assumed,
+                              ptr(in_buf), ptr(out_buf), stream_ptr(device)), "wcn_kmap_fill")
         status = L.wcn_kmap_read_result(ptr(ws), M, K, host_offsets, stream_ptr(device))
         if status == ERR_TABLE_OVERFLOW:
             table._grow()
@@ -75,12 +84,16 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
         table._checked = True
         break
     total = int(host_offsets[K])
-    in_maps = torch.empty(total, dtype=torch.int32, device=device)
-    out_maps = torch.empty(total, dtype=torch.int32, device=device)
-    check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), ptr(in_maps),
-                          ptr(out_maps), stream_ptr(device)), "wcn_kmap_fill")
-    offsets = torch.tensor(list(host_offsets), dtype=torch.int32)
+    if total <= assumed:
+        in_maps, out_maps = in_buf[:total], out_buf[:total]
+    else:
+        in_maps = torch.empty(total, dtype=torch.int32, device=device)
+        out_maps = torch.empty(total, dtype=torch.int32, device=device)
+        check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), total,
+                              ptr(in_maps), ptr(out_maps), stream_ptr(device)), "wcn_kmap_fill")
+    offsets = torch.from_numpy(np.ctypeslib.as_array(host_offsets).astype(np.int32))
     result = IntSearchResult(in_maps, out_maps, offsets, identity_map_index=identity_map_index)
+    result._host_offsets = host_offsets  # the contraction passes them on as they are
     # by-products the contraction reuses: pairs ascend in output row inside every offset, and
     # the workspace (kept alive by the reference below) holds their per-64-row group starts
     result._out_ascend = True

@@ -67,6 +67,15 @@ def _is_random_order(order) -> bool:
 # Feature contraction
 # ------------------------------------------------------------------------------------------------
 
+def _host_offsets_of(km: IntSearchResult):
+    """(K + 1) ctypes int64 array of the map's offsets, made once per map object."""
+    kept = km._host_offsets
+    if kept is None or len(kept) != len(km.offsets):
+        kept = (ctypes.c_int64 * len(km.offsets))(*[int(v) for v in km.offsets.tolist()])
+        km._host_offsets = kept
+    return kept
+
+
 @torch.no_grad()
 def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSearchResult,
                         num_out_coords: int, bias: Optional[Tensor] = None,
@@ -105,11 +114,11 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
     group_start = None
     if ascend and km._group_start is not None and km._group_start[2] == (K, num_out_coords):
         group_start = ctypes.c_void_p(km._group_start[1])
-    num_pairs = int(km.offsets[-1])
+    host_offsets = _host_offsets_of(km)
+    num_pairs = int(host_offsets[K])
     nbytes = L.wcn_conv_workspace_bytes(num_out_coords, K, c_in, c_out, DTYPE_CODE[x.dtype],
                                         num_pairs, ascend)
     ws = workspace(nbytes, device)
-    host_offsets = (ctypes.c_int64 * (K + 1))(*[int(v) for v in km.offsets.tolist()])
     iden = -1 if km.identity_map_index is None else int(km.identity_map_index)
     check(L.wcn_sparse_conv_fwd(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(w),
                                 DTYPE_CODE[w.dtype], K, c_out, ptr(b), ptr(km.in_maps),
@@ -148,8 +157,8 @@ def sparse_conv_backward(grad_output: Tensor, in_features: Tensor, weight: Tenso
     n_in, n_out = x.shape[0], gy.shape[0]
     device = x.device
     L = lib()
-    num_pairs = int(km.offsets[-1])
-    host_offsets = (ctypes.c_int64 * (K + 1))(*[int(v) for v in km.offsets.tolist()])
+    host_offsets = _host_offsets_of(km)
+    num_pairs = int(host_offsets[K])
     iden = -1 if km.identity_map_index is None else int(km.identity_map_index)
     code = DTYPE_CODE[dtype]
     grad_x = grad_w = None
