@@ -342,12 +342,13 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
   int32_t* row = groups + (int64_t)blockIdx.x * (G + 1);
   const int lane = wcn_lane(), wave = threadIdx.x >> 6;
   int64_t carry = 0;
-  for (int64_t start = 0; start < G; start += 4096) {
-    const int64_t idx = start + (int64_t)threadIdx.x * 4;
-    int v[4];
+  constexpr int PER = 4;  // entries per thread and round (one 16-byte load)
+  for (int64_t start = 0; start < G; start += 1024 * PER) {
+    const int64_t idx = start + (int64_t)threadIdx.x * PER;
+    int v[PER];
     int sum = 0;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < PER; ++t) {
       v[t] = idx + t < G ? row[idx + t] : 0;
       sum += v[t];
     }
@@ -363,35 +364,48 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
     }
     int run = (int)carry + before + incl - sum;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < PER; ++t) {
       if (idx + t < G) row[idx + t] = run;
       run += v[t];
     }
     carry += all;
     __syncthreads();
   }
+  __shared__ int s_last;
   if (threadIdx.x == 0) {
     // a row of the per-offset counts holds at most M < 2^31 pairs; the row of all hits can
     // exceed int32, which the host turns into WCN_ERR_TOO_MANY_PAIRS
     row[G] = (int32_t)carry;
     row_total[blockIdx.x] = carry;
+    s_last = 0;
     if (fin.result) {
-      // the workgroup that finishes last turns the row totals into offsets[K+1] and copies the
-      // table's status next to them, so the host needs one read for everything
       __threadfence();
-      if (atomicAdd(fin.ticket, 1) == (int32_t)gridDim.x - 1) {
-        __threadfence();
-        int64_t run = 0;
-        fin.result[0] = 0;
-        for (int k = 0; k < fin.K; ++k) {
-          run += __hip_atomic_load(&row_total[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          fin.result[k + 1] = run;
-        }
-        fin.result[fin.K + 1] = fin.hdr->status;
-        fin.result[fin.K + 2] = (int64_t)fin.hdr->num_blocks | ((int64_t)(fin.hdr->has_duplicates != 0) << 32);
-        *fin.ticket = 0;
-      }
+      s_last = atomicAdd(fin.ticket, 1) == (int32_t)gridDim.x - 1;
     }
+  }
+  __syncthreads();
+  if (!s_last || wave != 0) return;
+  // The workgroup that finishes last turns the row totals into offsets[K+1] and copies the
+  // table's status next to them, so the host needs one read for everything.  Its first wave
+  // fetches 64 totals at a time (independent loads) and scans them.
+  __threadfence();
+  int64_t run = 0;
+  for (int k0 = 0; k0 < fin.K; k0 += 64) {
+    const int k = k0 + lane;
+    int64_t v = k < fin.K ? __hip_atomic_load(&row_total[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int64_t t = __shfl_up(v, d, 64);
+      if (lane >= d) v += t;
+    }
+    if (k < fin.K) fin.result[k + 1] = run + v;
+    run += __shfl(v, 63, 64);
+  }
+  if (lane == 0) {
+    fin.result[0] = 0;
+    fin.result[fin.K + 1] = fin.hdr->status;
+    fin.result[fin.K + 2] = (int64_t)fin.hdr->num_blocks | ((int64_t)(fin.hdr->has_duplicates != 0) << 32);
+    *fin.ticket = 0;
   }
 }
 
