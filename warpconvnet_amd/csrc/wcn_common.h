@@ -33,10 +33,13 @@ struct WcnTableHeader {  // first 256 bytes of a table workspace
   int32_t num_blocks;    // occupied slots
   int32_t status;        // WCN_DEV_* bits
   int32_t total;         // running sum of block populations (ends at the number of distinct keys)
-  int32_t has_duplicates;  // some key was inserted more than once
+  int32_t num_keys;      // keys inserted; more keys than set bits (`total`) means some key came twice
   int32_t reserved[52];
 };
 static_assert(sizeof(WcnTableHeader) == 256, "header is 256 bytes");
+
+// Valid once the populations have been summed (table_base): every distinct key set one bit.
+#define WCN_HAS_DUPLICATES(hdr) ((hdr)->total != (hdr)->num_keys)
 
 struct WcnTableView {  // host-computed addresses inside a table workspace
   WcnTableHeader* hdr;

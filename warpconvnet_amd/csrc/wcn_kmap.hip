@@ -404,7 +404,7 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
   if (lane == 0) {
     fin.result[0] = 0;
     fin.result[fin.K + 1] = fin.hdr->status;
-    fin.result[fin.K + 2] = (int64_t)fin.hdr->num_blocks | ((int64_t)(fin.hdr->has_duplicates != 0) << 32);
+    fin.result[fin.K + 2] = (int64_t)fin.hdr->num_blocks | ((int64_t)(WCN_HAS_DUPLICATES(fin.hdr) ? 1 : 0) << 32);
     *fin.ticket = 0;
   }
 }

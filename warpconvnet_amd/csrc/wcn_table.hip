@@ -28,7 +28,7 @@ __global__ void __launch_bounds__(256) table_clear(WcnTableHeader* __restrict__ 
     hdr->num_blocks = 0;
     hdr->status = 0;
     hdr->total = 0;
-    hdr->has_duplicates = 0;
+    hdr->num_keys = (int32_t)n_keys;
   }
   // each slot is two 16-byte stores: {EMPTY, 0} and {0, 0, 0, 0}
   uint4* raw = reinterpret_cast<uint4*>(slots);
@@ -113,9 +113,10 @@ __global__ void __launch_bounds__(256) table_insert(const int4* __restrict__ key
       if (seen == WCN_EMPTY_KEY) seen = key;  // this thread claimed the slot
     }
     if (seen == key) {
-      // a bit that is already set means the same coordinate was inserted before
+      // the result of the atomic is not used, so it is issued without waiting for a reply;
+      // repeated keys show up later as fewer set bits than keys
       uint32_t* half = reinterpret_cast<uint32_t*>(&slots[h].mask) + (bit_index >> 5);
-      if (atomicOr(half, bit) & bit) hdr->has_duplicates = 1;
+      atomicOr(half, bit);
       placed = (int32_t)h;
       break;
     }
@@ -185,7 +186,7 @@ __global__ void __launch_bounds__(256) table_perm(const int4* __restrict__ keys,
   const int32_t pos = slots[h].base + wcn_rank_below(km.y, wcn_block_bit(r));
   if (pos < 0 || pos >= n_keys) return;
   // without duplicate keys every position has exactly one writer
-  if (hdr->has_duplicates) atomicMin(&perm[pos], (int32_t)i); else perm[pos] = (int32_t)i;
+  if (WCN_HAS_DUPLICATES(hdr)) atomicMin(&perm[pos], (int32_t)i); else perm[pos] = (int32_t)i;
 }
 
 __global__ void __launch_bounds__(256) table_query(const WcnTableHeader* __restrict__ hdr,
