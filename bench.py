@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
 # each scaled by what the same counter reads for the 1 GiB device copy of --calibrate-copy
 # (FETCH_SIZE reads 0.5 GiB for it -> x2.0; WRITE_SIZE reads 1 GiB -> x1.0).  Summary kept in
 # profiles/conv_fwd_cfg2_hbm_traffic.txt; to be re-measured whenever the kernel changes.
-CONV_FWD_TRAFFIC_BYTES = (282586 * 2.0 + 160172 * 1.0) * 1024
+CONV_FWD_TRAFFIC_BYTES = (282610 * 2.0 + 160171 * 1.0) * 1024
 
 METRIC = "voxels/sec, 3x3x3 C64->64 fp16 conv @1M voxels; kernel-map build ms"
 
@@ -372,7 +372,7 @@ def main():
             "contraction_frac_of_mfma_peak": conv_flops / (conv_kernel_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
         },
         "roofline": {
-            "kernel": "conv_fwd_ring<f16, 6>",
+            "kernel": "conv_fwd_ring<f16, 6, false, 0>",
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
