@@ -9,6 +9,7 @@ HBM before the timed region starts.  Prints ONE JSON line.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 """
 import argparse
+import gc
 import ctypes
 import json
 import os
@@ -166,6 +167,37 @@ def secondary_configs(dev, steps, warmup):
     out["max pooling 2x2x2 s2 over the configs[2] map, 64 channels fp16 (warm map)"] = {
         "num_voxels": n, "num_coarse": m, "call_ms": t_pool,
         "algorithmic_GBps": pool_bytes / (t_pool * 1e-3) / 1e9}
+    # the step before the path: 4 x 1M points -> voxels of 2 cm with the mean of 32 fp16 channels,
+    # beside the torch ops the reference composes for it (voxel.py:92-100, unique.py:84-100)
+    from warpconvnet_amd.geometry.coords.ops.voxel import voxel_downsample_csr_mapping
+    from warpconvnet_amd.ops.reductions import segment_reduction
+    gp = torch.Generator(device=dev).manual_seed(7)
+    npts = 4_000_000
+    pts = torch.rand((npts, 3), device=dev, generator=gp) * torch.tensor([8.0, 8.0, 0.1], device=dev)
+    poffsets = torch.tensor([0, 1_000_000, 2_000_000, 3_000_000, npts])
+    pfeat = torch.randn((npts, 32), device=dev, generator=gp).to(torch.float16)
+
+    def voxelize():
+        _, _, ci, co, tu = voxel_downsample_csr_mapping(pts, poffsets, 0.02)
+        return segment_reduction(pfeat, co, "mean", indices=ci, segment_of=tu.to_orig_indices)
+
+    def voxelize_torch_ops():
+        rows = torch.cat([torch.searchsorted(poffsets[1:].to(dev), torch.arange(npts, device=dev),
+                                             right=True).int().unsqueeze(1),
+                          torch.floor(pts / 0.02).int()], dim=1)
+        u, inv, cnt = torch.unique(rows, dim=0, sorted=True, return_inverse=True, return_counts=True)
+        order = inv.argsort(stable=True)
+        sums = torch.zeros((len(u), 32), device=dev).index_add_(0, inv, pfeat.float())
+        return (sums / cnt[:, None]).half(), order
+
+    t_vox, vox = timed(voxelize)
+    t_vox_torch, _ = timed(voxelize_torch_ops)
+    mvox = len(vox)
+    vox_bytes = 12 * npts + 16 * npts + 3 * 8 * npts + 2 * 32 * (npts + mvox) + 8 * npts + 16 * mvox
+    out["points -> voxels: 4 x 1M points, 2 cm voxels, mean of 32 fp16 channels"] = {
+        "num_points": npts, "num_voxels": mvox, "call_ms": t_vox, "points_per_s": npts / (t_vox * 1e-3),
+        "algorithmic_GBps": vox_bytes / (t_vox * 1e-3) / 1e9, "same_result_with_torch_ops_ms": t_vox_torch}
+    del pts, pfeat, vox
     out["configs[2]: 2x2x2 s2 96->128 + transposed 128->96 bf16, 1M fine voxels"] = {
         "num_voxels": n, "num_coarse": m, "num_pairs": int(km.offsets[-1]),
         "coords_and_kernel_map_build_ms": t_map, "down_contraction_call_ms": t_down,
@@ -308,33 +340,51 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
-        km, out, _ = step()
-    torch.cuda.synchronize()
+    def run_steps(count):
+        """`count` steps back to back between two synchronisations; wall time and the events."""
+        kernel_events = []
+        for _ in range(count):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()  # creates the underlying hipEvent_t; re-recorded by the library
+            b.record()
+            kernel_events.append((a, b))
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+        ends = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+        mids = []
+        last = None
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(count):
+            starts[i].record()
+            km, out, mid = step(kernel_events[i])
+            ends[i].record()
+            mids.append(mid)
+            last = (km, out)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, starts, mids, ends, kernel_events, last
 
-    kernel_events = []
-    for _ in range(args.steps):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()  # creates the underlying hipEvent_t; re-recorded by the library
-        b.record()
-        kernel_events.append((a, b))
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    mids = []
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        starts[i].record()
-        km, out, mid = step(kernel_events[i])
-        ends[i].record()
-        mids.append(mid)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    # The warm-up steps go through the very code of the timed ones (events included): the first
+    # pass through it in a process has cost a single stall of tens of milliseconds on a fresh machine.
+    if args.warmup > 0:
+        run_steps(args.warmup)
+    # As timeit does: no collection of the interpreter's garbage inside the timed region (a full
+    # collection of a heap with torch loaded takes tens of milliseconds, dozens of steps).
+    gc.collect()
+    gc.disable()
+    try:
+        elapsed, starts, mids, ends, kernel_events, (km, out) = run_steps(args.steps)
+    finally:
+        gc.enable()
 
     ms_per_step = elapsed * 1e3 / args.steps
     map_ms = float(np.mean([s.elapsed_time(m) for s, m in zip(starts, mids)]))
     conv_call_ms = float(np.mean([m.elapsed_time(e) for m, e in zip(mids, ends)]))
     conv_kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in kernel_events]))
+    if os.environ.get("WCN_BENCH_TRACE"):  # per-step device times, for looking into an odd average
+        for i in range(args.steps):
+            print(f"step {i}: map {starts[i].elapsed_time(mids[i]):.3f} ms, contraction call "
+                  f"{mids[i].elapsed_time(ends[i]):.3f} ms, kernel "
+                  f"{kernel_events[i][0].elapsed_time(kernel_events[i][1]):.3f} ms", file=sys.stderr)
 
     num_pairs = int(km.offsets[-1])
     c_in, c_out, K, s = 64, 64, 27, 2

@@ -300,6 +300,62 @@ int wcn_morton_codes(const int32_t* coords, int64_t n, int32_t columns, int32_t 
                      const int32_t* device_origin, const int32_t host_axes[3], int64_t* codes,
                      void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Voxelisation front-end: points -> voxel rows -> sorted distinct voxels with the CSR grouping of
+ * the points, and reductions over those groups.
+ *
+ * wcn_voxel_rows replaces `torch.floor(batched_points / voxel_size).int()` +
+ * `batch_index_from_offset` + `torch.cat` (warpconvnet/geometry/coords/ops/voxel.py:92-95,136-141):
+ * rows[i] = [batch item of point i, floor(x * r), floor(y * r), floor(z * r)] with
+ * r = (float)(1.0 / voxel_size), which is how torch divides a float tensor by a host scalar on the
+ * device.  points (N, 3) fp32; host_batch_offsets (B + 1) int64 on the host; for more than
+ * WCN_VOXEL_MAX_BATCH batch items the same offsets must also be given in device memory.
+ *
+ * wcn_unique_rows_csr replaces unique_torch (warpconvnet/utils/unique.py:57-109), i.e.
+ * torch.unique(x, dim=0, sorted=True, return_inverse=True, return_counts=True), the stable argsort
+ * of the inverse, the cumulative sum of the counts and the scatter that picks a representative:
+ *   unique_rows (M, columns) int32  distinct rows in ascending lexicographic order
+ *   to_orig     (N) int64           unique_rows[to_orig[i]] == rows[i]
+ *   csr_indices (N) int64           rows grouped by distinct row, ascending row index inside a group
+ *   csr_offsets (M + 1) int64       group u is csr_indices[csr_offsets[u] .. csr_offsets[u + 1])
+ *   to_unique   (M) int64           lowest row index of each group (the reference's choice is whichever
+ *                                   write of a scatter with repeated indices lands last)
+ * Every output may be NULL; output buffers must hold N (N + 1 for csr_offsets) entries, the count M
+ * is returned through *num_unique.  rows (N, columns) int32, 1 <= columns <= 4; the per-column
+ * ranges must pack into 64 bits together (WCN_ERR_COORD_RANGE otherwise).  The call waits for the
+ * stream twice (key width, then M).
+ *
+ * wcn_segment_reduce replaces `row_reduction(features[to_csr_indices], to_csr_offsets, reduction)`
+ * (warpconvnet/ops/reductions.py:36-72, torch_scatter.segment_csr; called from
+ * warpconvnet/nn/functional/point_pool.py:298-302): out[u] = sum / mean / max / min (mode 0..3, as
+ * for wcn_sparse_pool_fwd) over e in [segment_offsets[u], segment_offsets[u + 1]) of
+ * features[indices[e]] (features[e] when indices is NULL); empty segments give 0.  argmax (M, C)
+ * int64 receives the feature row behind each extremum.  wcn_segment_reduce_bwd is its gradient for
+ * disjoint segments: segment_of_row (N) names each feature row's segment (out of range = none).
+ * ------------------------------------------------------------------------------------------- */
+
+#define WCN_VOXEL_MAX_BATCH 64
+
+int wcn_voxel_rows(const float* points, int64_t num_points, const int64_t* host_batch_offsets,
+                   const int64_t* device_batch_offsets_or_null, int32_t batch_size, double voxel_size,
+                   int32_t* rows, void* stream);
+
+size_t wcn_unique_rows_workspace_bytes(int64_t num_rows);
+
+int wcn_unique_rows_csr(const int32_t* rows, int64_t num_rows, int32_t columns, void* workspace,
+                        size_t workspace_bytes, int32_t* unique_rows, int64_t* to_orig,
+                        int64_t* csr_indices, int64_t* csr_offsets, int64_t* to_unique,
+                        int64_t* num_unique, void* stream);
+
+int wcn_segment_reduce(const void* features, int64_t num_in, int32_t channels, int32_t dtype,
+                       const int64_t* segment_offsets, const int64_t* indices_or_null,
+                       int64_t num_segments, int32_t mode, void* out, int64_t* argmax_or_null,
+                       void* stream);
+
+int wcn_segment_reduce_bwd(const void* grad_out, int64_t num_segments, int32_t channels, int32_t dtype,
+                           const int64_t* segment_offsets, const int64_t* segment_of_row, int64_t num_in,
+                           int32_t mode, const int64_t* argmax_or_null, void* grad_in, void* stream);
+
 /* Measurement hook (no counterpart in the reference, which times whole calls with CUDA events:
  * warpconvnet/utils/timer.py:41-60).  The two hipEvent_t handles are recorded on the call's
  * stream immediately before and after the contraction kernel of the NEXT wcn_sparse_conv_fwd

@@ -337,3 +337,93 @@ def test_depthwise_dense_cube_equals_grouped_conv3d(oracle):
         got = explicit_depthwise_forward(feats, w, torch.as_tensor(im), torch.as_tensor(om), off,
                                          use_iden, len(coords))
         assert (got - want).abs().max() < 1e-12
+
+
+# ---- point -> voxel front-end (oracle/voxelize.py) ------------------------------------------------
+def _cloud_points(seed, n, batch, extent=1.0):
+    rng = np.random.default_rng(seed)
+    sizes = rng.multinomial(n - batch, np.ones(batch) / batch) + 1
+    offsets = np.concatenate([[0], np.cumsum(sizes)])
+    pts = ((rng.random((n, 3)) - 0.3) * extent).astype(np.float32)  # negative coordinates included
+    return pts, offsets
+
+
+def test_voxelize_equals_dictionary_brute_force():
+    from oracle import voxelize
+    pts, offsets = _cloud_points(5, 700, 3)
+    feats = np.random.default_rng(6).standard_normal((700, 5))
+    vs = 0.26
+    rows = voxelize.voxel_rows(pts, offsets, vs)
+    # the rows themselves: python floats, one point at a time
+    inv = float(np.float32(1.0 / vs))
+    for i in (0, 1, 350, 699):
+        b = int(np.searchsorted(offsets, i, side="right") - 1)
+        cell = [int(np.floor(np.float32(np.float32(v) * np.float32(inv)))) for v in pts[i]]
+        assert rows[i].tolist() == [b] + cell
+    groups = {}
+    for i, r in enumerate(map(tuple, rows.tolist())):
+        groups.setdefault(r, []).append(i)
+    keys = sorted(groups)  # tuples compare lexicographically
+    assert any(len(g) > 3 for g in groups.values()) and len(keys) > 100
+    unique, to_orig, csr_indices, csr_offsets, to_unique = voxelize.unique_rows_csr(rows)
+    assert unique.tolist() == [list(k) for k in keys]
+    assert csr_indices.tolist() == [i for k in keys for i in groups[k]]
+    assert csr_offsets.tolist() == [0] + list(np.cumsum([len(groups[k]) for k in keys]))
+    assert to_unique.tolist() == [groups[k][0] for k in keys]
+    assert all(keys[to_orig[i]] == tuple(rows[i]) for i in range(len(rows)))
+    ops = {"sum": lambda a: a.sum(0), "mean": lambda a: a.mean(0), "max": lambda a: a.max(0),
+           "min": lambda a: a.min(0)}
+    for name, op in ops.items():
+        want = np.stack([op(feats[groups[k]]) for k in keys])
+        got = voxelize.segment_reduce(feats, csr_offsets, name, indices=csr_indices)
+        assert np.abs(got - want).max() < 1e-12, name
+    coords, vfeats, voffsets = voxelize.points_to_voxels(pts, feats, offsets, vs, "mean")
+    assert coords.tolist() == [list(k[1:]) for k in keys]
+    assert voffsets.tolist() == [sum(k[0] < b for k in keys) for b in range(4)]
+    assert np.abs(vfeats - np.stack([feats[groups[k]].mean(0) for k in keys])).max() < 1e-12
+
+
+def test_voxelize_lattice_closed_form():
+    """c copies (jittered inside the cell) of every cell centre of an S^3 lattice, shuffled: S^3
+    voxels in lexicographic order, c points each, mean feature = the cell's own value."""
+    from oracle import voxelize
+    S, c, vs = 5, 3, 0.25
+    rng = np.random.default_rng(9)
+    cells = np.stack(np.meshgrid(np.arange(S), np.arange(S), np.arange(S), indexing="ij"), -1).reshape(-1, 3) - 2
+    cell_of_point = np.repeat(np.arange(S**3), c)
+    rng.shuffle(cell_of_point)
+    pts = ((cells[cell_of_point] + 0.5 + (rng.random((S**3 * c, 3)) - 0.5) * 0.8) * vs).astype(np.float32)
+    value = rng.standard_normal((S**3, 2))
+    feats = value[cell_of_point]
+    coords, vfeats, voffsets = voxelize.points_to_voxels(pts, feats, [0, len(pts)], vs, "mean")
+    assert coords.tolist() == cells.tolist()  # meshgrid 'ij' order is the lexicographic order
+    assert voffsets.tolist() == [0, S**3]
+    assert np.abs(vfeats - value).max() < 1e-12
+    summed = voxelize.points_to_voxels(pts, feats, [0, len(pts)], vs, "sum")[1]
+    assert np.abs(summed - c * value).max() < 1e-12
+
+
+def test_unique_identities_of_the_reference_test():
+    """tests/test_unique.py:21-35 of the reference: x == unique[to_orig] and x[csr_indices] sorted."""
+    from oracle import voxelize
+    x = np.random.default_rng(0).integers(0, 5, (10, 1))
+    unique, to_orig, csr_indices, csr_offsets, to_unique = voxelize.unique_rows_csr(x)
+    assert (unique[to_orig] == x).all()
+    assert (np.sort(x[csr_indices], axis=0) == x[csr_indices]).all()
+    assert (x[to_unique] == unique).all()
+    assert np.diff(csr_offsets).sum() == len(x)
+
+
+def test_device_division_differs_from_true_division_only_at_cell_borders():
+    from oracle import voxelize
+    rng = np.random.default_rng(3)
+    vs = 0.02
+    k = rng.integers(-2000, 2000, (4000, 3))
+    on_border = (k * np.float32(vs)).astype(np.float32)  # products rounded to float: within an ulp of a border
+    a = voxelize.voxel_rows(on_border, [0, 4000], vs, device_division=True)
+    b = voxelize.voxel_rows(on_border, [0, 4000], vs, device_division=False)
+    assert np.abs(a - b).max() == 1 and (a != b).any()
+    inside = ((k + 0.5) * vs).astype(np.float32)
+    a = voxelize.voxel_rows(inside, [0, 4000], vs, device_division=True)
+    b = voxelize.voxel_rows(inside, [0, 4000], vs, device_division=False)
+    assert (a == b).all() and (a[:, 1:] == k).all()

@@ -158,6 +158,104 @@ __global__ void __launch_bounds__(256) pool_bwd(const T* __restrict__ dY, int64_
   store_piece<T>(dX, n, channels, c0, vec, acc);
 }
 
+// ---- reduction over CSR segments (the point -> voxel pooling) -----------------------------------
+//
+//   out[u] = reduce over e in [offsets[u], offsets[u+1]) of X[indices ? indices[e] : e]
+//
+// (reference: warpconvnet/ops/reductions.py:36-72, torch_scatter.segment_csr over features that
+// were gathered with features[to_csr_indices] first; here the gather is part of the walk, so the
+// gathered copy is never written).  Offsets and indices are 64-bit, as torch.unique and argsort
+// return them.  arg[u][c] = the input row that supplied the extremum.
+template <typename T>
+__global__ void __launch_bounds__(256) segment_reduce(const T* __restrict__ X, int64_t num_in, int channels,
+                                                      const int64_t* __restrict__ offsets,
+                                                      const int64_t* __restrict__ indices,
+                                                      int64_t num_out, int mode, bool vec,
+                                                      T* __restrict__ out, int64_t* __restrict__ arg) {
+  constexpr int N = Piece<T>::N;
+  const int pieces = (channels + N - 1) / N;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= num_out * pieces) return;
+  const int64_t u = i / pieces;
+  const int c0 = (int)(i % pieces) * N;
+  const int64_t begin = offsets[u], end = offsets[u + 1];
+  float acc[N];
+  int64_t who[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    acc[j] = 0.f;
+    who[j] = -1;
+  }
+  for (int64_t e = begin; e < end; ++e) {
+    const int64_t r = indices ? indices[e] : e;
+    if ((uint64_t)r >= (uint64_t)num_in) continue;
+    float x[N];
+    load_piece<T>(X, r, channels, c0, vec, x);
+    if (mode >= POOL_MAX) {
+      const float sign = mode == POOL_MAX ? 1.f : -1.f;
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        const bool better = who[j] < 0 || sign * x[j] > sign * acc[j];
+        acc[j] = better ? x[j] : acc[j];
+        who[j] = better ? r : who[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) acc[j] += x[j];
+    }
+  }
+  if (mode == POOL_MEAN && end > begin) {
+    const float inv = 1.f / (float)(end - begin);
+#pragma unroll
+    for (int j = 0; j < N; ++j) acc[j] *= inv;
+  }
+  store_piece<T>(out, u, channels, c0, vec, acc);
+  if (mode >= POOL_MAX && arg) {
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+      if (c0 + j < channels) arg[u * channels + c0 + j] = who[j];
+  }
+}
+
+// Every input row lies in at most one segment: dX[n] = dY[u] (sum), dY[u] / count[u] (mean),
+// dY[u] where arg[u][c] == n (max, min), with u = segment_of[n]; 0 for rows outside every segment.
+template <typename T>
+__global__ void __launch_bounds__(256) segment_reduce_bwd(const T* __restrict__ dY, int64_t num_out,
+                                                          int channels, const int64_t* __restrict__ offsets,
+                                                          const int64_t* __restrict__ segment_of,
+                                                          int64_t num_in, int mode, bool vec,
+                                                          const int64_t* __restrict__ arg,
+                                                          T* __restrict__ dX) {
+  constexpr int N = Piece<T>::N;
+  const int pieces = (channels + N - 1) / N;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= num_in * pieces) return;
+  const int64_t n = i / pieces;
+  const int c0 = (int)(i % pieces) * N;
+  float acc[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) acc[j] = 0.f;
+  const int64_t u = segment_of[n];
+  if ((uint64_t)u < (uint64_t)num_out) {
+    float g[N];
+    load_piece<T>(dY, u, channels, c0, vec, g);
+    if (mode == POOL_MEAN) {
+      const int64_t cnt = offsets[u + 1] - offsets[u];
+      const float inv = cnt > 0 ? 1.f / (float)cnt : 0.f;
+#pragma unroll
+      for (int j = 0; j < N; ++j) acc[j] = g[j] * inv;
+    } else if (mode >= POOL_MAX) {
+#pragma unroll
+      for (int j = 0; j < N; ++j)
+        if (c0 + j < channels && arg[u * channels + c0 + j] == n) acc[j] = g[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) acc[j] = g[j];
+    }
+  }
+  store_piece<T>(dX, n, channels, c0, vec, acc);
+}
+
 // ---- depthwise convolution over the same rows form ---------------------------------------------
 //
 //   out[m][c] = sum over the pairs (n, m) of offset k of X[n][c] * W[k][c]
@@ -319,6 +417,26 @@ void launch_pool_bwd(const void* dY, int64_t num_out, int channels, const WcnRow
                      vec, out_ptr, arg, (T*)dX);
 }
 
+template <typename T>
+void launch_segment_reduce(const void* X, int64_t num_in, int channels, const int64_t* offsets,
+                           const int64_t* indices, int64_t num_out, int mode, bool vec, void* out,
+                           int64_t* arg, hipStream_t s) {
+  const int pieces = (channels + Piece<T>::N - 1) / Piece<T>::N;
+  const int64_t items = num_out * pieces;
+  hipLaunchKernelGGL(segment_reduce<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
+                     (const T*)X, num_in, channels, offsets, indices, num_out, mode, vec, (T*)out, arg);
+}
+
+template <typename T>
+void launch_segment_reduce_bwd(const void* dY, int64_t num_out, int channels, const int64_t* offsets,
+                               const int64_t* segment_of, int64_t num_in, int mode, bool vec,
+                               const int64_t* arg, void* dX, hipStream_t s) {
+  const int pieces = (channels + Piece<T>::N - 1) / Piece<T>::N;
+  const int64_t items = num_in * pieces;
+  hipLaunchKernelGGL(segment_reduce_bwd<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
+                     (const T*)dY, num_out, channels, offsets, segment_of, num_in, mode, vec, arg, (T*)dX);
+}
+
 bool map_args_ok(const int64_t* host_offsets, int K, const int32_t* in_maps, const int32_t* out_maps,
                  int64_t* pairs) {
   if (!host_offsets || K < 1 || K > WCN_MAX_OFFSETS || host_offsets[0] != 0) return false;
@@ -417,6 +535,65 @@ int wcn_sparse_pool_bwd(const void* grad_out, int64_t num_out, int32_t channels,
     default:
       launch_pool_bwd<__bf16>(grad_out, num_out, channels, v, num_in, mode, vec, out_ptr, argmax_or_null,
                               grad_in, s);
+      break;
+  }
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+int wcn_segment_reduce(const void* features, int64_t num_in, int32_t channels, int32_t dtype,
+                       const int64_t* segment_offsets, const int64_t* indices_or_null,
+                       int64_t num_segments, int32_t mode, void* out, int64_t* argmax_or_null,
+                       void* stream) {
+  if (dtype < 0 || dtype > 2 || mode < POOL_SUM || mode > POOL_MIN || channels < 1 || num_in < 0 ||
+      num_segments < 0 || channels > (1 << 20))
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (num_segments == 0) return WCN_OK;
+  if (!out || !segment_offsets || (num_in > 0 && !features)) return WCN_ERR_INVALID_ARGUMENT;
+  const bool vec = rows_are_vectors(features, channels, dtype) && rows_are_vectors(out, channels, dtype);
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case WCN_DTYPE_F32:
+      launch_segment_reduce<float>(features, num_in, channels, segment_offsets, indices_or_null,
+                                   num_segments, mode, vec, out, argmax_or_null, s);
+      break;
+    case WCN_DTYPE_F16:
+      launch_segment_reduce<_Float16>(features, num_in, channels, segment_offsets, indices_or_null,
+                                      num_segments, mode, vec, out, argmax_or_null, s);
+      break;
+    default:
+      launch_segment_reduce<__bf16>(features, num_in, channels, segment_offsets, indices_or_null,
+                                    num_segments, mode, vec, out, argmax_or_null, s);
+      break;
+  }
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+int wcn_segment_reduce_bwd(const void* grad_out, int64_t num_segments, int32_t channels, int32_t dtype,
+                           const int64_t* segment_offsets, const int64_t* segment_of_row, int64_t num_in,
+                           int32_t mode, const int64_t* argmax_or_null, void* grad_in, void* stream) {
+  if (dtype < 0 || dtype > 2 || mode < POOL_SUM || mode > POOL_MIN || channels < 1 || num_in < 0 ||
+      num_segments < 0 || channels > (1 << 20))
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (mode >= POOL_MAX && !argmax_or_null) return WCN_ERR_INVALID_ARGUMENT;
+  if (num_in == 0) return WCN_OK;
+  if (!grad_in || !segment_of_row || !segment_offsets || (num_segments > 0 && !grad_out))
+    return WCN_ERR_INVALID_ARGUMENT;
+  const bool vec = rows_are_vectors(grad_out, channels, dtype) && rows_are_vectors(grad_in, channels, dtype);
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case WCN_DTYPE_F32:
+      launch_segment_reduce_bwd<float>(grad_out, num_segments, channels, segment_offsets, segment_of_row,
+                                       num_in, mode, vec, argmax_or_null, grad_in, s);
+      break;
+    case WCN_DTYPE_F16:
+      launch_segment_reduce_bwd<_Float16>(grad_out, num_segments, channels, segment_offsets,
+                                          segment_of_row, num_in, mode, vec, argmax_or_null, grad_in, s);
+      break;
+    default:
+      launch_segment_reduce_bwd<__bf16>(grad_out, num_segments, channels, segment_offsets, segment_of_row,
+                                        num_in, mode, vec, argmax_or_null, grad_in, s);
       break;
   }
   WCN_LAUNCH_CHECK();

@@ -92,3 +92,18 @@ class IntSearchResult:
 
     def __repr__(self) -> str:
         return f"{self.__class__.__name__}(len={len(self)}, iden_map={self.identity_map_index})"
+
+
+class RealSearchResult:
+    """Neighbour lists in CSR form: `neighbor_indices` (N) split by `neighbor_row_splits` (M + 1)
+    (reference: search_results.py:14-60; the two-tensor constructor is the one this package uses)."""
+
+    def __init__(self, neighbor_indices: Tensor, neighbor_row_splits: Tensor):
+        self.neighbor_indices = neighbor_indices.long()
+        self.neighbor_row_splits = neighbor_row_splits.long()
+        self.neighbor_distances = None
+
+    def to(self, device):
+        self.neighbor_indices = self.neighbor_indices.to(device)
+        self.neighbor_row_splits = self.neighbor_row_splits.to(device)
+        return self

@@ -8,7 +8,6 @@ grouped by output row (`wcn_map_rows_build`) and reduced with fp32 accumulation
 (`wcn_sparse_pool_fwd`); the gradient runs in the same library (`wcn_sparse_pool_bwd`).
 """
 import ctypes
-import enum
 from typing import Optional, Tuple, Union
 
 import torch
@@ -22,20 +21,8 @@ from ...geometry.coords.search.cache import IntSearchCache, IntSearchCacheKey
 from ...geometry.coords.search.search_results import IntSearchResult
 from ...geometry.coords.search.torch_discrete import generate_kernel_map
 from ...geometry.types.voxels import Voxels
+from ...ops.reductions import REDUCTIONS
 from ...utils.ntuple import ntuple
-
-
-class REDUCTIONS(enum.Enum):
-    """The reductions of warpconvnet/ops/reductions.py:13-21; min, max, mean and sum are built."""
-    MIN = "min"
-    MAX = "max"
-    MEAN = "mean"
-    SUM = "sum"
-    MUL = "mul"
-    VAR = "var"
-    STD = "std"
-    RANDOM = "random"
-
 
 _MODE = {REDUCTIONS.SUM: 0, REDUCTIONS.MEAN: 1, REDUCTIONS.MAX: 2, REDUCTIONS.MIN: 3}
 
