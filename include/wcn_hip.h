@@ -347,6 +347,15 @@ int wcn_unique_rows_csr(const int32_t* rows, int64_t num_rows, int32_t columns, 
                         int64_t* csr_indices, int64_t* csr_offsets, int64_t* to_unique,
                         int64_t* num_unique, void* stream);
 
+/* wcn_voxel_rows + wcn_unique_rows_csr over 4-column rows in one call, without storing the rows:
+ * the whole of voxel_downsample_csr_mapping (warpconvnet/geometry/coords/ops/voxel.py:51-109) up to
+ * its batch offsets.  Same outputs and workspace as wcn_unique_rows_csr (num_rows = num_points). */
+int wcn_voxelize_points_csr(const float* points, int64_t num_points, const int64_t* host_batch_offsets,
+                            const int64_t* device_batch_offsets_or_null, int32_t batch_size,
+                            double voxel_size, void* workspace, size_t workspace_bytes,
+                            int32_t* unique_rows, int64_t* to_orig, int64_t* csr_indices,
+                            int64_t* csr_offsets, int64_t* to_unique, int64_t* num_unique, void* stream);
+
 int wcn_segment_reduce(const void* features, int64_t num_in, int32_t channels, int32_t dtype,
                        const int64_t* segment_offsets, const int64_t* indices_or_null,
                        int64_t num_segments, int32_t mode, void* out, int64_t* argmax_or_null,

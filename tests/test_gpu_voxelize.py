@@ -338,3 +338,62 @@ def test_points_to_voxels_full_size_properties():
     marks = (torch.arange(n, device=DEV) % 3).float().view(-1, 1).expand(-1, 4).contiguous()
     per_voxel = segment_reduction(marks, csr_offsets, "sum", indices=csr_indices)
     assert float(per_voxel[:, 0].double().sum()) == float(marks[:, 0].double().sum())
+
+
+def test_fused_points_call_equals_rows_then_unique_and_gradient_flows():
+    """wcn_voxelize_points_csr = wcn_voxel_rows + wcn_unique_rows_csr; the inverse, derived on
+    demand, equals the one the library writes; the gradient of to_voxels reaches the points'
+    features."""
+    from warpconvnet_amd.geometry.coords.ops.voxel import voxel_rows
+    from warpconvnet_amd.geometry.types.points import Points
+    from warpconvnet_amd.utils.unique import ToUnique, unique_torch
+    pts, offsets = _points(51, 150_000, 3)
+    d = torch.as_tensor(pts, device=DEV)
+    off = torch.as_tensor(offsets)
+    fused = ToUnique(return_to_unique_indices=True)
+    unique = fused.points_to_unique_voxel_rows(d, off, 0.07)
+    want = unique_torch(voxel_rows(d, off, 0.07), return_to_unique_indices=True)
+    assert torch.equal(unique, want[0])
+    assert torch.equal(fused.to_orig_indices, want[1])  # derived from the grouping
+    assert torch.equal(fused.to_csr_indices, want[2])
+    assert torch.equal(fused.to_csr_offsets, want[3])
+    assert torch.equal(fused.to_unique_indices, want[4])
+
+    feats = normal_features(len(pts), 8, seed=9).to(DEV).requires_grad_(True)
+    st = Points(d, feats, offsets=off).to_voxels(0.07, reduction="mean")
+    gy = normal_features(len(st), 8, seed=10)
+    st.feature_tensor.backward(gy.to(DEV))
+    seg = want[1].cpu().numpy()
+    counts = np.diff(want[3].cpu().numpy())
+    want_gx = gy.double().numpy()[seg] / counts[seg][:, None]
+    assert rel_err(feats.grad.double().cpu().numpy(), want_gx) <= 1e-5
+
+
+def test_voxel_downsample_mapping():
+    """tests/coords/test_voxel_ops.py:34-75 of the reference: every point maps to the voxel (or the
+    down-sampled point) of its own cell; points outside every occupied cell are reported invalid."""
+    from warpconvnet_amd.geometry.coords.ops.voxel import voxel_downsample_mapping
+    from warpconvnet_amd.geometry.types.points import Points
+    pts, offsets = _points(61, 90_000, 3, extent=1.0)
+    feats = normal_features(len(pts), 7, seed=7)
+    pc = Points(torch.as_tensor(pts, device=DEV), feats.to(DEV), offsets=torch.as_tensor(offsets))
+    vs = 0.025
+    down = pc.voxel_downsample(vs)
+    up_map, down_map, valid = voxel_downsample_mapping(pc.coordinate_tensor, pc.offsets,
+                                                       down.coordinate_tensor, down.offsets, vs)
+    assert bool(valid.all()) and len(up_map) == len(pts)
+    assert torch.equal(torch.floor(pc.coordinate_tensor[up_map] / vs),
+                       torch.floor(down.coordinate_tensor[down_map] / vs))
+    st = pc.to_voxels(vs)
+    up_cells = torch.floor(pc.coordinate_tensor / vs).int()
+    up_map, down_map, valid = voxel_downsample_mapping(up_cells, pc.offsets, st.coordinate_tensor, st.offsets)
+    assert bool(valid.all())
+    assert torch.equal(up_cells[up_map], st.coordinate_tensor[down_map.long()])
+    # batch items must match too
+    up_batch = torch.as_tensor(np.repeat(np.arange(3), np.diff(offsets)), device=DEV)
+    down_batch = torch.as_tensor(np.repeat(np.arange(3), np.diff(st.offsets.numpy())), device=DEV)
+    assert torch.equal(up_batch[up_map], down_batch[down_map.long()])
+    moved = up_cells.clone()
+    moved[:100] += 10_000  # far outside
+    _, _, valid = voxel_downsample_mapping(moved, pc.offsets, st.coordinate_tensor, st.offsets)
+    assert int((~valid).sum()) == 100 and not bool(valid[:100].any())

@@ -7,8 +7,10 @@
 // (warpconvnet/utils/unique.py:57-109).  Here every row is packed into one 64-bit key whose numeric
 // order is the rows' lexicographic order (fields relative to the bounding box, first column most
 // significant), the (key, row index) pairs go through one stable radix sort over just the bits in
-// use, and one pass over the sorted pairs writes all five results.  The radix sort and the prefix
-// sum are rocPRIM's (plain library primitives); everything else is written here.
+// use (as 32-bit words when they fit), and one pass over the sorted pairs writes all five results.
+// For points the rows are never stored: the box and the keys are computed from the points directly.
+// The radix sort and the prefix sum are rocPRIM's (plain library primitives); everything else is
+// written here.
 #include "wcn_common.h"
 
 #include <cstring>
@@ -39,23 +41,33 @@ struct UniqueView {
   size_t temp_bytes;
 };
 
+template <typename KeyT>
 struct HeadFlag {  // 1 where a sorted key differs from its predecessor
-  const unsigned long long* keys;
+  const KeyT* keys;
   __device__ uint32_t operator()(uint32_t i) const {
     return (i == 0 || keys[i] != keys[i - 1]) ? 1u : 0u;
   }
 };
-using HeadIterator = rocprim::transform_iterator<rocprim::counting_iterator<uint32_t>, HeadFlag, uint32_t>;
+template <typename KeyT>
+using HeadIterator =
+    rocprim::transform_iterator<rocprim::counting_iterator<uint32_t>, HeadFlag<KeyT>, uint32_t>;
 
-size_t prim_temp_bytes(int64_t n) {
+template <typename KeyT>
+size_t prim_temp_bytes_for(int64_t n) {
   size_t sort_bytes = 0, scan_bytes = 0;
-  unsigned long long* k = nullptr;
+  KeyT* k = nullptr;
   uint32_t* v = nullptr;
-  (void)rocprim::radix_sort_pairs(nullptr, sort_bytes, k, k, v, v, (size_t)n, 0u, 64u, (hipStream_t)0);
-  HeadIterator heads(rocprim::counting_iterator<uint32_t>(0), HeadFlag{nullptr});
+  (void)rocprim::radix_sort_pairs(nullptr, sort_bytes, k, k, v, v, (size_t)n, 0u,
+                                  (unsigned)(8 * sizeof(KeyT)), (hipStream_t)0);
+  HeadIterator<KeyT> heads(rocprim::counting_iterator<uint32_t>(0), HeadFlag<KeyT>{nullptr});
   (void)rocprim::inclusive_scan(nullptr, scan_bytes, heads, v, (size_t)n, rocprim::plus<uint32_t>(),
                                 (hipStream_t)0);
   return sort_bytes > scan_bytes ? sort_bytes : scan_bytes;
+}
+
+size_t prim_temp_bytes(int64_t n) {
+  const size_t a = prim_temp_bytes_for<unsigned long long>(n), b = prim_temp_bytes_for<uint32_t>(n);
+  return a > b ? a : b;
 }
 
 size_t unique_layout(void* base, int64_t n, UniqueView* v) {
@@ -88,38 +100,60 @@ size_t unique_layout(void* base, int64_t n, UniqueView* v) {
   return off;
 }
 
-// ---- points -> [batch, floor(p * inv)] ----------------------------------------------------------
+// ---- where the rows come from -------------------------------------------------------------------
 // torch divides a float tensor by a host scalar as a multiplication with the scalar's reciprocal
 // (taken in double, rounded to float); the product is floored and converted to int32 the same way.
-// One thread per point; three consecutive points of a thread would make wider loads but the rows
-// are 12 bytes, so lanes read adjacent 4-byte words and the 16-byte output rows are full vectors.
 struct BatchStarts {
   int64_t start[WCN_VOXEL_MAX_BATCH + 1];
 };
 
-__global__ void __launch_bounds__(256) voxel_rows(const float* __restrict__ points, int64_t n,
-                                                  float inv, BatchStarts starts, int batch_size,
-                                                  const int64_t* __restrict__ device_starts,
-                                                  int4* __restrict__ rows) {
+struct PointRows {  // row i = [batch item of point i, floor(p * inv)]
+  const float* points;
+  float inv;
+  BatchStarts starts;
+  int batch_size;
+  const int64_t* device_starts;  // used instead of `starts` when there are too many batch items
+  __device__ __forceinline__ void load(int64_t i, int v[4]) const {
+    const float x = points[3 * i], y = points[3 * i + 1], z = points[3 * i + 2];
+    int lo = 0, hi = batch_size;  // the item lies in [lo, hi)
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      const int64_t s = device_starts ? device_starts[mid] : starts.start[mid];
+      if (s <= i) lo = mid; else hi = mid;
+    }
+    v[0] = lo;
+    v[1] = (int)floorf(x * inv);
+    v[2] = (int)floorf(y * inv);
+    v[3] = (int)floorf(z * inv);
+  }
+  __device__ __forceinline__ int columns() const { return 4; }
+};
+
+struct IntRows {  // (n, columns) int32, row-major
+  const int32_t* rows;
+  int ncol;
+  __device__ __forceinline__ void load(int64_t i, int v[4]) const {
+    if (ncol == 4) {
+      const int4 r = reinterpret_cast<const int4*>(rows)[i];
+      v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+    } else {
+      v[0] = v[1] = v[2] = v[3] = 0;
+      for (int d = 0; d < ncol; ++d) v[d] = rows[i * ncol + d];
+    }
+  }
+  __device__ __forceinline__ int columns() const { return ncol; }
+};
+
+// One thread per point: 12 bytes read (lanes read adjacent words), one 16-byte row written.
+__global__ void __launch_bounds__(256) voxel_rows(PointRows src, int64_t n, int4* __restrict__ rows) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const float x = points[3 * i], y = points[3 * i + 1], z = points[3 * i + 2];
-  // batch item = number of starts (beyond the first) that are <= i
-  int lo = 0, hi = batch_size;  // answer in [lo, hi)
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    const int64_t s = device_starts ? device_starts[mid] : starts.start[mid];
-    if (s <= i) lo = mid; else hi = mid;
-  }
-  int4 r;
-  r.x = lo;
-  r.y = (int)floorf(x * inv);
-  r.z = (int)floorf(y * inv);
-  r.w = (int)floorf(z * inv);
-  rows[i] = r;
+  int v[4];
+  src.load(i, v);
+  rows[i] = make_int4(v[0], v[1], v[2], v[3]);
 }
 
-// ---- bounding box of (n, columns) int32 rows ---------------------------------------------------
+// ---- bounding box of the rows --------------------------------------------------------------------
 __global__ void unique_init(UniqueHeader* __restrict__ h) {
   const int t = threadIdx.x;
   if (t < 4) {
@@ -129,26 +163,21 @@ __global__ void unique_init(UniqueHeader* __restrict__ h) {
   if (t == 4) h->count = 0;
 }
 
-__global__ void __launch_bounds__(256) unique_bbox(const int32_t* __restrict__ rows, int64_t n,
-                                                   int columns, UniqueHeader* __restrict__ h) {
+// A few large workgroups: the closing atomics of all workgroups land on the same eight words and
+// are served one after the other, so there is one workgroup per compute unit.
+template <class Src>
+__global__ void __launch_bounds__(1024) unique_bbox(Src src, int64_t n, UniqueHeader* __restrict__ h) {
   int mn[4] = {INT32_MAX, INT32_MAX, INT32_MAX, INT32_MAX};
   int mx[4] = {INT32_MIN, INT32_MIN, INT32_MIN, INT32_MIN};
+  const int columns = src.columns();
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-    if (columns == 4) {
-      const int4 r = reinterpret_cast<const int4*>(rows)[i];
-      const int v[4] = {r.x, r.y, r.z, r.w};
+    int v[4];
+    src.load(i, v);
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        mn[d] = min(mn[d], v[d]);
-        mx[d] = max(mx[d], v[d]);
-      }
-    } else {
-      for (int d = 0; d < columns; ++d) {
-        const int v = rows[i * columns + d];
-        mn[d] = min(mn[d], v);
-        mx[d] = max(mx[d], v);
-      }
+    for (int d = 0; d < 4; ++d) {
+      mn[d] = min(mn[d], v[d]);
+      mx[d] = max(mx[d], v[d]);
     }
   }
 #pragma unroll
@@ -159,7 +188,7 @@ __global__ void __launch_bounds__(256) unique_bbox(const int32_t* __restrict__ r
       mx[d] = max(mx[d], __shfl_xor(mx[d], s, 64));
     }
   }
-  __shared__ int smn[4][4], smx[4][4];
+  __shared__ int smn[16][4], smx[16][4];
   const int wave = threadIdx.x >> 6;
   if (wcn_lane() == 0) {
 #pragma unroll
@@ -171,8 +200,9 @@ __global__ void __launch_bounds__(256) unique_bbox(const int32_t* __restrict__ r
   __syncthreads();
   if (threadIdx.x < (unsigned)columns) {
     const int d = threadIdx.x;
+    const int waves = (int)(blockDim.x >> 6);
     int a = smn[0][d], b = smx[0][d];
-    for (int w = 1; w < 4; ++w) {
+    for (int w = 1; w < waves; ++w) {
       a = min(a, smn[w][d]);
       b = max(b, smx[w][d]);
     }
@@ -182,7 +212,8 @@ __global__ void __launch_bounds__(256) unique_bbox(const int32_t* __restrict__ r
 }
 
 // Field widths of the packed key: column d takes bits(mx - mn); the first column is the most
-// significant.  The host computes the same from its copy of the box.
+// significant.  The host computes the same from its copy of the box.  Keys of at most 32 bits are
+// stored, sorted and compared as 32-bit words (half the sort's key traffic).
 struct KeyLayout {
   uint32_t mn[4];
   uint32_t shift[4];
@@ -212,38 +243,38 @@ __host__ __device__ inline KeyLayout key_layout(const int32_t* mn, const int32_t
   return L;
 }
 
-__global__ void __launch_bounds__(256) unique_pack(const int32_t* __restrict__ rows, int64_t n,
-                                                   int columns, const UniqueHeader* __restrict__ h,
-                                                   unsigned long long* __restrict__ keys,
-                                                   uint32_t* __restrict__ idx) {
+template <class Src>
+__global__ void __launch_bounds__(256) unique_pack(Src src, int64_t n, const UniqueHeader* __restrict__ h,
+                                                   void* __restrict__ keys, uint32_t* __restrict__ idx) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
+  const int columns = src.columns();
   const KeyLayout L = key_layout(h->mn, h->mx, columns);
-  int v[4] = {0, 0, 0, 0};
-  if (columns == 4) {
-    const int4 r = reinterpret_cast<const int4*>(rows)[i];
-    v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
-  } else {
-    for (int d = 0; d < columns; ++d) v[d] = rows[i * columns + d];
-  }
+  int v[4];
+  src.load(i, v);
   unsigned long long key = 0;
 #pragma unroll
   for (int d = 0; d < 4; ++d)
-    if (d < columns && L.bits[d] > 0)  // a shift by 64 (a single 64-bit field at shift 0 never is) stays out
+    if (d < columns && L.bits[d] > 0)  // fields of width 0 stay out (their shift may be 64)
       key |= (unsigned long long)((uint32_t)v[d] - L.mn[d]) << L.shift[d];
-  keys[i] = key;
+  if (L.total <= 32u)
+    reinterpret_cast<uint32_t*>(keys)[i] = (uint32_t)key;
+  else
+    reinterpret_cast<unsigned long long*>(keys)[i] = key;
   idx[i] = (uint32_t)i;
 }
 
 // One pass over the sorted (key, row) pairs.  rank[i] = number of segment heads in [0, i].
+template <typename KeyT>
 __global__ void __launch_bounds__(256) unique_emit(
-    const unsigned long long* __restrict__ keys, const uint32_t* __restrict__ idx,
-    const uint32_t* __restrict__ rank, int64_t n, int columns, UniqueHeader* __restrict__ h,
-    int32_t* __restrict__ unique_rows, int64_t* __restrict__ to_orig, int64_t* __restrict__ csr_indices,
-    int64_t* __restrict__ csr_offsets, int64_t* __restrict__ to_unique) {
+    const KeyT* __restrict__ keys, const uint32_t* __restrict__ idx, const uint32_t* __restrict__ rank,
+    int64_t n, int columns, UniqueHeader* __restrict__ h, int32_t* __restrict__ unique_rows,
+    int64_t* __restrict__ to_orig, int64_t* __restrict__ csr_indices, int64_t* __restrict__ csr_offsets,
+    int64_t* __restrict__ to_unique) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const unsigned long long key = keys[i];
+  const KeyLayout L = key_layout(h->mn, h->mx, columns);  // the same for every thread: scalar work
+  const KeyT key = keys[i];
   const uint32_t row = idx[i];
   const int64_t u = (int64_t)rank[i] - 1;
   const bool head = i == 0 || keys[i - 1] != key;
@@ -254,11 +285,18 @@ __global__ void __launch_bounds__(256) unique_emit(
     // the sort is stable, so the head of a segment is the lowest row of its key
     if (to_unique) to_unique[u] = row;
     if (unique_rows) {
-      const KeyLayout L = key_layout(h->mn, h->mx, columns);
-      for (int d = 0; d < columns; ++d) {
-        const uint32_t field =
-            L.bits[d] == 0 ? 0u : (uint32_t)((key >> L.shift[d]) & ((1ull << L.bits[d]) - 1ull));
-        unique_rows[u * columns + d] = (int32_t)(field + L.mn[d]);
+      int32_t field[4];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const uint32_t f =
+            L.bits[d] == 0 ? 0u
+                           : (uint32_t)(((unsigned long long)key >> L.shift[d]) & ((1ull << L.bits[d]) - 1ull));
+        field[d] = (int32_t)(f + L.mn[d]);
+      }
+      if (columns == 4) {
+        reinterpret_cast<int4*>(unique_rows)[u] = make_int4(field[0], field[1], field[2], field[3]);
+      } else {
+        for (int d = 0; d < columns; ++d) unique_rows[u * columns + d] = field[d];
       }
     }
   }
@@ -268,13 +306,73 @@ __global__ void __launch_bounds__(256) unique_emit(
   }
 }
 
-}  // namespace
+// Sort, rank and emit for one key width.
+template <typename KeyT>
+int unique_finish(const UniqueView& v, int64_t n, int columns, unsigned key_bits, int32_t* unique_rows,
+                  int64_t* to_orig, int64_t* csr_indices, int64_t* csr_offsets, int64_t* to_unique,
+                  hipStream_t s) {
+  KeyT* keys_a = reinterpret_cast<KeyT*>(v.keys_a);
+  KeyT* keys_b = reinterpret_cast<KeyT*>(v.keys_b);
+  size_t temp_bytes = v.temp_bytes;
+  if (key_bits > 0) {
+    if (rocprim::radix_sort_pairs(v.temp, temp_bytes, keys_a, keys_b, v.idx_a, v.idx_b, (size_t)n, 0u,
+                                  key_bits, s) != hipSuccess)
+      return WCN_ERR_LAUNCH;
+  }
+  const KeyT* keys = key_bits > 0 ? keys_b : keys_a;  // all rows equal: nothing to sort
+  const uint32_t* idx = key_bits > 0 ? v.idx_b : v.idx_a;
+  HeadIterator<KeyT> heads(rocprim::counting_iterator<uint32_t>(0), HeadFlag<KeyT>{keys});
+  temp_bytes = v.temp_bytes;
+  if (rocprim::inclusive_scan(v.temp, temp_bytes, heads, v.rank, (size_t)n, rocprim::plus<uint32_t>(), s) !=
+      hipSuccess)
+    return WCN_ERR_LAUNCH;
+  hipLaunchKernelGGL(unique_emit<KeyT>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, idx,
+                     (const uint32_t*)v.rank, n, columns, v.hdr, unique_rows, to_orig, csr_indices,
+                     csr_offsets, to_unique);
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
 
-extern "C" {
+// The whole pipeline over a row source.
+template <class Src>
+int unique_run(const Src& src, int64_t n, int columns, void* workspace, size_t workspace_bytes,
+               int32_t* unique_rows, int64_t* to_orig, int64_t* csr_indices, int64_t* csr_offsets,
+               int64_t* to_unique, int64_t* num_unique, hipStream_t s) {
+  if (workspace_bytes < unique_layout(nullptr, n, nullptr)) return WCN_ERR_WORKSPACE;
+  UniqueView v;
+  unique_layout(workspace, n, &v);
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  hipLaunchKernelGGL(unique_init, dim3(1), dim3(64), 0, s, v.hdr);
+  WCN_LAUNCH_CHECK();
+  const unsigned big_blocks = (unsigned)((n + 1023) / 1024);
+  hipLaunchKernelGGL(unique_bbox<Src>, dim3(big_blocks < 256u ? big_blocks : 256u), dim3(1024), 0, s, src, n,
+                     v.hdr);
+  WCN_LAUNCH_CHECK();
+  // The sort needs the number of key bits on the host: one small read, while the keys are packed.
+  if (wcn_read_early_begin(v.hdr, 32, s) != WCN_OK) return WCN_ERR_LAUNCH;
+  hipLaunchKernelGGL(unique_pack<Src>, dim3(blocks), dim3(256), 0, s, src, n, (const UniqueHeader*)v.hdr,
+                     (void*)v.keys_a, v.idx_a);
+  WCN_LAUNCH_CHECK();
+  int32_t box[8];
+  if (wcn_read_early_end(box, v.hdr, 32, s) != WCN_OK) return WCN_ERR_LAUNCH;
+  const KeyLayout L = key_layout(box, box + 4, columns);
+  if (L.total > 64u) return WCN_ERR_COORD_RANGE;
+  const int rc = L.total <= 32u
+                     ? unique_finish<uint32_t>(v, n, columns, L.total, unique_rows, to_orig, csr_indices,
+                                               csr_offsets, to_unique, s)
+                     : unique_finish<unsigned long long>(v, n, columns, L.total, unique_rows, to_orig,
+                                                         csr_indices, csr_offsets, to_unique, s);
+  if (rc != WCN_OK) return rc;
+  int32_t count = 0;
+  if (wcn_read_small(&count, &v.hdr->count, sizeof(count), s) != WCN_OK) return WCN_ERR_LAUNCH;
+  *num_unique = count;
+  return WCN_OK;
+}
 
-int wcn_voxel_rows(const float* points, int64_t num_points, const int64_t* host_batch_offsets,
-                   const int64_t* device_batch_offsets_or_null, int32_t batch_size, double voxel_size,
-                   int32_t* rows, void* stream) {
+// Checks the batch offsets and fills the by-value copy the kernels take.
+int make_point_rows(const float* points, int64_t num_points, const int64_t* host_batch_offsets,
+                    const int64_t* device_batch_offsets_or_null, int32_t batch_size, double voxel_size,
+                    PointRows* src) {
   if (num_points < 0 || num_points >= (1ll << 31) || batch_size < 1 || !host_batch_offsets ||
       !(voxel_size > 0.0))
     return WCN_ERR_INVALID_ARGUMENT;
@@ -283,16 +381,36 @@ int wcn_voxel_rows(const float* points, int64_t num_points, const int64_t* host_
   for (int b = 0; b < batch_size; ++b)
     if (host_batch_offsets[b + 1] < host_batch_offsets[b]) return WCN_ERR_INVALID_ARGUMENT;
   if (batch_size > WCN_VOXEL_MAX_BATCH && !device_batch_offsets_or_null) return WCN_ERR_INVALID_ARGUMENT;
-  if (num_points == 0) return WCN_OK;
-  if (!points || !rows) return WCN_ERR_INVALID_ARGUMENT;
-  BatchStarts starts;
+  if (num_points > 0 && !points) return WCN_ERR_INVALID_ARGUMENT;
+  src->points = points;
+  src->inv = (float)(1.0 / voxel_size);
+  src->batch_size = batch_size;
+  src->device_starts = batch_size > WCN_VOXEL_MAX_BATCH ? device_batch_offsets_or_null : nullptr;
   for (int b = 0; b <= WCN_VOXEL_MAX_BATCH; ++b)
-    starts.start[b] = b <= batch_size && batch_size <= WCN_VOXEL_MAX_BATCH ? host_batch_offsets[b] : 0;
-  const float inv = (float)(1.0 / voxel_size);
+    src->starts.start[b] = b <= batch_size && batch_size <= WCN_VOXEL_MAX_BATCH ? host_batch_offsets[b] : 0;
+  return WCN_OK;
+}
+
+int empty_result(int64_t* csr_offsets, hipStream_t s) {
+  if (csr_offsets && hipMemsetAsync(csr_offsets, 0, sizeof(int64_t), s) != hipSuccess) return WCN_ERR_LAUNCH;
+  return WCN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int wcn_voxel_rows(const float* points, int64_t num_points, const int64_t* host_batch_offsets,
+                   const int64_t* device_batch_offsets_or_null, int32_t batch_size, double voxel_size,
+                   int32_t* rows, void* stream) {
+  PointRows src;
+  const int rc = make_point_rows(points, num_points, host_batch_offsets, device_batch_offsets_or_null,
+                                 batch_size, voxel_size, &src);
+  if (rc != WCN_OK) return rc;
+  if (num_points == 0) return WCN_OK;
+  if (!rows) return WCN_ERR_INVALID_ARGUMENT;
   hipLaunchKernelGGL(voxel_rows, dim3((unsigned)((num_points + 255) / 256)), dim3(256), 0,
-                     (hipStream_t)stream, points, num_points, inv, starts, batch_size,
-                     batch_size > WCN_VOXEL_MAX_BATCH ? device_batch_offsets_or_null : nullptr,
-                     (int4*)rows);
+                     (hipStream_t)stream, src, num_points, (int4*)rows);
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }
@@ -309,57 +427,28 @@ int wcn_unique_rows_csr(const int32_t* rows, int64_t num_rows, int32_t columns, 
   if (num_rows < 0 || num_rows >= (1ll << 31) || columns < 1 || columns > 4 || !num_unique)
     return WCN_ERR_INVALID_ARGUMENT;
   *num_unique = 0;
-  hipStream_t s = (hipStream_t)stream;
-  if (num_rows == 0) {
-    if (csr_offsets) {
-      if (hipMemsetAsync(csr_offsets, 0, sizeof(int64_t), s) != hipSuccess) return WCN_ERR_LAUNCH;
-    }
-    return WCN_OK;
-  }
+  if (num_rows == 0) return empty_result(csr_offsets, (hipStream_t)stream);
   if (!rows || !workspace) return WCN_ERR_INVALID_ARGUMENT;
-  if (workspace_bytes < wcn_unique_rows_workspace_bytes(num_rows)) return WCN_ERR_WORKSPACE;
-  UniqueView v;
-  unique_layout(workspace, num_rows, &v);
-  const unsigned blocks = (unsigned)((num_rows + 255) / 256);
+  const IntRows src{rows, (int)columns};
+  return unique_run(src, num_rows, (int)columns, workspace, workspace_bytes, unique_rows, to_orig,
+                    csr_indices, csr_offsets, to_unique, num_unique, (hipStream_t)stream);
+}
 
-  hipLaunchKernelGGL(unique_init, dim3(1), dim3(64), 0, s, v.hdr);
-  WCN_LAUNCH_CHECK();
-  // one workgroup per compute unit: the closing atomics of all workgroups land on the same eight
-  // words and are served one after the other
-  const unsigned box_blocks = blocks < 256u ? blocks : 256u;
-  hipLaunchKernelGGL(unique_bbox, dim3(box_blocks), dim3(256), 0, s, rows, num_rows, (int)columns, v.hdr);
-  WCN_LAUNCH_CHECK();
-  // The sort needs the number of key bits on the host: one small read, while the keys are packed.
-  if (wcn_read_early_begin(v.hdr, 32, s) != WCN_OK) return WCN_ERR_LAUNCH;
-  hipLaunchKernelGGL(unique_pack, dim3(blocks), dim3(256), 0, s, rows, num_rows, (int)columns,
-                     (const UniqueHeader*)v.hdr, v.keys_a, v.idx_a);
-  WCN_LAUNCH_CHECK();
-  int32_t box[8];
-  if (wcn_read_early_end(box, v.hdr, 32, s) != WCN_OK) return WCN_ERR_LAUNCH;
-  const KeyLayout L = key_layout(box, box + 4, columns);
-  if (L.total > 64u) return WCN_ERR_COORD_RANGE;
-
-  size_t temp_bytes = v.temp_bytes;
-  if (L.total > 0) {
-    if (rocprim::radix_sort_pairs(v.temp, temp_bytes, v.keys_a, v.keys_b, v.idx_a, v.idx_b,
-                                  (size_t)num_rows, 0u, L.total, s) != hipSuccess)
-      return WCN_ERR_LAUNCH;
-  }
-  const unsigned long long* keys = L.total > 0 ? v.keys_b : v.keys_a;  // all rows equal: nothing to sort
-  const uint32_t* idx = L.total > 0 ? v.idx_b : v.idx_a;
-  HeadIterator heads(rocprim::counting_iterator<uint32_t>(0), HeadFlag{keys});
-  temp_bytes = v.temp_bytes;
-  if (rocprim::inclusive_scan(v.temp, temp_bytes, heads, v.rank, (size_t)num_rows,
-                              rocprim::plus<uint32_t>(), s) != hipSuccess)
-    return WCN_ERR_LAUNCH;
-  hipLaunchKernelGGL(unique_emit, dim3(blocks), dim3(256), 0, s, keys, idx, (const uint32_t*)v.rank,
-                     num_rows, (int)columns, v.hdr, unique_rows, to_orig, csr_indices, csr_offsets,
-                     to_unique);
-  WCN_LAUNCH_CHECK();
-  int32_t count = 0;
-  if (wcn_read_small(&count, &v.hdr->count, sizeof(count), s) != WCN_OK) return WCN_ERR_LAUNCH;
-  *num_unique = count;
-  return WCN_OK;
+int wcn_voxelize_points_csr(const float* points, int64_t num_points, const int64_t* host_batch_offsets,
+                            const int64_t* device_batch_offsets_or_null, int32_t batch_size,
+                            double voxel_size, void* workspace, size_t workspace_bytes,
+                            int32_t* unique_rows, int64_t* to_orig, int64_t* csr_indices,
+                            int64_t* csr_offsets, int64_t* to_unique, int64_t* num_unique, void* stream) {
+  if (!num_unique) return WCN_ERR_INVALID_ARGUMENT;
+  *num_unique = 0;
+  PointRows src;
+  const int rc = make_point_rows(points, num_points, host_batch_offsets, device_batch_offsets_or_null,
+                                 batch_size, voxel_size, &src);
+  if (rc != WCN_OK) return rc;
+  if (num_points == 0) return empty_result(csr_offsets, (hipStream_t)stream);
+  if (!workspace) return WCN_ERR_INVALID_ARGUMENT;
+  return unique_run(src, num_points, 4, workspace, workspace_bytes, unique_rows, to_orig, csr_indices,
+                    csr_offsets, to_unique, num_unique, (hipStream_t)stream);
 }
 
 }  // extern "C"

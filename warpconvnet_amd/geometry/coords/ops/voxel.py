@@ -54,9 +54,9 @@ def voxel_downsample_csr_mapping(batched_points: Tensor, offsets: Tensor, voxel_
     n = len(batched_points)
     batch = len(offsets) - 1
     assert int(offsets[-1]) == n, f"Offsets {offsets} does not match the number of points {n}"
-    rows = voxel_rows(batched_points, offsets, voxel_size)
     to_unique = ToUnique(return_to_unique_indices=True, unique_method=unique_method)
-    unique_rows, to_csr_indices, to_csr_offsets = to_unique.to_unique_csr(rows, dim=0)
+    unique_rows = to_unique.points_to_unique_voxel_rows(batched_points, offsets, voxel_size)
+    to_csr_indices, to_csr_offsets = to_unique.to_csr_indices, to_unique.to_csr_offsets
     if batch == 1:
         unique_offsets = torch.IntTensor([0, len(unique_rows)])
         unique_coords = unique_rows[:, 1:]
@@ -75,15 +75,46 @@ def voxel_downsample_random_indices(batched_points: Tensor, offsets: Tensor,
     The representative is the lowest row of each voxel (the reference's depends on a race)."""
     n = len(batched_points)
     assert int(offsets[-1]) == n, f"Offsets {offsets} does not match the number of points {n}"
-    if voxel_size is not None:
-        voxel_coords = torch.floor(batched_points / voxel_size).int()
+    if (voxel_size is not None and batched_points.is_cuda and batched_points.dtype == torch.float32
+            and batched_points.shape[1] == 3):
+        keys = voxel_rows(batched_points, offsets, voxel_size)  # one kernel for floor, cast, batch column, cat
     else:
-        voxel_coords = batched_points.int()
-    batch_index = batch_index_from_offset(offsets).to(batched_points.device)
-    keys = torch.cat([batch_index.unsqueeze(1).int(), voxel_coords], dim=1)
+        if voxel_size is not None:
+            voxel_coords = torch.floor(batched_points / voxel_size).int()
+        else:
+            voxel_coords = batched_points.int()
+        batch_index = batch_index_from_offset(offsets).to(batched_points.device)
+        keys = torch.cat([batch_index.unsqueeze(1).int(), voxel_coords], dim=1)
     table = TorchHashTable(max(16, 2 * n), device=keys.device)
     table.insert(keys)
     unique_indices = table.unique_index.long()
-    counts = torch.bincount(batch_index[unique_indices], minlength=len(offsets) - 1).cpu()
+    counts = torch.bincount(keys[unique_indices, 0], minlength=len(offsets) - 1).cpu()
     batch_offsets = torch.cat([counts.new_zeros(1), counts.cumsum(dim=0)])
     return unique_indices, batch_offsets
+
+
+def _voxel_rows_of(points_or_cells: Tensor, offsets: Tensor, voxel_size: Optional[float]) -> Tensor:
+    if voxel_size is not None and points_or_cells.dtype == torch.float32:
+        return voxel_rows(points_or_cells, offsets, voxel_size)
+    cells = (torch.floor(points_or_cells / voxel_size) if voxel_size is not None else points_or_cells).int()
+    batch_index = batch_index_from_offset(offsets).to(cells.device)
+    return torch.cat([batch_index.unsqueeze(1).int(), cells], dim=1)
+
+
+@torch.no_grad()
+def voxel_downsample_mapping(up_batched_points: Tensor, up_offsets: Tensor, down_batched_points: Tensor,
+                             down_offsets: Tensor, voxel_size: Optional[float] = None,
+                             find_nearest_for_invalid: bool = False) -> Tuple[Tensor, Tensor, Tensor]:
+    """up_map, down_map, valid with voxel(up[up_map]) == voxel(down[down_map]): every up point is
+    looked up in a coordinate table of the down points' voxels (voxel.py:189-258).  Filling the
+    misses with the nearest down point needs a nearest-neighbour search and is not built."""
+    require_device(up_batched_points, "up_batched_points")
+    assert up_batched_points.device == down_batched_points.device, \
+        "up_batched_points and down_batched_points must be on the same device"
+    if find_nearest_for_invalid:
+        raise NotImplementedError("find_nearest_for_invalid needs a nearest-neighbour search, which is not built")
+    up_rows = _voxel_rows_of(up_batched_points, up_offsets, voxel_size)
+    down_rows = _voxel_rows_of(down_batched_points, down_offsets, voxel_size)
+    down_map = TorchHashTable.from_keys(down_rows).search(up_rows)
+    valid = down_map >= 0
+    return torch.nonzero(valid).squeeze(1), down_map[valid], valid

@@ -60,7 +60,7 @@ class Points(Geometry):
         _, unique_offsets, csr_indices, csr_offsets, to_unique = voxel_downsample_csr_mapping(
             self.coordinate_tensor, self.offsets, voxel_size)
         down = segment_reduction(self.feature_tensor, csr_offsets, reduction, indices=csr_indices,
-                                 segment_of=to_unique.to_orig_indices)
+                                 segment_of=lambda: to_unique.to_orig_indices)
         return self.__class__(
             RealCoords(self.coordinate_tensor[to_unique.to_unique_indices], offsets=unique_offsets),
             CatFeatures(down, offsets=unique_offsets), **extra)

@@ -65,7 +65,7 @@ def point_pool(pc, reduction: Union[REDUCTIONS, str], downsample_max_num_points:
     _, unique_offsets, csr_indices, csr_offsets, to_unique = voxel_downsample_csr_mapping(
         pc.coordinate_tensor, pc.offsets, downsample_voxel_size, unique_method=unique_method)
     down_features = segment_reduction(pc.feature_tensor, csr_offsets, reduction, indices=csr_indices,
-                                      segment_of=to_unique.to_orig_indices)
+                                      segment_of=lambda: to_unique.to_orig_indices)
     if return_type == "voxel":
         rows = to_unique.unique_rows  # (M, 4) [batch, x, y, z]: what the convolutions' tables are built from
         coords = IntCoords(rows[:, 1:].contiguous(), offsets=unique_offsets)
@@ -74,7 +74,7 @@ def point_pool(pc, reduction: Union[REDUCTIONS, str], downsample_max_num_points:
     else:
         if avereage_pooled_coordinates:
             xyz = segment_reduction(pc.coordinate_tensor, csr_offsets, REDUCTIONS.MEAN,
-                                    indices=csr_indices, segment_of=to_unique.to_orig_indices)
+                                    indices=csr_indices, segment_of=lambda: to_unique.to_orig_indices)
         else:
             xyz = pc.coordinate_tensor[to_unique.to_unique_indices]
         out = Points(RealCoords(xyz, offsets=unique_offsets), down_features,

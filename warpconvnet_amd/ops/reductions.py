@@ -41,7 +41,8 @@ def _segment_of_rows(offsets: Tensor, indices: Optional[Tensor], num_in: int) ->
 class _SegmentReduceFunction(Function):
     """out[u] = reduce of features[indices[e]] over e in [offsets[u], offsets[u + 1]).  The
     gradient assumes that no feature row lies in two segments (true for the grouping of points by
-    voxel); `segment_of` may be passed when the caller already has it (unique's inverse)."""
+    voxel); `segment_of` (a tensor, or a function returning it, called in the backward pass only)
+    may be passed when the caller has the segment of every row (unique's inverse)."""
 
     @staticmethod
     def forward(ctx, features: Tensor, offsets: Tensor, indices: Optional[Tensor], mode: int,
@@ -69,6 +70,8 @@ class _SegmentReduceFunction(Function):
         offsets, indices, segment_of, arg = ctx.saved
         gy = grad_out.contiguous()
         m, channels = gy.shape
+        if callable(segment_of):
+            segment_of = segment_of()
         if segment_of is None:
             segment_of = _segment_of_rows(offsets, indices, ctx.n_in)
         segment_of = segment_of.to(torch.int64).contiguous()
