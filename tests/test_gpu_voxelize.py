@@ -397,3 +397,38 @@ def test_voxel_downsample_mapping():
     moved[:100] += 10_000  # far outside
     _, _, valid = voxel_downsample_mapping(moved, pc.offsets, st.coordinate_tensor, st.offsets)
     assert int((~valid).sum()) == 100 and not bool(valid[:100].any())
+
+
+def test_point_to_sparse_wrapper_and_unpool():
+    """Points -> voxels (mean) -> 3x3x3 convolution -> back onto the points: every point receives
+    the output row of its own voxel, concatenated with its own features
+    (reference: nn/modules/sparse_pool.py:172-189; its default unique_method "morton" takes the
+    plain torch.unique branch of ToUnique)."""
+    from oracle import voxelize
+    from warpconvnet_amd.geometry.types.points import Points
+    from warpconvnet_amd.nn.functional.point_pool import point_pool
+    from warpconvnet_amd.nn.modules.point_pool import PointMaxPool, PointToSparseWrapper, PointUnpool
+    from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d
+    pts, offsets = _points(71, 50_000, 2, extent=2.0)
+    feats = normal_features(len(pts), 16, seed=8)
+    pc = Points(torch.as_tensor(pts, device=DEV), feats.to(DEV), offsets=torch.as_tensor(offsets))
+    torch.manual_seed(1)
+    conv = SparseConv3d(16, 32, kernel_size=3).to(DEV)
+    out = PointToSparseWrapper(conv, voxel_size=0.1, concat_unpooled_pc=True)(pc)
+    assert isinstance(out, Points) and len(out) == len(pc) and out.num_channels == 32 + 16
+    assert torch.equal(out.coordinate_tensor, pc.coordinate_tensor)
+    st, tu = point_pool(pc, "mean", downsample_voxel_size=0.1, return_type="voxel", return_to_unique=True)
+    want_rows = conv(st).feature_tensor
+    rows = voxelize.voxel_rows(pts, offsets, 0.1)
+    inverse = voxelize.unique_rows_csr(rows)[1]
+    assert np.array_equal(tu.to_orig_indices.cpu().numpy(), inverse)
+    assert torch.equal(out.feature_tensor[:, :32], want_rows[torch.as_tensor(inverse, device=DEV)])
+    assert torch.equal(out.feature_tensor[:, 32:], pc.feature_tensor)
+    # module form (test_point_pool.py:95-121 of the reference, with the pooling's ToUnique handed over)
+    pooled, tu = point_pool(pc, "max", downsample_voxel_size=0.1, return_to_unique=True)
+    back = PointUnpool(concat_unpooled_pc=False)(pooled, pc, to_unique=tu)
+    assert len(back) == len(pc) and back.num_channels == pooled.num_channels
+    assert torch.equal(back.feature_tensor, pooled.feature_tensor[tu.to_orig_indices])
+    assert bool((back.feature_tensor >= pc.feature_tensor).all())  # a maximum over a set containing the point
+    with pytest.raises(NotImplementedError):
+        PointUnpool()(PointMaxPool(downsample_voxel_size=0.1)(pc), pc)  # needs a nearest-neighbour search

@@ -43,7 +43,7 @@ def _offsets_of_sorted_batch_column(rows: Tensor, batch_size: int) -> Tensor:
 
 @torch.no_grad()
 def voxel_downsample_csr_mapping(batched_points: Tensor, offsets: Tensor, voxel_size: float,
-                                 unique_method: Optional[str] = None
+                                 unique_method: Optional[str] = None, return_to_orig_indices: bool = False
                                  ) -> Tuple[Tensor, Tensor, Tensor, Tensor, ToUnique]:
     """Distinct voxels of the points in ascending (batch, x, y, z) order with the grouping of the
     points by voxel (voxel.py:51-109):
@@ -54,7 +54,8 @@ def voxel_downsample_csr_mapping(batched_points: Tensor, offsets: Tensor, voxel_
     n = len(batched_points)
     batch = len(offsets) - 1
     assert int(offsets[-1]) == n, f"Offsets {offsets} does not match the number of points {n}"
-    to_unique = ToUnique(return_to_unique_indices=True, unique_method=unique_method)
+    to_unique = ToUnique(return_to_unique_indices=True, unique_method=unique_method,
+                         return_to_orig_indices=return_to_orig_indices)
     unique_rows = to_unique.points_to_unique_voxel_rows(batched_points, offsets, voxel_size)
     to_csr_indices, to_csr_offsets = to_unique.to_csr_indices, to_unique.to_csr_offsets
     if batch == 1:

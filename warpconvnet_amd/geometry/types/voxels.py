@@ -110,6 +110,19 @@ class Voxels(Geometry):
             feats[outside] = 0
         return target.replace(batched_features=feats)
 
+    def to_point(self, voxel_size: Optional[float] = None):
+        """Points at the voxels' corners, `coordinates * voxel_size` (times the tensor stride)
+        (reference: voxels.py:228-246)."""
+        if voxel_size is None:
+            assert self.voxel_size is not None, \
+                "Voxel size must be provided or the object must have been initialized with a voxel size to convert to point."
+            voxel_size = self.voxel_size
+        if self.tensor_stride is not None:
+            voxel_size = torch.tensor([[voxel_size * s for s in self.tensor_stride]], device=self.device)
+        from ..coords.real import RealCoords
+        from .points import Points
+        return Points(RealCoords(self.coordinate_tensor * voxel_size, self.offsets), self.batched_features)
+
     def to_dense(self, channel_dim: int = 1, spatial_shape: Optional[Tuple[int, ...]] = None,
                  min_coords: Optional[Tuple[int, ...]] = None,
                  max_coords: Optional[Tuple[int, ...]] = None) -> Tensor:

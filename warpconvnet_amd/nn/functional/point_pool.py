@@ -62,9 +62,11 @@ def point_pool(pc, reduction: Union[REDUCTIONS, str], downsample_max_num_points:
             "return_neighbor_search_result must be False when reduction is RANDOM."
         return _pool_by_random_sample(pc, downsample_voxel_size, return_type)
 
+    feats = pc.feature_tensor
     _, unique_offsets, csr_indices, csr_offsets, to_unique = voxel_downsample_csr_mapping(
-        pc.coordinate_tensor, pc.offsets, downsample_voxel_size, unique_method=unique_method)
-    down_features = segment_reduction(pc.feature_tensor, csr_offsets, reduction, indices=csr_indices,
+        pc.coordinate_tensor, pc.offsets, downsample_voxel_size, unique_method=unique_method,
+        return_to_orig_indices=return_to_unique or (feats.requires_grad and torch.is_grad_enabled()))
+    down_features = segment_reduction(feats, csr_offsets, reduction, indices=csr_indices,
                                       segment_of=lambda: to_unique.to_orig_indices)
     if return_type == "voxel":
         rows = to_unique.unique_rows  # (M, 4) [batch, x, y, z]: what the convolutions' tables are built from

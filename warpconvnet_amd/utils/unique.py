@@ -107,21 +107,27 @@ class UniqueInfo:
 class ToUnique:
     """(unique.py:157-251).  "torch" and "ravel" give the same result here: ravelling keeps the
     lexicographic order, and the library packs the rows into one key anyway."""
+
     unique_info: UniqueInfo
 
     def __init__(self, unique_method: Optional[Literal["torch", "ravel", "encode"]] = "torch",
-                 return_to_unique_indices: bool = False):
+                 return_to_unique_indices: bool = False, return_to_orig_indices: bool = False):
         if unique_method is None:
             unique_method = "torch"
-        if unique_method not in ("torch", "ravel"):
-            raise NotImplementedError(f"unique_method {unique_method!r} is not built (torch, ravel are)")
+        if unique_method == "encode":
+            raise NotImplementedError("unique_method 'encode' (order of the Morton codes) is not built")
+        # any other name takes the reference's plain torch.unique branch (unique.py:176-177), also
+        # the "morton" that its point modules pass by default
         self.unique_method = unique_method
         self.return_to_unique_indices = return_to_unique_indices or unique_method == "ravel"
+        # ask the library for the inverse when it is known to be read (gradients, unpooling);
+        # otherwise it is derived on first access
+        self.return_to_orig_indices = return_to_orig_indices
 
     def to_unique(self, x: Tensor, dim: int = 0) -> Tensor:
         assert dim == 0, "rows are compared along dim 0"
         unique, to_orig, csr_indices, csr_offsets, to_unique = _unique_rows(
-            x, False, self.return_to_unique_indices)
+            x, self.return_to_orig_indices, self.return_to_unique_indices)
         self.unique_info = UniqueInfo(to_orig, csr_indices, csr_offsets, to_unique)
         return unique
 
@@ -148,7 +154,7 @@ class ToUnique:
                   "wcn_voxelize_points_csr")
 
         unique, to_orig, csr_indices, csr_offsets, to_unique = _run_unique(
-            call, n, 4, pts.device, False, self.return_to_unique_indices)
+            call, n, 4, pts.device, self.return_to_orig_indices, self.return_to_unique_indices)
         self.unique_info = UniqueInfo(to_orig, csr_indices, csr_offsets, to_unique)
         return unique
 
