@@ -290,3 +290,81 @@ def test_voxels_dense_round_trip():
     # two spatial dimensions
     d2 = torch.randn(1, 2, 4, 4, generator=g) * (torch.rand(1, 1, 4, 4, generator=g) < 0.5)
     assert torch.equal(Voxels.from_dense(d2).to_dense(spatial_shape=(4, 4)), d2)
+
+
+def test_voxelisation_entry_points_reject_bad_arguments():
+    from warpconvnet_amd._lib import lib
+    L = lib()
+    null = ctypes.c_void_p(0)
+    fake = ctypes.c_void_p(4096)  # never dereferenced: validation fails first
+    count = ctypes.c_int64(7)
+    ok = (ctypes.c_int64 * 3)(0, 4, 10)
+    assert L.wcn_unique_rows_workspace_bytes(-1) == 0 and L.wcn_unique_rows_workspace_bytes(1 << 31) == 0
+    small, large = L.wcn_unique_rows_workspace_bytes(1000), L.wcn_unique_rows_workspace_bytes(10**6)
+    assert small >= 256 + 1000 * 28 and large >= 256 + 10**6 * 28
+    assert L.wcn_unique_rows_csr(fake, 10, 5, fake, 1 << 30, null, null, null, null, null, ctypes.byref(count), null) == -1
+    assert L.wcn_unique_rows_csr(fake, 10, 0, fake, 1 << 30, null, null, null, null, null, ctypes.byref(count), null) == -1
+    assert L.wcn_unique_rows_csr(fake, 10, 4, fake, 1 << 30, null, null, null, null, null, None, null) == -1
+    assert L.wcn_unique_rows_csr(null, 10, 4, fake, 1 << 30, null, null, null, null, null, ctypes.byref(count), null) == -1
+    assert L.wcn_unique_rows_csr(fake, 10, 4, fake, 64, null, null, null, null, null, ctypes.byref(count), null) == -6
+    assert count.value == 0
+    for offsets, batch, size in ((ok, 2, 0.0), (ok, 2, -1.0), ((ctypes.c_int64 * 3)(0, 4, 9), 2, 0.1),
+                                 ((ctypes.c_int64 * 3)(1, 4, 10), 2, 0.1), ((ctypes.c_int64 * 3)(0, 11, 10), 2, 0.1),
+                                 (ok, 0, 0.1), (None, 2, 0.1)):
+        assert L.wcn_voxel_rows(fake, 10, offsets, null, batch, size, fake, null) == -1
+        assert L.wcn_voxelize_points_csr(fake, 10, offsets, null, batch, size, fake, 1 << 30, null, null, null,
+                                         null, null, ctypes.byref(count), null) == -1
+    many = (ctypes.c_int64 * 102)(*range(0, 102))  # 101 batch items: the offsets must also be on the device
+    assert L.wcn_voxel_rows(fake, 101, many, null, 101, 0.1, fake, null) == -1
+    assert L.wcn_voxelize_points_csr(fake, 10, ok, null, 2, 0.1, fake, 64, null, null, null, null, null,
+                                     ctypes.byref(count), null) == -6
+    offs = (ctypes.c_int64 * 2)(0, 5)
+    assert L.wcn_segment_reduce(fake, 5, 8, 7, offs, null, 1, 0, fake, null, null) == -1     # dtype
+    assert L.wcn_segment_reduce(fake, 5, 8, 0, offs, null, 1, 4, fake, null, null) == -1     # mode
+    assert L.wcn_segment_reduce(fake, 5, 0, 0, offs, null, 1, 0, fake, null, null) == -1     # channels
+    assert L.wcn_segment_reduce(fake, 5, 8, 0, None, null, 1, 0, fake, null, null) == -1
+    assert L.wcn_segment_reduce(fake, 5, 8, 0, offs, null, 0, 0, null, null, null) == 0      # nothing to do
+    assert L.wcn_segment_reduce_bwd(fake, 1, 8, 0, offs, fake, 5, 2, null, fake, null) == -1  # max without argmax
+    assert L.wcn_segment_reduce_bwd(fake, 1, 8, 0, offs, null, 5, 0, null, fake, null) == -1  # no segment ids
+
+
+def test_points_reductions_and_unique_host_logic():
+    import torch
+    from warpconvnet_amd.geometry.types.points import Points
+    from warpconvnet_amd.nn.functional.point_pool import point_pool
+    from warpconvnet_amd.ops.reductions import REDUCTIONS, row_reduction
+    from warpconvnet_amd.utils.unique import ToUnique, UniqueInfo
+    import warpconvnet_amd.nn.functional.sparse_pool as sparse_pool
+    assert sparse_pool.REDUCTIONS is REDUCTIONS  # one enum for both pooling paths
+    coords = [torch.rand(5, 3), torch.rand(7, 3)]
+    feats = [torch.rand(5, 4), torch.rand(7, 4)]
+    pc = Points(coords, feats)
+    assert len(pc) == 12 and pc.batch_size == 2 and pc.offsets.tolist() == [0, 5, 12] and pc.num_channels == 4
+    assert Points(torch.cat(coords), torch.cat(feats), offsets=torch.tensor([0, 5, 12])).equal_shape(pc)
+    with pytest.raises(AssertionError):
+        Points(torch.rand(5, 2), torch.rand(5, 4), offsets=torch.tensor([0, 5]))  # not 3-D
+    with pytest.raises(AssertionError):
+        Points(coords, feats[:1])
+    with pytest.raises(AssertionError):
+        point_pool(pc, "mean")  # neither a voxel size nor a point count
+    with pytest.raises(AssertionError):
+        point_pool(pc, "mean", downsample_voxel_size=0.1, return_type="grid")
+    with pytest.raises(AssertionError):
+        point_pool(pc, "mean", downsample_voxel_size=0.1, return_type="voxel", avereage_pooled_coordinates=True)
+    with pytest.raises(NotImplementedError):
+        point_pool(pc, "mean", downsample_max_num_points=4)
+    with pytest.raises(AssertionError):
+        point_pool(pc, "random", downsample_voxel_size=0.1, return_to_unique=True)
+    with pytest.raises((ValueError, RuntimeError)):
+        point_pool(pc, "mean", downsample_voxel_size=0.1)  # CPU tensors: the library path refuses them
+    with pytest.raises(NotImplementedError):
+        ToUnique(unique_method="encode")
+    assert ToUnique(unique_method="morton").unique_method == "morton"  # the point modules' default
+    with pytest.raises(AssertionError):
+        row_reduction(torch.rand(5, 2), torch.tensor([0, 2, 4]), "sum")  # splits do not cover the rows
+    with pytest.raises(ValueError):
+        REDUCTIONS("median")
+    # the inverse is derived from the grouping on first access
+    info = UniqueInfo(None, torch.tensor([2, 0, 3, 1, 4]), torch.tensor([0, 2, 3, 5]), None)
+    assert info.to_orig_indices.tolist() == [0, 2, 0, 1, 2]
+    assert info.to_orig_indices is info.to_orig_indices
