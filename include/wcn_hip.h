@@ -329,7 +329,8 @@ int wcn_morton_codes(const int32_t* coords, int64_t n, int32_t columns, int32_t 
  * (warpconvnet/ops/reductions.py:36-72, torch_scatter.segment_csr; called from
  * warpconvnet/nn/functional/point_pool.py:298-302): out[u] = sum / mean / max / min (mode 0..3, as
  * for wcn_sparse_pool_fwd) over e in [segment_offsets[u], segment_offsets[u + 1]) of
- * features[indices[e]] (features[e] when indices is NULL); empty segments give 0.  argmax (M, C)
+ * features[indices[e]] (features[e] when indices is NULL); num_entries is the length of the entry
+ * list (offsets beyond it are cut to it); empty segments give 0.  argmax (M, C)
  * int64 receives the feature row behind each extremum.  wcn_segment_reduce_bwd is its gradient for
  * disjoint segments: segment_of_row (N) names each feature row's segment (out of range = none).
  * ------------------------------------------------------------------------------------------- */
@@ -358,8 +359,8 @@ int wcn_voxelize_points_csr(const float* points, int64_t num_points, const int64
 
 int wcn_segment_reduce(const void* features, int64_t num_in, int32_t channels, int32_t dtype,
                        const int64_t* segment_offsets, const int64_t* indices_or_null,
-                       int64_t num_segments, int32_t mode, void* out, int64_t* argmax_or_null,
-                       void* stream);
+                       int64_t num_entries, int64_t num_segments, int32_t mode, void* out,
+                       int64_t* argmax_or_null, void* stream);
 
 int wcn_segment_reduce_bwd(const void* grad_out, int64_t num_segments, int32_t channels, int32_t dtype,
                            const int64_t* segment_offsets, const int64_t* segment_of_row, int64_t num_in,

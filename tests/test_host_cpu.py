@@ -319,11 +319,11 @@ def test_voxelisation_entry_points_reject_bad_arguments():
     assert L.wcn_voxelize_points_csr(fake, 10, ok, null, 2, 0.1, fake, 64, null, null, null, null, null,
                                      ctypes.byref(count), null) == -6
     offs = (ctypes.c_int64 * 2)(0, 5)
-    assert L.wcn_segment_reduce(fake, 5, 8, 7, offs, null, 1, 0, fake, null, null) == -1     # dtype
-    assert L.wcn_segment_reduce(fake, 5, 8, 0, offs, null, 1, 4, fake, null, null) == -1     # mode
-    assert L.wcn_segment_reduce(fake, 5, 0, 0, offs, null, 1, 0, fake, null, null) == -1     # channels
-    assert L.wcn_segment_reduce(fake, 5, 8, 0, None, null, 1, 0, fake, null, null) == -1
-    assert L.wcn_segment_reduce(fake, 5, 8, 0, offs, null, 0, 0, null, null, null) == 0      # nothing to do
+    assert L.wcn_segment_reduce(fake, 5, 8, 7, offs, null, 5, 1, 0, fake, null, null) == -1     # dtype
+    assert L.wcn_segment_reduce(fake, 5, 8, 0, offs, null, 5, 1, 4, fake, null, null) == -1     # mode
+    assert L.wcn_segment_reduce(fake, 5, 0, 0, offs, null, 5, 1, 0, fake, null, null) == -1     # channels
+    assert L.wcn_segment_reduce(fake, 5, 8, 0, None, null, 5, 1, 0, fake, null, null) == -1
+    assert L.wcn_segment_reduce(fake, 5, 8, 0, offs, null, 5, 0, 0, null, null, null) == 0      # nothing to do
     assert L.wcn_segment_reduce_bwd(fake, 1, 8, 0, offs, fake, 5, 2, null, fake, null) == -1  # max without argmax
     assert L.wcn_segment_reduce_bwd(fake, 1, 8, 0, offs, null, 5, 0, null, fake, null) == -1  # no segment ids
 

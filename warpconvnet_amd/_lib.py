@@ -60,7 +60,7 @@ SIGNATURES = {
     "wcn_unique_rows_csr": (ctypes.c_int, [_vp, _i64, _i32, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _i64p, _vp]),
     "wcn_voxelize_points_csr": (ctypes.c_int, [_vp, _i64, _i64p, _vp, _i32, ctypes.c_double, _vp, _sz, _vp, _vp,
                                                _vp, _vp, _vp, _i64p, _vp]),
-    "wcn_segment_reduce": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, _i64, _i32, _vp, _vp, _vp]),
+    "wcn_segment_reduce": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp]),
     "wcn_segment_reduce_bwd": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, _i64, _i32, _vp, _vp, _vp]),
 }
 

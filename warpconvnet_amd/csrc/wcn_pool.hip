@@ -170,15 +170,19 @@ template <typename T>
 __global__ void __launch_bounds__(256) segment_reduce(const T* __restrict__ X, int64_t num_in, int channels,
                                                       const int64_t* __restrict__ offsets,
                                                       const int64_t* __restrict__ indices,
-                                                      int64_t num_out, int mode, bool vec,
-                                                      T* __restrict__ out, int64_t* __restrict__ arg) {
+                                                      int64_t num_entries, int64_t num_out, int mode,
+                                                      bool vec, T* __restrict__ out,
+                                                      int64_t* __restrict__ arg) {
   constexpr int N = Piece<T>::N;
   const int pieces = (channels + N - 1) / N;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= num_out * pieces) return;
   const int64_t u = i / pieces;
   const int c0 = (int)(i % pieces) * N;
-  const int64_t begin = offsets[u], end = offsets[u + 1];
+  // offsets that do not fit the entry list are cut to it: nothing is read past its end
+  int64_t begin = offsets[u], end = offsets[u + 1];
+  begin = begin < 0 ? 0 : begin;
+  end = end > num_entries ? num_entries : end;
   float acc[N];
   int64_t who[N];
 #pragma unroll
@@ -419,12 +423,13 @@ void launch_pool_bwd(const void* dY, int64_t num_out, int channels, const WcnRow
 
 template <typename T>
 void launch_segment_reduce(const void* X, int64_t num_in, int channels, const int64_t* offsets,
-                           const int64_t* indices, int64_t num_out, int mode, bool vec, void* out,
-                           int64_t* arg, hipStream_t s) {
+                           const int64_t* indices, int64_t num_entries, int64_t num_out, int mode,
+                           bool vec, void* out, int64_t* arg, hipStream_t s) {
   const int pieces = (channels + Piece<T>::N - 1) / Piece<T>::N;
   const int64_t items = num_out * pieces;
   hipLaunchKernelGGL(segment_reduce<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
-                     (const T*)X, num_in, channels, offsets, indices, num_out, mode, vec, (T*)out, arg);
+                     (const T*)X, num_in, channels, offsets, indices, num_entries, num_out, mode, vec, (T*)out,
+                     arg);
 }
 
 template <typename T>
@@ -543,10 +548,10 @@ int wcn_sparse_pool_bwd(const void* grad_out, int64_t num_out, int32_t channels,
 
 int wcn_segment_reduce(const void* features, int64_t num_in, int32_t channels, int32_t dtype,
                        const int64_t* segment_offsets, const int64_t* indices_or_null,
-                       int64_t num_segments, int32_t mode, void* out, int64_t* argmax_or_null,
-                       void* stream) {
+                       int64_t num_entries, int64_t num_segments, int32_t mode, void* out,
+                       int64_t* argmax_or_null, void* stream) {
   if (dtype < 0 || dtype > 2 || mode < POOL_SUM || mode > POOL_MIN || channels < 1 || num_in < 0 ||
-      num_segments < 0 || channels > (1 << 20))
+      num_segments < 0 || channels > (1 << 20) || num_entries < 0)
     return WCN_ERR_INVALID_ARGUMENT;
   if (num_segments == 0) return WCN_OK;
   if (!out || !segment_offsets || (num_in > 0 && !features)) return WCN_ERR_INVALID_ARGUMENT;
@@ -555,15 +560,15 @@ int wcn_segment_reduce(const void* features, int64_t num_in, int32_t channels, i
   switch (dtype) {
     case WCN_DTYPE_F32:
       launch_segment_reduce<float>(features, num_in, channels, segment_offsets, indices_or_null,
-                                   num_segments, mode, vec, out, argmax_or_null, s);
+                                   num_entries, num_segments, mode, vec, out, argmax_or_null, s);
       break;
     case WCN_DTYPE_F16:
       launch_segment_reduce<_Float16>(features, num_in, channels, segment_offsets, indices_or_null,
-                                      num_segments, mode, vec, out, argmax_or_null, s);
+                                      num_entries, num_segments, mode, vec, out, argmax_or_null, s);
       break;
     default:
       launch_segment_reduce<__bf16>(features, num_in, channels, segment_offsets, indices_or_null,
-                                    num_segments, mode, vec, out, argmax_or_null, s);
+                                    num_entries, num_segments, mode, vec, out, argmax_or_null, s);
       break;
   }
   WCN_LAUNCH_CHECK();

@@ -58,8 +58,10 @@ class _SegmentReduceFunction(Function):
         m = len(offsets) - 1
         out = torch.empty((m, channels), dtype=x.dtype, device=x.device)
         arg = torch.empty((m, channels), dtype=torch.int64, device=x.device) if mode >= 2 else None
+        entries = n_in if indices is None else indices.shape[0]
         check(lib().wcn_segment_reduce(ptr(x), n_in, channels, DTYPE_CODE[x.dtype], ptr(offsets),
-                                       ptr(indices), m, mode, ptr(out), ptr(arg), stream_ptr(x.device)),
+                                       ptr(indices), entries, m, mode, ptr(out), ptr(arg),
+                                       stream_ptr(x.device)),
               "wcn_segment_reduce")
         ctx.saved = (offsets, indices, segment_of, arg)
         ctx.mode, ctx.n_in = mode, n_in
