@@ -191,3 +191,42 @@ def test_gradients_are_adjoints_at_benchmark_size():
     gx2, _ = sparse_conv_backward(y, x, w, km, need_weight_grad=False)
     km._symmetric = True
     assert rel_err(gx2.float().cpu().numpy(), gx.float().cpu().numpy()) <= 2e-3
+
+
+def test_every_device_result_is_bitwise_reproducible():
+    """No result depends on the order in which waves happen to run: maps, the contraction, both
+    gradients, pooling, the depthwise weight gradient and the point -> voxel grouping come out
+    bit for bit the same from two runs (the reductions run in a fixed order, nothing is summed
+    with floating-point atomics)."""
+    from warpconvnet_amd.geometry.coords.ops.voxel import voxel_downsample_csr_mapping
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_backward, sparse_conv_forward
+    from warpconvnet_amd.nn.functional.sparse_conv_depth import spatially_sparse_depthwise_conv
+    from warpconvnet_amd.nn.functional.sparse_pool import sparse_reduce
+    from warpconvnet_amd.ops.reductions import segment_reduction
+    items = [synthetic.indoor_scene(seed=300 + b, n_target=30_000, voxel_size=0.04) for b in range(2)]
+    bc = torch.as_tensor(synthetic.batch_indexed(items), device=DEV)
+    n = len(bc)
+    x = normal_features(n, 64, seed=1, dtype=torch.float16).to(DEV)
+    w = kaiming_weight(27, 64, 64, seed=2, dtype=torch.float16).to(DEV)
+    gy = normal_features(n, 64, seed=3, dtype=torch.float16).to(DEV)
+    wd = normal_features(27, 64, seed=4, dtype=torch.float16).to(DEV)
+    pts = torch.rand((200_000, 3), device=DEV, generator=torch.Generator(device=DEV).manual_seed(5)) * 4
+    pf = normal_features(200_000, 16, seed=6).to(DEV)
+
+    def run():
+        km = generate_kernel_map(bc.clone(), bc.clone(), (1, 1, 1), (3, 3, 3))
+        y = sparse_conv_forward(x, w, km, n)
+        gx, gw = sparse_conv_backward(gy, x, w, km)
+        xd = x.clone().requires_grad_(True)
+        wdp = wd.clone().requires_grad_(True)
+        spatially_sparse_depthwise_conv(xd, wdp, km, n).backward(gy)
+        pooled = sparse_reduce(_voxels(items, x.cpu()), 2, 2, "mean").feature_tensor
+        _, _, ci, co, tu = voxel_downsample_csr_mapping(pts, torch.tensor([0, 90_000, 200_000]), 0.05)
+        vf = segment_reduction(pf, co, "mean", indices=ci)
+        return [km.in_maps, km.out_maps, km.offsets, y, gx, gw, xd.grad, wdp.grad, pooled, ci, co,
+                tu.to_unique_indices, vf]
+
+    first, second = run(), run()
+    for i, (a, b) in enumerate(zip(first, second)):
+        assert torch.equal(a, b), i
