@@ -48,6 +48,12 @@ constexpr int NBW = TN / 16 / (THREADS / 256);  // 16-channel blocks per wave
 constexpr int A_ROWS = 128;  // gathered input rows resident in LDS (pairs per batch)
 constexpr int BATCH = 4;     // offsets per batch, at most
 
+// Up to 128 offsets of a kernel map (K + 1 <= 128) travel as a kernel argument.
+constexpr int OFFSETS_BY_VALUE = 128;
+struct OffsetsByValue {
+  int64_t v[OFFSETS_BY_VALUE];
+};
+
 // The kernels multiply by tiles Wt[k][n][c] (n: channel of the result, c: channel of the gathered
 // rows), converted to T and zero padded to (c_out_pad, c_in_pad).
 //   forward        Wt[k][n][c] = W[k][c][n]            (W is (K, c_in, c_out))
@@ -57,8 +63,14 @@ template <typename T, typename WT>
 __global__ void __launch_bounds__(256) conv_prep_weight(const WT* __restrict__ W, int K, int c_in,
                                                         int c_out, int c_in_pad, int c_out_pad,
                                                         int as_stored, int flip_k,
-                                                        T* __restrict__ Wt, uint32_t* __restrict__ zeros) {
-  if (blockIdx.x == 0) zeros[threadIdx.x] = 0u;  // 256 threads x 4 bytes
+                                                        T* __restrict__ Wt, uint32_t* __restrict__ zeros,
+                                                        int64_t* __restrict__ offsets_dst,
+                                                        int n_offsets, OffsetsByValue ov) {
+  if (blockIdx.x == 0) {
+    zeros[threadIdx.x] = 0u;  // 256 threads x 4 bytes
+    // the map's offsets, handed over in the kernel arguments (saves a copy command per call)
+    if ((int)threadIdx.x < n_offsets) offsets_dst[threadIdx.x] = ov.v[threadIdx.x];
+  }
   const int64_t total = (int64_t)K * c_out_pad * c_in_pad;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
@@ -1083,17 +1095,21 @@ thread_local hipEvent_t g_time_stop = nullptr;
 
 template <typename T>
 int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dtype, int as_stored,
-                int flip_k, hipStream_t s) {
+                int flip_k, const int64_t* host_offsets_or_null, hipStream_t s) {
+  OffsetsByValue ov;
+  const int n_ov = host_offsets_or_null ? a.K + 1 : 0;
+  for (int i = 0; i < OFFSETS_BY_VALUE; ++i) ov.v[i] = i < n_ov ? host_offsets_or_null[i] : 0;
   const int64_t total = (int64_t)a.K * a.c_out_pad * a.c_in_pad;
   const int pgrid = (int)std::min<int64_t>(4096, (total + 255) / 256);
   if (weight_dtype == dtype) {
     hipLaunchKernelGGL((conv_prep_weight<T, T>), dim3(pgrid), dim3(256), 0, s, (const T*)weight,
                        a.K, a.c_in, a.c_out, a.c_in_pad, a.c_out_pad, as_stored, flip_k, (T*)a.Wt,
-                       (uint32_t*)a.zeros);
+                       (uint32_t*)a.zeros, const_cast<int64_t*>(a.offsets), n_ov, ov);
   } else {
     hipLaunchKernelGGL((conv_prep_weight<T, float>), dim3(pgrid), dim3(256), 0, s,
                        (const float*)weight, a.K, a.c_in, a.c_out, a.c_in_pad, a.c_out_pad,
-                       as_stored, flip_k, (T*)a.Wt, (uint32_t*)a.zeros);
+                       as_stored, flip_k, (T*)a.Wt, (uint32_t*)a.zeros, const_cast<int64_t*>(a.offsets),
+                       n_ov, ov);
   }
   const dim3 grid((unsigned)((a.num_out + ROWS - 1) / ROWS), (unsigned)(a.c_out_pad / TN));
   constexpr int NC = WCN_RING_NC;  // multiplying waves per workgroup of the ring kernel
@@ -1238,7 +1254,12 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   hipStream_t s = (hipStream_t)stream;
   ConvWorkspace w;
   conv_layout(workspace, num_out, num_offsets, c_in, c_out, dtype, out_maps_ascend ? -1 : L, &w);
-  if (hipMemcpyAsync(w.offsets, host_offsets, sizeof(int64_t) * (size_t)(num_offsets + 1),
+  // With the builder's group starts at hand nothing before the weight preparation reads the
+  // offsets on the device, and that kernel can bring them along in its arguments.
+  const bool offsets_by_value =
+      out_maps_ascend && group_start_or_null && num_offsets + 1 <= OFFSETS_BY_VALUE;
+  if (!offsets_by_value &&
+      hipMemcpyAsync(w.offsets, host_offsets, sizeof(int64_t) * (size_t)(num_offsets + 1),
                      hipMemcpyHostToDevice, s) != hipSuccess)
     return WCN_ERR_LAUNCH;
 
@@ -1305,11 +1326,14 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   a.split = (a.vec_in && w.partial != nullptr) ? 1 : 0;
   switch (dtype) {
     case WCN_DTYPE_F32:
-      return launch_conv<float>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, s);
+      return launch_conv<float>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets,
+                                offsets_by_value ? host_offsets : nullptr, s);
     case WCN_DTYPE_F16:
-      return launch_conv<_Float16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, s);
+      return launch_conv<_Float16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets,
+                                  offsets_by_value ? host_offsets : nullptr, s);
     default:
-      return launch_conv<__bf16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, s);
+      return launch_conv<__bf16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets,
+                                  offsets_by_value ? host_offsets : nullptr, s);
   }
 }
 
