@@ -188,6 +188,16 @@ int wcn_read_small(void* host_dst, const void* device_src, size_t bytes, hipStre
 int wcn_read_early_begin(const void* device_src, size_t bytes, hipStream_t stream);
 int wcn_read_early_end(void* host_dst, const void* device_src, size_t bytes, hipStream_t stream);
 
+// A result the device writes straight into pinned host memory (no copy command): `begin` hands out
+// this thread's mailbox (device-visible address of up to 16 KiB - 8 bytes of payload behind an
+// 8-byte sequence word) and a fresh sequence number; the kernel writes the payload, a system-scope
+// fence, then the sequence number into word 0.  `end` polls word 0 (and `done`, an event recorded
+// after the kernel, so that a kernel that never wrote cannot stall the host: it then returns
+// WCN_ERR_LAUNCH and the caller reads the device copy instead) and copies the payload out.
+int wcn_mailbox_begin(int64_t** device_visible_box, int64_t* sequence);
+int wcn_mailbox_mark(hipStream_t stream);  // records `done` behind the writing kernel
+int wcn_mailbox_end(void* host_dst, size_t payload_bytes, int64_t sequence);
+
 // Output-row form of a pair list (rows of the map grouped by output row, inside a row ascending
 // in kernel offset): row_mask[m] has bit k set if offset k has a pair for output row m,
 // row_in[row_ptr[m] .. row_ptr[m + 1]) are the input rows of those pairs.  Built by

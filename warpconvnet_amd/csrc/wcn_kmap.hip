@@ -333,6 +333,8 @@ struct KmapFinish {  // null `result`: no finishing step
   int32_t* ticket;              // zero before the launch; left at zero
   const WcnTableHeader* hdr;
   int32_t K;
+  int64_t* mailbox;             // pinned host memory (or null): the same K + 3 words behind a sequence word
+  int64_t sequence;
 };
 
 __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ groups, int64_t G,
@@ -398,14 +400,30 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
       const int64_t t = __shfl_up(v, d, 64);
       if (lane >= d) v += t;
     }
-    if (k < fin.K) fin.result[k + 1] = run + v;
+    if (k < fin.K) {
+      fin.result[k + 1] = run + v;
+      if (fin.mailbox) fin.mailbox[1 + k + 1] = run + v;
+    }
     run += __shfl(v, 63, 64);
   }
   if (lane == 0) {
+    const int64_t status = fin.hdr->status;
+    const int64_t blocks = (int64_t)fin.hdr->num_blocks | ((int64_t)(WCN_HAS_DUPLICATES(fin.hdr) ? 1 : 0) << 32);
     fin.result[0] = 0;
-    fin.result[fin.K + 1] = fin.hdr->status;
-    fin.result[fin.K + 2] = (int64_t)fin.hdr->num_blocks | ((int64_t)(WCN_HAS_DUPLICATES(fin.hdr) ? 1 : 0) << 32);
+    fin.result[fin.K + 1] = status;
+    fin.result[fin.K + 2] = blocks;
+    if (fin.mailbox) {
+      fin.mailbox[1] = 0;
+      fin.mailbox[1 + fin.K + 1] = status;
+      fin.mailbox[1 + fin.K + 2] = blocks;
+    }
     *fin.ticket = 0;
+  }
+  if (fin.mailbox) {
+    // the host polls the sequence word: everything this wave wrote into the mailbox is visible to
+    // it before the word changes
+    __threadfence_system();
+    if (lane == 0) __hip_atomic_store(&fin.mailbox[0], fin.sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 
@@ -558,13 +576,16 @@ __global__ void stride_finish(int64_t* __restrict__ result, const int32_t* __res
 
 // Row-wise exclusive scan, shared with the contraction's map conversion.
 void wcn_scan_rows_launch(int32_t* groups, int64_t G, int rows, int64_t* row_total, hipStream_t s) {
-  const KmapFinish none = {nullptr, nullptr, nullptr, 0};
+  const KmapFinish none = {nullptr, nullptr, nullptr, 0, nullptr, 0};
   hipLaunchKernelGGL(kmap_scan_rows, dim3(rows), dim3(1024), 0, s, groups, G, row_total, none);
 }
 
 // what the last wcn_kmap_read_result of this host thread learned about the table (bit 0: some
 // key was inserted more than once)
 static thread_local int32_t g_last_table_flags = 0;
+// the mailbox write the last count call of this thread armed, and the result block it mirrors
+static thread_local int64_t g_pending_sequence = 0;
+static thread_local const void* g_pending_result = nullptr;
 
 extern "C" {
 
@@ -591,12 +612,26 @@ int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const in
   } else {
     hipLaunchKernelGGL(kmap_zero_ticket, dim3(1), dim3(1), 0, s, w.ticket);
   }
-  const KmapFinish fin = {w.result, w.ticket, v.hdr, g.K};
+  // The scan's finishing wave writes the result into device memory (the emit pass reads it there)
+  // and into this thread's pinned mailbox, where wcn_kmap_read_result picks it up without a copy
+  // command on the stream, ahead of anything the caller enqueues next (an emit pass into buffers of
+  // assumed size, say).
+  int64_t* box = nullptr;
+  int64_t sequence = 0;
+  if (wcn_mailbox_begin(&box, &sequence) != WCN_OK) {  // no mailbox: a copy command instead
+    box = nullptr;
+    sequence = 0;
+  }
+  g_pending_sequence = sequence;
+  g_pending_result = w.result;
+  const KmapFinish fin = {w.result, w.ticket, v.hdr, g.K, box, sequence};
   hipLaunchKernelGGL(kmap_scan_rows, dim3(g.K + 1), dim3(1024), 0, s, w.groups, w.G, w.row_total, fin);
   WCN_LAUNCH_CHECK();
-  // the result's trip to the host starts here, ahead of anything the caller enqueues next (an emit
-  // pass into buffers of assumed size, say); wcn_kmap_read_result collects it
-  if (wcn_read_early_begin(w.result, sizeof(int64_t) * (size_t)(g.K + 3), s) != WCN_OK) return WCN_ERR_LAUNCH;
+  if (box) {
+    if (wcn_mailbox_mark(s) != WCN_OK) return WCN_ERR_LAUNCH;
+  } else if (wcn_read_early_begin(w.result, sizeof(int64_t) * (size_t)(g.K + 3), s) != WCN_OK) {
+    return WCN_ERR_LAUNCH;
+  }
   return WCN_OK;
 }
 
@@ -610,7 +645,13 @@ int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_off
   kmap_layout(const_cast<void*>(workspace), num_out, num_offsets, &w);
   int64_t tmp[WCN_MAX_OFFSETS + 3];
   const size_t bytes = sizeof(int64_t) * (size_t)(num_offsets + 3);
-  if (wcn_read_early_end(tmp, w.result, bytes, (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
+  // from the mailbox the count call armed; otherwise (another thread, a count call that failed
+  // half-way) from the device copy
+  const int64_t sequence = g_pending_result == (const void*)w.result ? g_pending_sequence : 0;
+  if (sequence != 0) g_pending_sequence = 0;
+  if (sequence == 0 || wcn_mailbox_end(tmp, bytes, sequence) != WCN_OK) {
+    if (wcn_read_early_end(tmp, w.result, bytes, (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
+  }
   for (int k = 0; k <= num_offsets; ++k) host_offsets[k] = tmp[k];
   g_last_table_flags = (int32_t)((tmp[num_offsets + 2] >> 32) & 1);
   const int st = wcn_table_status_from_bits((int32_t)tmp[num_offsets + 1]);
@@ -676,7 +717,7 @@ int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_strid
                        (int4*)nullptr, (int32_t*)nullptr);
   }
   {
-    const KmapFinish none = {nullptr, nullptr, nullptr, 0};
+    const KmapFinish none = {nullptr, nullptr, nullptr, 0, nullptr, 0};
     hipLaunchKernelGGL(kmap_scan_rows, dim3(1), dim3(1024), 0, s, w.groups, w.G, w.result + 2, none);
   }
   hipLaunchKernelGGL(stride_finish, dim3(1), dim3(64), 0, s, w.result, w.groups, w.G, v.hdr);

@@ -329,6 +329,61 @@ int wcn_read_early_end(void* host_dst, const void* device_src, size_t bytes, hip
   return WCN_OK;
 }
 
+namespace {
+constexpr size_t kMailboxBytes = 16384;
+thread_local int64_t* g_box = nullptr;        // pinned, coherent, mapped
+thread_local hipEvent_t g_box_done = nullptr;
+thread_local int g_box_device = -1;
+thread_local int64_t g_box_sequence = 0;
+}  // namespace
+
+int wcn_mailbox_begin(int64_t** device_visible_box, int64_t* sequence) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return WCN_ERR_LAUNCH;
+  if (!g_box) {
+    void* p = nullptr;
+    if (hipHostMalloc(&p, kMailboxBytes, hipHostMallocCoherent | hipHostMallocMapped) != hipSuccess)
+      return WCN_ERR_LAUNCH;
+    g_box = (int64_t*)p;
+    g_box[0] = 0;
+  }
+  if (!g_box_done || g_box_device != device) {
+    if (g_box_done) (void)hipEventDestroy(g_box_done);
+    if (hipEventCreateWithFlags(&g_box_done, hipEventDisableTiming) != hipSuccess) {
+      g_box_done = nullptr;
+      return WCN_ERR_LAUNCH;
+    }
+    g_box_device = device;
+  }
+  void* dev = nullptr;
+  if (hipHostGetDevicePointer(&dev, g_box, 0) != hipSuccess) return WCN_ERR_LAUNCH;
+  *device_visible_box = (int64_t*)dev;
+  *sequence = ++g_box_sequence;
+  return WCN_OK;
+}
+
+int wcn_mailbox_mark(hipStream_t stream) {
+  if (!g_box_done) return WCN_ERR_LAUNCH;
+  return hipEventRecord(g_box_done, stream) == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
+}
+
+int wcn_mailbox_end(void* host_dst, size_t payload_bytes, int64_t sequence) {
+  if (!g_box || !g_box_done || payload_bytes + 8 > kMailboxBytes) return WCN_ERR_INVALID_ARGUMENT;
+  volatile int64_t* word0 = g_box;
+  for (;;) {
+    if (*word0 == sequence) break;
+    const hipError_t e = hipEventQuery(g_box_done);
+    if (e == hipErrorNotReady) continue;
+    if (e != hipSuccess) return WCN_ERR_LAUNCH;
+    // the kernel is over: its write must be there by now, or it never happened
+    if (*word0 == sequence) break;
+    return WCN_ERR_LAUNCH;
+  }
+  __atomic_thread_fence(__ATOMIC_ACQUIRE);
+  memcpy(host_dst, (const void*)(g_box + 1), payload_bytes);
+  return WCN_OK;
+}
+
 int wcn_table_status_from_bits(int32_t bits) {
   if (bits & WCN_DEV_RANGE) return WCN_ERR_COORD_RANGE;
   if (bits & WCN_DEV_OVERFLOW) return WCN_ERR_TABLE_OVERFLOW;
