@@ -177,6 +177,27 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
                         const int32_t* group_start_or_null, void* out, int64_t num_out,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* wcn_sparse_conv_fwd for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments and results as wcn_sparse_conv_fwd, minus the workspace: the scratch memory is a
+ * device-resident array of WCN_CONV_STATIC_SCRATCH_BYTES inside the library (each GPU the library
+ * runs on holds it until the process ends).  The call enqueues kernels only: no allocation, no
+ * free, no copy command.  It returns WCN_ERR_WORKSPACE when
+ * wcn_conv_workspace_bytes(num_out, K, c_in, c_out, dtype, L, out_maps_ascend) exceeds that size
+ * and WCN_ERR_INVALID_ARGUMENT for more than 127 offsets (they travel in kernel arguments).
+ * Every call on a GPU uses that GPU's one array: calls that overlap on the same GPU (different
+ * streams or host threads) race.  The first call on a device looks the array's address up and
+ * must therefore be made outside graph capture. */
+#define WCN_CONV_STATIC_SCRATCH_BYTES (4u << 20)
+
+int wcn_sparse_conv_fwd_static(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                               const void* weight, int32_t weight_dtype, int32_t num_offsets,
+                               int32_t c_out, const void* bias_or_null, const int32_t* in_maps,
+                               const int32_t* out_maps, const int64_t* host_offsets,
+                               int32_t identity_offset, int32_t out_maps_ascend,
+                               const int32_t* group_start_or_null, void* out, int64_t num_out,
+                               void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Gradients of the contraction.  Replace the per-offset loops of the reference backward
  * (sparse_conv.py:314-355 explicit, :418-492 implicit, :547-627 CUTLASS) and the native calls

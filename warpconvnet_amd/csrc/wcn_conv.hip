@@ -30,6 +30,7 @@
 // L2 / Infinity Cache when the voxel order has locality), the map once (8 L), the output once
 // (M * C_out * s); the weights (K * C_in * C_out * s) stay cache resident.
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "wcn_common.h"
@@ -1093,9 +1094,10 @@ inline size_t conv_layout(void* base, int64_t num_out, int K, int c_in, int c_ou
 thread_local hipEvent_t g_time_start = nullptr;
 thread_local hipEvent_t g_time_stop = nullptr;
 
+// Weight tiles, the block of zeros and (when given) the map's offsets: first launch of every call.
 template <typename T>
-int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dtype, int as_stored,
-                int flip_k, const int64_t* host_offsets_or_null, hipStream_t s) {
+void launch_prep(const ConvArgs& a, const void* weight, int weight_dtype, int dtype, int as_stored,
+                 int flip_k, const int64_t* host_offsets_or_null, hipStream_t s) {
   OffsetsByValue ov;
   const int n_ov = host_offsets_or_null ? a.K + 1 : 0;
   for (int i = 0; i < OFFSETS_BY_VALUE; ++i) ov.v[i] = i < n_ov ? host_offsets_or_null[i] : 0;
@@ -1111,6 +1113,10 @@ int launch_conv(const ConvArgs& a, const void* weight, int weight_dtype, int dty
                        as_stored, flip_k, (T*)a.Wt, (uint32_t*)a.zeros, const_cast<int64_t*>(a.offsets),
                        n_ov, ov);
   }
+}
+
+template <typename T>
+int launch_conv(const ConvArgs& a, hipStream_t s) {
   const dim3 grid((unsigned)((a.num_out + ROWS - 1) / ROWS), (unsigned)(a.c_out_pad / TN));
   constexpr int NC = WCN_RING_NC;  // multiplying waves per workgroup of the ring kernel
   if (a.vec_in) {
@@ -1225,14 +1231,16 @@ size_t wcn_conv_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_
 }
 
 // Shared body of the forward product and the input gradient.  weight_as_stored / flip_offsets
-// choose how the caller's weight becomes the kernels' tiles (see conv_prep_weight).
+// choose how the caller's weight becomes the kernels' tiles (see conv_prep_weight).  With
+// `no_copy_commands` the call enqueues kernels only (the offsets must then fit the kernel
+// arguments of the weight preparation).
 static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
                     const void* weight, int32_t weight_dtype, int32_t num_offsets, int32_t c_out,
                     const void* bias_or_null, const int32_t* in_maps, const int32_t* out_maps,
                     const int64_t* host_offsets, int32_t identity_offset, int32_t out_maps_ascend,
                     const int32_t* group_start_or_null, void* out, int64_t num_out,
                     void* workspace, size_t workspace_bytes, int weight_as_stored,
-                    int flip_offsets, void* stream) {
+                    int flip_offsets, bool no_copy_commands, void* stream) {
   if (dtype < 0 || dtype > 2 || (weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32))
     return WCN_ERR_INVALID_ARGUMENT;
   if (num_in < 0 || num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || c_in < 1 ||
@@ -1254,16 +1262,45 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   hipStream_t s = (hipStream_t)stream;
   ConvWorkspace w;
   conv_layout(workspace, num_out, num_offsets, c_in, c_out, dtype, out_maps_ascend ? -1 : L, &w);
-  // With the builder's group starts at hand nothing before the weight preparation reads the
-  // offsets on the device, and that kernel can bring them along in its arguments.
-  const bool offsets_by_value =
-      out_maps_ascend && group_start_or_null && num_offsets + 1 <= OFFSETS_BY_VALUE;
-  if (!offsets_by_value &&
-      hipMemcpyAsync(w.offsets, host_offsets, sizeof(int64_t) * (size_t)(num_offsets + 1),
-                     hipMemcpyHostToDevice, s) != hipSuccess)
-    return WCN_ERR_LAUNCH;
+  // Up to 127 offsets reach the device in the arguments of the weight preparation, which is the
+  // first launch of the call: no copy command.
+  const bool offsets_by_value = num_offsets + 1 <= OFFSETS_BY_VALUE;
+  if (!offsets_by_value) {
+    if (no_copy_commands) return WCN_ERR_INVALID_ARGUMENT;
+    if (hipMemcpyAsync(w.offsets, host_offsets, sizeof(int64_t) * (size_t)(num_offsets + 1),
+                       hipMemcpyHostToDevice, s) != hipSuccess)
+      return WCN_ERR_LAUNCH;
+  }
 
   ConvArgs a;
+  a.offsets = w.offsets;
+  a.X = features;
+  a.Wt = w.Wt;
+  a.zeros = w.zeros;
+  a.bias = bias_or_null;
+  a.out = out;
+  a.num_in = num_in;
+  a.num_out = num_out;
+  a.G = w.G;
+  a.K = num_offsets;
+  a.c_in = c_in;
+  a.c_out = c_out;
+  a.c_in_pad = w.c_in_pad;
+  a.c_out_pad = w.c_out_pad;
+  a.identity = identity_offset;
+  const int64_t* by_value = offsets_by_value ? host_offsets : nullptr;
+  switch (dtype) {
+    case WCN_DTYPE_F32:
+      launch_prep<float>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, by_value, s);
+      break;
+    case WCN_DTYPE_F16:
+      launch_prep<_Float16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, by_value, s);
+      break;
+    default:
+      launch_prep<__bf16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, by_value, s);
+      break;
+  }
+
   a.in_maps = in_maps;
   a.out_maps = out_maps;
   a.group_start = group_start_or_null;
@@ -1303,21 +1340,6 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
                        out_maps, (const int64_t*)w.offsets, num_offsets, w.G, w.group_start);
     a.group_start = w.group_start;
   }
-  a.offsets = w.offsets;
-  a.X = features;
-  a.Wt = w.Wt;
-  a.zeros = w.zeros;
-  a.bias = bias_or_null;
-  a.out = out;
-  a.num_in = num_in;
-  a.num_out = num_out;
-  a.G = w.G;
-  a.K = num_offsets;
-  a.c_in = c_in;
-  a.c_out = c_out;
-  a.c_in_pad = w.c_in_pad;
-  a.c_out_pad = w.c_out_pad;
-  a.identity = identity_offset;
   const size_t es = elem_size(dtype);
   a.vec_in = (((size_t)c_in * es) % 16 == 0 && ((uintptr_t)features % 16) == 0) ? 1 : 0;
   a.vec_out = (((size_t)c_out * es) % 16 == 0 && ((uintptr_t)out % 16) == 0) ? 1 : 0;
@@ -1326,15 +1348,60 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   a.split = (a.vec_in && w.partial != nullptr) ? 1 : 0;
   switch (dtype) {
     case WCN_DTYPE_F32:
-      return launch_conv<float>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets,
-                                offsets_by_value ? host_offsets : nullptr, s);
+      return launch_conv<float>(a, s);
     case WCN_DTYPE_F16:
-      return launch_conv<_Float16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets,
-                                  offsets_by_value ? host_offsets : nullptr, s);
+      return launch_conv<_Float16>(a, s);
     default:
-      return launch_conv<__bf16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets,
-                                  offsets_by_value ? host_offsets : nullptr, s);
+      return launch_conv<__bf16>(a, s);
   }
+}
+
+// ---- the contraction for callers that cannot allocate ------------------------------------------
+// One device-resident scratch array per GPU serves as the workspace of wcn_sparse_conv_fwd_static.
+// Host code never uses the array's name as an address: the per-device address comes from
+// hipGetSymbolAddress, once per device, and is what the kernels receive.
+static __device__ __align__(256) unsigned char scratch[WCN_CONV_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device (looked up on the first call on that device).
+int static_scratch(void** ptr) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return WCN_ERR_LAUNCH;
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return WCN_ERR_LAUNCH;
+    g_scratch_ptr[device] = p;
+  }
+  *ptr = g_scratch_ptr[device];
+  return WCN_OK;
+}
+}  // namespace
+
+int wcn_sparse_conv_fwd_static(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                               const void* weight, int32_t weight_dtype, int32_t num_offsets,
+                               int32_t c_out, const void* bias_or_null, const int32_t* in_maps,
+                               const int32_t* out_maps, const int64_t* host_offsets,
+                               int32_t identity_offset, int32_t out_maps_ascend,
+                               const int32_t* group_start_or_null, void* out, int64_t num_out,
+                               void* stream) {
+  if (!host_offsets || num_offsets < 1 || num_offsets + 1 > OFFSETS_BY_VALUE)
+    return WCN_ERR_INVALID_ARGUMENT;
+  const size_t need = wcn_conv_workspace_bytes(num_out, num_offsets, c_in, c_out, dtype,
+                                               host_offsets[num_offsets], out_maps_ascend);
+  if (need == 0) return WCN_ERR_INVALID_ARGUMENT;
+  if (need > (size_t)WCN_CONV_STATIC_SCRATCH_BYTES) return WCN_ERR_WORKSPACE;
+  void* ws = nullptr;
+  const int st = static_scratch(&ws);
+  if (st != WCN_OK) return st;
+  return conv_run(features, num_in, c_in, dtype, weight, weight_dtype, num_offsets, c_out,
+                  bias_or_null, in_maps, out_maps, host_offsets, identity_offset, out_maps_ascend,
+                  group_start_or_null, out, num_out, ws, WCN_CONV_STATIC_SCRATCH_BYTES, 0, 0, true,
+                  stream);
 }
 
 int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
@@ -1346,7 +1413,7 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
                         void* workspace, size_t workspace_bytes, void* stream) {
   return conv_run(features, num_in, c_in, dtype, weight, weight_dtype, num_offsets, c_out,
                   bias_or_null, in_maps, out_maps, host_offsets, identity_offset, out_maps_ascend,
-                  group_start_or_null, out, num_out, workspace, workspace_bytes, 0, 0, stream);
+                  group_start_or_null, out, num_out, workspace, workspace_bytes, 0, 0, false, stream);
 }
 
 int wcn_sparse_conv_dgrad(const void* grad_out, int64_t num_out, int32_t c_out, int32_t dtype,
@@ -1363,13 +1430,14 @@ int wcn_sparse_conv_dgrad(const void* grad_out, int64_t num_out, int32_t c_out, 
     return conv_run(grad_out, num_out, c_out, dtype, weight, weight_dtype, num_offsets, c_in,
                     nullptr, in_maps, out_maps, host_offsets,
                     identity_offset < 0 ? -1 : num_offsets - 1 - identity_offset, 1,
-                    group_start_or_null, grad_in, num_in, workspace, workspace_bytes, 1, 1, stream);
+                    group_start_or_null, grad_in, num_in, workspace, workspace_bytes, 1, 1, false,
+                    stream);
   }
   // in general: the same contraction over the map with in and out exchanged
   return conv_run(grad_out, num_out, c_out, dtype, weight, weight_dtype, num_offsets, c_in, nullptr,
                   out_maps, in_maps, host_offsets, identity_offset, in_maps_ascend,
                   in_maps_ascend ? group_start_or_null : nullptr, grad_in, num_in, workspace,
-                  workspace_bytes, 1, 0, stream);
+                  workspace_bytes, 1, 0, false, stream);
 }
 
 }  // extern "C"
