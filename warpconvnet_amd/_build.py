@@ -21,21 +21,36 @@ HIPCC_FLAGS = [
 ]
 
 
-def build_library(verbose: bool = False) -> str:
-    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    sources = sorted(glob.glob(os.path.join(_PKG, "csrc", "*.hip")))
-    if not sources:
-        raise RuntimeError("no HIP sources found under csrc/")
-    cmd = [hipcc, *HIPCC_FLAGS, "-o", LIB_PATH, *sources]
-    if verbose:
-        print(" ".join(cmd))
+def _run(cmd):
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     noise = "is not a recognized feature for this target"
     log = "\n".join(l for l in proc.stdout.splitlines() if noise not in l)
     if proc.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{log}")
-    if verbose and log.strip():
-        print(log)
+        raise RuntimeError(f"hipcc failed ({proc.returncode}): {' '.join(cmd)}\n{log}")
+    return log
+
+
+def build_library(verbose: bool = False) -> str:
+    """Every source file is compiled to an object of its own (in parallel), then linked."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    sources = sorted(glob.glob(os.path.join(_PKG, "csrc", "*.hip")))
+    if not sources:
+        raise RuntimeError("no HIP sources found under csrc/")
+    objdir = os.path.join(_PKG, "build")
+    os.makedirs(objdir, exist_ok=True)
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    objects = [os.path.join(objdir, os.path.basename(src)[:-4] + ".o") for src in sources]
+    cmds = [[hipcc, *compile_flags, "-c", "-o", obj, src] for src, obj in zip(sources, objects)]
+    with ThreadPoolExecutor(max_workers=min(8, len(cmds))) as pool:
+        logs = list(pool.map(_run, cmds))
+    logs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", LIB_PATH, *objects]))
+    if verbose:
+        for cmd in cmds:
+            print(" ".join(cmd))
+        text = "\n".join(l for l in logs if l.strip())
+        if text:
+            print(text)
     return LIB_PATH
 
 
