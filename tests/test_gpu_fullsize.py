@@ -122,3 +122,24 @@ def test_cfg5b_wide_channels_small_map():
     want = explicit_gemm_forward(x, w, torch.as_tensor(im), torch.as_tensor(om), off, iden, n,
                                  compute_dtype=torch.float32)
     assert rel_err(got.float().cpu().numpy(), want.float().numpy()) <= 1e-2
+
+
+def test_cfg1_spheres_fp32_contraction_matches_oracle(oracle):
+    """configs[0] at its own size: 3x3x3, 32 -> 32, fp32, ~100k voxels on 3 spheres at 1 cm.  The
+    kernel map is the oracle's bit for bit and the contraction matches the fp64 oracle <= 1e-5."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    from helpers import normal_features
+    bc = synthetic.batch_indexed([synthetic.spheres_scene(0, 100_000, 0.01)])
+    n = len(bc)
+    assert n == 100_000
+    coords = torch.as_tensor(bc, device=DEV)
+    km = generate_kernel_map(coords, coords, (1, 1, 1), (3, 3, 3))
+    im, om, off, iden = oracle.kernel_map(bc, bc, (3, 3, 3))
+    assert np.array_equal(km.in_maps.cpu().numpy(), im) and np.array_equal(km.out_maps.cpu().numpy(), om)
+    assert np.array_equal(km.offsets.numpy().astype(np.int64), off) and km.identity_map_index == iden == 13
+    x = normal_features(n, 32, seed=21)
+    w = kaiming_weight(27, 32, 32, seed=22)
+    got = sparse_conv_forward(x.to(DEV), w.to(DEV), km, n)
+    want = oracle.explicit_conv_f64(x.double().numpy(), w.double().numpy(), im, om, off, iden, n)
+    assert rel_err(got.cpu().numpy(), want) <= 1e-5

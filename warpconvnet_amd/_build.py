@@ -30,6 +30,39 @@ def _run(cmd):
     return log
 
 
+# Sources whose kernels issue loads in inline assembly and wait for them by count: a register the
+# compiler spills (or otherwise moves) while such a load is still in flight would be overwritten
+# later by the landing data.  These files must compile without any scratch memory.
+NO_SCRATCH_SOURCES = ("wcn_conv_pack.hip",)
+_REMARK = "-Rpass-analysis=kernel-resource-usage"
+
+
+def _extra_flags(src):
+    return [_REMARK] if os.path.basename(src) in NO_SCRATCH_SOURCES else []
+
+
+def _without_remarks(log):
+    return "\n".join(l for l in log.splitlines() if _REMARK not in l)
+
+
+def _check_no_scratch(src, log):
+    if os.path.basename(src) not in NO_SCRATCH_SOURCES:
+        return
+    name, seen = None, 0
+    for line in log.splitlines():
+        if "remark: Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line or "VGPRs Spill:" in line:
+            seen += 1
+            value = int(line.split(":")[-1].split("[")[0].strip())
+            if value != 0:
+                raise RuntimeError(f"{os.path.basename(src)}: kernel {name} uses scratch memory / spills vector "
+                                   f"registers ({line.split('remark:')[1].strip()}); its hand-counted loads "
+                                   "make that unsafe")
+    if seen == 0:
+        raise RuntimeError(f"{os.path.basename(src)}: no resource-usage remarks found; cannot vouch for its kernels")
+
+
 def build_library(verbose: bool = False) -> str:
     """Every source file is compiled to an object of its own (in parallel), then linked."""
     from concurrent.futures import ThreadPoolExecutor
@@ -41,9 +74,13 @@ def build_library(verbose: bool = False) -> str:
     os.makedirs(objdir, exist_ok=True)
     compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
     objects = [os.path.join(objdir, os.path.basename(src)[:-4] + ".o") for src in sources]
-    cmds = [[hipcc, *compile_flags, "-c", "-o", obj, src] for src, obj in zip(sources, objects)]
+    cmds = [[hipcc, *compile_flags, *_extra_flags(src), "-c", "-o", obj, src]
+            for src, obj in zip(sources, objects)]
     with ThreadPoolExecutor(max_workers=min(8, len(cmds))) as pool:
         logs = list(pool.map(_run, cmds))
+    for src, log in zip(sources, logs):
+        _check_no_scratch(src, log)
+    logs = [_without_remarks(log) for log in logs]
     logs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", LIB_PATH, *objects]))
     if verbose:
         for cmd in cmds:

@@ -30,10 +30,13 @@
 // L2 / Infinity Cache when the voxel order has locality), the map once (8 L), the output once
 // (M * C_out * s); the weights (K * C_in * C_out * s) stay cache resident.
 #include <algorithm>
+#include <cstdlib>
 #include <mutex>
+#include <string>
 #include <type_traits>
 
 #include "wcn_common.h"
+#include "wcn_conv_args.h"
 #include "wcn_mma.h"
 
 void wcn_scan_rows_launch(int32_t* groups, int64_t G, int rows, int64_t* row_total, hipStream_t s);
@@ -85,28 +88,6 @@ __global__ void __launch_bounds__(256) conv_prep_weight(const WT* __restrict__ W
     Wt[i] = from_float<T>(v);
   }
 }
-
-struct ConvArgs {
-  const void* X;
-  const void* Wt;
-  const void* zeros;           // 1 KiB of zeros (source of loads that have nothing to fetch)
-  const void* bias;            // same dtype as X, or null
-  const int32_t* in_maps;      // pair lists; inside every offset out_maps ascends
-  const int32_t* out_maps;
-  const int64_t* offsets;      // (K + 1), device
-  const int32_t* group_start;  // (K, G + 1): pairs of offset k below output row 64 * g
-  void* out;
-  int64_t num_in, num_out, G;
-  int32_t K, c_in, c_out, c_in_pad, c_out_pad, identity;
-  int32_t vec_in;   // feature rows are 16-byte aligned and a whole number of 16-byte vectors
-  int32_t vec_out;  // same for output rows
-  int32_t flat_in;  // c_in is a multiple of the staged row and the feature matrix is below 4 GiB
-  // Few output tiles and several slices of input channels (small maps with wide features): the
-  // slices go to different workgroups (blockIdx.z), each writes its fp32 sums to
-  // partial[slice][row][c_out_pad] and conv_split_reduce adds them in slice order.
-  int32_t split;
-  float* partial;
-};
 
 // One batch = up to BATCH offsets and A_ROWS pairs; the pairs of one offset may be split over
 // consecutive batches.  Packed descriptor of one (batch, offset) entry.
@@ -1117,6 +1098,22 @@ void launch_prep(const ConvArgs& a, const void* weight, int weight_dtype, int dt
 
 template <typename T>
 int launch_conv(const ConvArgs& a, hipStream_t s) {
+  constexpr int dtype = std::is_same<T, float>::value ? WCN_DTYPE_F32
+                        : std::is_same<T, _Float16>::value ? WCN_DTYPE_F16 : WCN_DTYPE_BF16;
+  // Rows of at most one k-slice go to the pair-packed kernel.  WCN_CONV_KERNEL=ring in the
+  // environment keeps them on the output-stationary kernels below, whose results are bitwise
+  // reproducible from run to run (no atomics).
+  static const bool ring_only = [] {
+    const char* e = getenv("WCN_CONV_KERNEL");
+    return e && std::string(e) == "ring";
+  }();
+  if (!ring_only && wcn_conv_pack_takes(a, dtype)) {
+    if (g_time_start) (void)hipEventRecord(g_time_start, s);
+    const int st = wcn_conv_pack_launch(a, dtype, s);
+    if (g_time_stop) (void)hipEventRecord(g_time_stop, s);
+    g_time_start = g_time_stop = nullptr;
+    return st;
+  }
   const dim3 grid((unsigned)((a.num_out + ROWS - 1) / ROWS), (unsigned)(a.c_out_pad / TN));
   constexpr int NC = WCN_RING_NC;  // multiplying waves per workgroup of the ring kernel
   if (a.vec_in) {

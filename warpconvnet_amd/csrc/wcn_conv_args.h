@@ -1,0 +1,33 @@
+// Arguments shared by the contraction kernels of wcn_conv.hip and wcn_conv_pack.hip.
+#ifndef WCN_CONV_ARGS_H_
+#define WCN_CONV_ARGS_H_
+#include "wcn_common.h"
+
+struct ConvArgs {
+  const void* X;
+  const void* Wt;
+  const void* zeros;           // 1 KiB of zeros (source of loads that have nothing to fetch)
+  const void* bias;            // same dtype as X, or null
+  const int32_t* in_maps;      // pair lists; inside every offset out_maps ascends
+  const int32_t* out_maps;
+  const int64_t* offsets;      // (K + 1), device
+  const int32_t* group_start;  // (K, G + 1): pairs of offset k below output row 64 * g
+  void* out;
+  int64_t num_in, num_out, G;
+  int32_t K, c_in, c_out, c_in_pad, c_out_pad, identity;
+  int32_t vec_in;   // feature rows are 16-byte aligned and a whole number of 16-byte vectors
+  int32_t vec_out;  // same for output rows
+  int32_t flat_in;  // c_in is a multiple of the staged row and the feature matrix is below 4 GiB
+  // Few output tiles and several slices of input channels (small maps with wide features): the
+  // slices go to different workgroups (blockIdx.z), each writes its fp32 sums to
+  // partial[slice][row][c_out_pad] and conv_split_reduce adds them in slice order.
+  int32_t split;
+  float* partial;
+};
+
+
+// The pair-packed contraction (wcn_conv_pack.hip): whether it takes a problem, and its launch.
+bool wcn_conv_pack_takes(const ConvArgs& a, int dtype);
+int wcn_conv_pack_launch(const ConvArgs& a, int dtype, hipStream_t stream);
+
+#endif  // WCN_CONV_ARGS_H_
