@@ -3,8 +3,19 @@
  *
  * Conventions shared by every entry point
  *   - every pointer argument is a DEVICE pointer owned by the caller unless its name starts with
- *     `host_`; nothing is allocated or freed by the library; scratch memory is passed in as a
- *     workspace whose size comes from the matching *_bytes() query;
+ *     `host_`; no DEVICE memory is allocated or freed by the library: scratch memory is passed in
+ *     as a workspace whose size comes from the matching *_bytes() query.  What the library does
+ *     keep, per host thread that calls a *_read_* function, is up to three pinned host buffers of
+ *     16 KiB and three events (staging of the few bytes those calls bring to the host), created on
+ *     first use and held until wcn_thread_release() or the end of the process; and, per process,
+ *     the device-resident array behind wcn_sparse_conv_fwd_static;
+ *   - per-thread state crosses calls in three places, all named where they are declared:
+ *     wcn_kmap_count arms the result mailbox that the same thread's wcn_kmap_read_result collects,
+ *     wcn_kmap_last_table_flags reports on that thread's last read, and
+ *     wcn_conv_set_timing_events arms the thread's next contraction call;
+ *   - a call that waits for the device (the *_read_* functions) polls with an upper bound of
+ *     WCN_WAIT_LIMIT_MS milliseconds (environment variable, default 60000) and returns
+ *     WCN_ERR_LAUNCH when the stream has not got there by then;
  *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it and, unless stated,
  *     the call returns without waiting for the device;
  *   - the return value is a status: 0 = success, negative = error (wcn_status_string());
@@ -48,6 +59,10 @@ extern "C" {
 
 /* Library version (major*10000 + minor*100 + patch). */
 int wcn_version(void);
+
+/* Frees the calling thread's pinned staging buffers and events (see the conventions above); they
+ * come back on the thread's next *_read_* call.  No counterpart in the reference. */
+int wcn_thread_release(void);
 
 /* Text for a status code; replaces gemm_status_to_string (warpconvnet_pybind.cpp:1207-1226). */
 const char* wcn_status_string(int status);
@@ -97,6 +112,19 @@ size_t wcn_kmap_workspace_bytes(int64_t num_out, int32_t num_offsets);
 int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
                    int64_t num_out, const int32_t host_kernel_size[3],
                    const int32_t host_stride[3], void* workspace, void* stream);
+
+/* wcn_kmap_count for dilated and re-centred kernels: replaces the method="offset" branch of
+ * generate_kernel_map (torch_discrete.py:428-444: kernel_offsets_from_size :44-77 followed by the
+ * offset-table probe _kernel_map_from_offsets :160-241, discrete_kernels.cu:129-180).  Query
+ * coordinate of output m and offset (i, j, kk): out[m] * [1, sx, sy, sz] +
+ * (0, (i - c0) d0, (j - c1) d1, (kk - c2) d2) with d = host_dilation (>= 1) and c = host_centre
+ * (the reference's default: (size - 1) / 2 for odd sizes, 0 for even ones).  The other kernel-map
+ * calls (read_result, fill, group_start) are used as for wcn_kmap_count. */
+int wcn_kmap_count_dilated(const void* table, int64_t n_keys, int64_t capacity,
+                           const int32_t* out_coords, int64_t num_out,
+                           const int32_t host_kernel_size[3], const int32_t host_stride[3],
+                           const int32_t host_dilation[3], const int32_t host_centre[3],
+                           void* workspace, void* stream);
 
 /* Waits for the stream.  host_offsets[K+1] receives the exclusive prefix sums of the per-offset
  * pair counts (host_offsets[K] = L).  Returns the table status or WCN_ERR_TOO_MANY_PAIRS. */

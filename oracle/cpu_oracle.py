@@ -52,6 +52,9 @@ def lib():
         L.wcn_oracle_kernel_map_found.restype = ctypes.c_int
         L.wcn_oracle_kernel_map_found.argtypes = [i32p, ctypes.c_int, i32p, ctypes.c_int64, i32p,
                                                   i32p, ctypes.c_int, i32p]
+        L.wcn_oracle_kernel_map_offsets.restype = ctypes.c_int
+        L.wcn_oracle_kernel_map_offsets.argtypes = [i32p, ctypes.c_int, i32p, ctypes.c_int64, i32p,
+                                                    ctypes.c_int, i32p, ctypes.c_int, i32p]
         L.wcn_oracle_compact_found.restype = ctypes.c_int64
         L.wcn_oracle_compact_found.argtypes = [i32p, ctypes.c_int, ctypes.c_int64, i64p, i32p, i32p]
         L.wcn_oracle_stride_coords.restype = ctypes.c_int64
@@ -104,15 +107,6 @@ class HashTable:
         return out
 
 
-def kernel_offsets(kernel_size, dilation=(1, 1, 1)) -> np.ndarray:
-    ks, ksp = _i32(kernel_size)
-    dl, dlp = _i32(dilation)
-    K = int(np.prod(ks))
-    out = np.empty((K, 4), dtype=np.int32)
-    lib().wcn_oracle_kernel_offsets(ksp, dlp, _ptr(out, ctypes.c_int32))
-    return out
-
-
 def kernel_map_found(in_coords, out_coords, kernel_size, stride=(1, 1, 1), method=HASH_CITY):
     """Dense (K, M) table of found input indices (-1 where absent)."""
     ic, icp = _i32(in_coords)
@@ -141,9 +135,43 @@ def compact_found(found):
     return in_maps, out_maps, offsets
 
 
-def kernel_map(in_coords, out_coords, kernel_size, stride=(1, 1, 1), method=HASH_CITY):
-    """Reference-ordered kernel map plus the identity index rule of torch_discrete.py:418-425."""
-    found = kernel_map_found(in_coords, out_coords, kernel_size, stride, method)
+def kernel_offsets(kernel_size, dilation=(1, 1, 1), center_offset=None):
+    """(K, 4) offsets of kernel_offsets_from_size (torch_discrete.py:44-77): last dimension fastest,
+    (index - centre) * dilation, centre (s - 1) // 2 for odd sizes and 0 for even ones unless given."""
+    ks, ksp = _i32(kernel_size)
+    dl, dlp = _i32(dilation)
+    K = int(np.prod(ks))
+    out = np.empty((K, 4), dtype=np.int32)
+    lib().wcn_oracle_kernel_offsets(ksp, dlp, _ptr(out, ctypes.c_int32))
+    if center_offset is not None:  # the default centre is replaced, not shifted (:64-67)
+        default = np.array([(int(s) - 1) // 2 if int(s) % 2 == 1 else 0 for s in ks], dtype=np.int32)
+        out[:, 1:] += (default - np.asarray(center_offset, dtype=np.int32)) * dl
+    return out
+
+
+def kernel_map_found_offsets(in_coords, out_coords, offsets, stride=(1, 1, 1), method=HASH_CITY):
+    """Dense (K, M) table of found input indices for an explicit offset table (method="offset")."""
+    ic, icp = _i32(in_coords)
+    oc, ocp = _i32(out_coords)
+    of, ofp = _i32(offsets)
+    st, stp = _i32(stride)
+    found = np.empty((of.shape[0], oc.shape[0]), dtype=np.int32)
+    rc = lib().wcn_oracle_kernel_map_offsets(icp, ic.shape[0], ocp, oc.shape[0], ofp, of.shape[0], stp,
+                                             method, _ptr(found, ctypes.c_int32))
+    if rc != 0:
+        raise MemoryError("oracle allocation failed")
+    return found
+
+
+def kernel_map(in_coords, out_coords, kernel_size, stride=(1, 1, 1), method=HASH_CITY, dilation=None,
+               center_offset=None):
+    """Reference-ordered kernel map plus the identity index rule of torch_discrete.py:418-425.
+    With `dilation` / `center_offset` the offsets are those of method="offset"."""
+    if dilation is None and center_offset is None:
+        found = kernel_map_found(in_coords, out_coords, kernel_size, stride, method)
+    else:
+        offs = kernel_offsets(kernel_size, dilation or (1, 1, 1), center_offset)
+        found = kernel_map_found_offsets(in_coords, out_coords, offs, stride, method)
     in_maps, out_maps, offsets = compact_found(found)
     odd = all(int(k) % 2 == 1 for k in kernel_size)
     iden = int(np.prod(kernel_size)) // 2 if odd and len(in_coords) == len(out_coords) else None

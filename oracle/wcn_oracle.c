@@ -198,6 +198,37 @@ int wcn_oracle_kernel_map_found(const int32_t* in_coords, int n_in, const int32_
 }
 
 /*
+ * The method="offset" probe: torch_discrete.py:428-444 (offsets from kernel_offsets_from_size :44-77)
+ * + _kernel_map_from_offsets :160-241 + discrete_kernels.cu:129-180: found[k*M + m] = index of
+ * (out[m] * [1,s] + offsets[k]) among the input coordinates, or -1; `offsets` is (K, 4) with a zero
+ * batch column.  The reference's own call of this path is broken (its wrapper passes an argument
+ * the callee does not take), so this restates the intent its kernel and offset table spell out.
+ */
+int wcn_oracle_kernel_map_offsets(const int32_t* in_coords, int n_in, const int32_t* out_coords,
+                                  int64_t n_out, const int32_t* offsets, int K,
+                                  const int32_t stride[3], int method, int32_t* found /* K * n_out */) {
+  int capacity = n_in * 2 > 16 ? n_in * 2 : 16;
+  int32_t* kvs = (int32_t*)malloc(sizeof(int32_t) * 2 * (size_t)capacity);
+  int kk;
+  int64_t m;
+  if (!kvs) return -1;
+  wcn_oracle_table_init(kvs, capacity);
+  wcn_oracle_table_insert(kvs, capacity, in_coords, n_in, 4, method);
+  for (kk = 0; kk < K; ++kk) {
+    for (m = 0; m < n_out; ++m) {
+      int32_t q[4];
+      q[0] = out_coords[4 * m + 0] + offsets[4 * kk + 0];
+      q[1] = out_coords[4 * m + 1] * stride[0] + offsets[4 * kk + 1];
+      q[2] = out_coords[4 * m + 2] * stride[1] + offsets[4 * kk + 2];
+      q[3] = out_coords[4 * m + 3] * stride[2] + offsets[4 * kk + 3];
+      found[(int64_t)kk * n_out + m] = table_search_one(kvs, capacity, in_coords, q, 4, method);
+    }
+  }
+  free(kvs);
+  return 0;
+}
+
+/*
  * Row-wise stream compaction: torch_discrete.py:80-157 + discrete_kernels.cu:183-213.
  * offsets[K+1] (exclusive prefix of hits per offset row), and for every hit in row k at column m,
  * in ascending m: in_maps[pos] = found, out_maps[pos] = m.  Pass in_maps == NULL to get only the

@@ -326,3 +326,23 @@ def test_morton_ordered_output(oracle):
         assert (np.diff(codes[b == item]) > 0).all()
     want, _ = _oracle_out(oracle, x, w, bc, out_bc.cpu().numpy(), (2, 2, 2), (2, 2, 2))
     assert rel_err(out.feature_tensor.cpu().numpy(), want) <= 1e-5
+
+
+def test_dilated_convolution_matches_oracle(oracle):
+    """SparseConv3d(dilation=2): the map comes from the offset-based probe, the features match the
+    fp64 oracle over the oracle's dilated map."""
+    from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d
+    items = [synthetic.random_cloud(50 + b, 5000, 28)[:, 1:] for b in range(2)]
+    bc = synthetic.batch_indexed(items)
+    x = normal_features(len(bc), 16, seed=8)
+    vox = _voxels(items, x)
+    torch.manual_seed(2)
+    conv = SparseConv3d(16, 24, 3, dilation=2, bias=True).to(DEV)
+    with torch.no_grad():
+        y = conv(vox)
+    im, om, off, iden = oracle.kernel_map(bc, bc, (3, 3, 3), dilation=(2, 2, 2))
+    want = oracle.explicit_conv_f64(x.double().numpy(), conv.weight.detach().double().cpu().numpy(), im, om,
+                                    off, iden, len(bc)) + conv.bias.detach().double().cpu().numpy()
+    assert rel_err(y.feature_tensor.cpu().numpy(), want) <= 1e-5
+    km = next(iter(vox.cache.values()))
+    assert np.array_equal(km.in_maps.cpu().numpy(), im) and np.array_equal(km.out_maps.cpu().numpy(), om)

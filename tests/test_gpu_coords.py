@@ -116,6 +116,55 @@ def test_kernel_map_bit_exact(oracle, name, gen, ksize, stride):
                           canonical_pairs(ref_in, ref_out_map, ref_off))
 
 
+DILATED = [
+    ("k3_d2", (3, 3, 3), (1, 1, 1), (2, 2, 2), None),
+    ("k3_d123", (3, 3, 3), (1, 1, 1), (1, 2, 3), None),
+    ("k2s2_d212", (2, 2, 2), (2, 2, 2), (2, 1, 2), None),
+    ("k3_centre", (3, 3, 3), (1, 1, 1), (1, 1, 1), (0, 2, 1)),
+    ("k323_d231_centre", (3, 2, 3), (1, 1, 1), (2, 3, 1), (1, 1, 0)),
+    ("k5_d2", (5, 5, 5), (1, 1, 1), (2, 2, 2), None),
+]
+
+
+@pytest.mark.parametrize("name,ksize,stride,dilation,centre", DILATED, ids=[c[0] for c in DILATED])
+def test_dilated_kernel_map_bit_exact(oracle, name, ksize, stride, dilation, centre):
+    """method="offset": dilated and re-centred kernels, bit-exact in native order against the oracle's
+    offset-table probe (itself pinned by a dictionary brute force)."""
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    in_coords = synthetic.random_cloud(31, 20000, 40, batch_size=2)
+    if any(s != 1 for s in stride):
+        out_coords = stride_coords(_dev(in_coords), stride)[0].cpu().numpy()
+    else:
+        out_coords = in_coords
+    km = generate_kernel_map(_dev(in_coords), _dev(out_coords), stride, ksize, kernel_dilation=dilation,
+                             kernel_center_offset=centre, method="offset")
+    ref_in, ref_out, ref_off, ref_iden = oracle.kernel_map(in_coords, out_coords, ksize, stride,
+                                                           dilation=dilation, center_offset=centre)
+    assert int(ref_off[-1]) > 0
+    assert np.array_equal(km.offsets.numpy().astype(np.int64), ref_off)
+    assert np.array_equal(km.in_maps.cpu().numpy(), ref_in)
+    assert np.array_equal(km.out_maps.cpu().numpy(), ref_out)
+    assert km.identity_map_index == (None if centre is not None else ref_iden)
+
+
+def test_ordered_stride_coords():
+    """stride_coords with a Morton ordering: the same set of coarse voxels, batch items contiguous,
+    Morton codes ascending inside every batch item."""
+    from warpconvnet_amd.geometry.coords.ops.serialization import POINT_ORDERING, morton_code
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    in_coords = synthetic.random_cloud(33, 30000, 48, batch_size=3)
+    plain, plain_off = stride_coords(_dev(in_coords), (2, 2, 2))
+    ordered, off = stride_coords(_dev(in_coords), (2, 2, 2), order=POINT_ORDERING.MORTON_XYZ)
+    assert torch.equal(off, plain_off)
+    assert np.array_equal(sort_rows(ordered.cpu().numpy()), sort_rows(plain.cpu().numpy()))
+    assert bool((torch.diff(ordered[:, 0]) >= 0).all())
+    codes = morton_code(ordered[:, 1:].contiguous(), order=POINT_ORDERING.MORTON_XYZ)
+    for b in range(3):
+        seg = codes[int(off[b]):int(off[b + 1])]
+        assert bool((torch.diff(seg) >= 0).all())
+
+
 def test_kernel_map_invariants_full_size():
     """Size-independent properties at the benchmark's size (4 x 250k voxels, 3x3x3):
     identity row, offset symmetry, duplicate-free rows."""

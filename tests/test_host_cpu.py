@@ -191,6 +191,26 @@ def test_kernel_offsets_from_size_matches_oracle(oracle):
         assert np.array_equal(kernel_offsets_from_size(ks, dil).numpy(), oracle.kernel_offsets(ks, dil))
 
 
+def test_reference_import_path_resolves_to_the_same_modules():
+    """`warpconvnet.*` (the reference's package name) names the very modules of this package."""
+    import importlib
+    import warpconvnet  # noqa: F401
+    for rel in ("nn.modules.sparse_conv", "nn.functional.sparse_conv", "geometry.types.voxels",
+                "geometry.coords.search.torch_discrete", "geometry.coords.ops.stride"):
+        assert importlib.import_module("warpconvnet." + rel) is importlib.import_module("warpconvnet_amd." + rel)
+    from warpconvnet.nn.modules.sparse_conv import SparseConv3d
+    from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d as ours
+    assert SparseConv3d is ours
+    with pytest.raises(ModuleNotFoundError):
+        importlib.import_module("warpconvnet.nn.modules.attention")
+
+
+def test_thread_release_without_any_call_is_a_no_op():
+    from warpconvnet_amd._lib import lib
+    assert lib().wcn_thread_release() == 0
+    assert lib().wcn_thread_release() == 0
+
+
 # ---- module / functional argument handling -----------------------------------------------------
 
 def test_module_parameters_and_init_bound():

@@ -82,17 +82,18 @@ def test_table_search_invariants(oracle, method):
 
 # ---- kernel map ------------------------------------------------------------------------------
 
-def brute_force_kernel_map(in_coords, out_coords, ksize, stride):
+def brute_force_kernel_map(in_coords, out_coords, ksize, stride, dilation=(1, 1, 1), centre=None):
     """Independent restatement: a Python dict of coordinate tuples, offsets from itertools."""
     lookup = {}
     for i, r in enumerate(map(tuple, in_coords.tolist())):
         lookup.setdefault(r, i)
-    centre = [s // 2 if s % 2 == 1 else 0 for s in ksize]
+    if centre is None:
+        centre = [s // 2 if s % 2 == 1 else 0 for s in ksize]
     ins, outs, offsets = [], [], [0]
     for i, j, k in itertools.product(range(ksize[0]), range(ksize[1]), range(ksize[2])):
         for m, (b, x, y, z) in enumerate(out_coords.tolist()):
-            q = (b, x * stride[0] + i - centre[0], y * stride[1] + j - centre[1],
-                 z * stride[2] + k - centre[2])
+            q = (b, x * stride[0] + (i - centre[0]) * dilation[0], y * stride[1] + (j - centre[1]) * dilation[1],
+                 z * stride[2] + (k - centre[2]) * dilation[2])
             hit = lookup.get(q)
             if hit is not None:
                 ins.append(hit)
@@ -119,6 +120,32 @@ def test_kernel_map_equals_brute_force(oracle, ksize, stride):
         assert np.array_equal(g, w)
     odd = all(k % 2 == 1 for k in ksize)
     assert got[3] == (int(np.prod(ksize)) // 2 if odd and len(in_coords) == len(out_coords) else None)
+
+
+DILATED_CASES = [((3, 3, 3), (1, 1, 1), (2, 2, 2), None), ((3, 3, 3), (1, 1, 1), (1, 2, 3), None),
+                 ((2, 2, 2), (2, 2, 2), (2, 1, 2), None), ((3, 3, 3), (1, 1, 1), (1, 1, 1), (0, 2, 1)),
+                 ((3, 2, 3), (1, 1, 1), (2, 3, 1), (1, 1, 0))]
+
+
+@pytest.mark.parametrize("ksize,stride,dilation,centre", DILATED_CASES)
+def test_dilated_kernel_map_equals_brute_force(oracle, ksize, stride, dilation, centre):
+    """The offset-table probe (dilation, custom centre): every offset, scale and sign is fixed by the
+    dictionary brute force; with dilation 1 and the default centre it is the size-based map."""
+    in_coords = synthetic.random_cloud(9, 1500, 14, batch_size=2)
+    if any(s != 1 for s in stride):
+        out_coords = np.unique(np.concatenate(
+            [in_coords[:, :1], np.floor_divide(in_coords[:, 1:], np.array(stride))], axis=1), axis=0)
+    else:
+        out_coords = in_coords
+    got = oracle.kernel_map(in_coords, out_coords, ksize, stride, dilation=dilation, center_offset=centre)
+    want = brute_force_kernel_map(in_coords, out_coords, ksize, stride, dilation, centre)
+    for g, w in zip(got[:3], want):
+        assert np.array_equal(g, w)
+    assert int(want[2][-1]) > 0
+    plain = oracle.kernel_map(in_coords, out_coords, ksize, stride)
+    same = oracle.kernel_map(in_coords, out_coords, ksize, stride, dilation=(1, 1, 1))
+    for g, w in zip(same[:3], plain[:3]):
+        assert np.array_equal(g, w)
 
 
 @pytest.mark.parametrize("method", [0, 1, 2])

@@ -19,6 +19,7 @@ _i32p, _i64p = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64)
 SIGNATURES = {
     "wcn_version": (ctypes.c_int, []),
     "wcn_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "wcn_thread_release": (ctypes.c_int, []),
     "wcn_table_default_capacity": (_i64, [_i64]),
     "wcn_table_bytes": (_sz, [_i64, _i64]),
     "wcn_table_build": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
@@ -26,6 +27,7 @@ SIGNATURES = {
     "wcn_table_read_status": (ctypes.c_int, [_vp, _i32p, _vp]),
     "wcn_kmap_workspace_bytes": (_sz, [_i64, _i32]),
     "wcn_kmap_count": (ctypes.c_int, [_vp, _i64, _i64, _vp, _i64, _i32p, _i32p, _vp, _vp]),
+    "wcn_kmap_count_dilated": (ctypes.c_int, [_vp, _i64, _i64, _vp, _i64, _i32p, _i32p, _i32p, _i32p, _vp, _vp]),
     "wcn_kmap_read_result": (ctypes.c_int, [_vp, _i64, _i32, _i64p, _vp]),
     "wcn_kmap_fill": (ctypes.c_int, [_vp, _i64, _i64, _vp, _i64, _i32p, _i32p, _vp, _i64, _vp, _vp,
                                      _vp]),

@@ -21,7 +21,8 @@ namespace {
 struct KmapGeom {
   int32_t kx, ky, kz;  // kernel size
   int32_t sx, sy, sz;  // in-to-out stride ratio applied to the output coordinates
-  int32_t cx, cy, cz;  // centre: size/2 for odd sizes, 0 for even (discrete_kernels.cu:291-294)
+  int32_t cx, cy, cz;  // centre: size/2 for odd sizes, 0 for even (discrete_kernels.cu:291-294), or the caller's
+  int32_t dx, dy, dz;  // dilation: offset (i, j, kk) is ((i - cx) dx, (j - cy) dy, (kk - cz) dz)
   int32_t K;
 };
 
@@ -89,9 +90,9 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
   if (live) c = out_coords[m];
   // query origin relative to the table's box, modulo 2^32 like the reference's int arithmetic
   const uint32_t rb = (uint32_t)c.x - L.amin[0];
-  const uint32_t rx0 = (uint32_t)c.y * (uint32_t)g.sx - (uint32_t)g.cx - L.amin[1];
-  const uint32_t ry0 = (uint32_t)c.z * (uint32_t)g.sy - (uint32_t)g.cy - L.amin[2];
-  const uint32_t rz0 = (uint32_t)c.w * (uint32_t)g.sz - (uint32_t)g.cz - L.amin[3];
+  const uint32_t rx0 = (uint32_t)c.y * (uint32_t)g.sx - (uint32_t)(g.cx * g.dx) - L.amin[1];
+  const uint32_t ry0 = (uint32_t)c.z * (uint32_t)g.sy - (uint32_t)(g.cy * g.dy) - L.amin[2];
+  const uint32_t rz0 = (uint32_t)c.w * (uint32_t)g.sz - (uint32_t)(g.cz * g.dz) - L.amin[3];
   const bool usable = live && L.ok && rb <= L.span[0];
 
   unsigned long long cached_key = WCN_EMPTY_KEY, cached_mask = 0ull;
@@ -101,7 +102,7 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
     for (int j = 0; j < g.ky; ++j) {
       for (int kk = 0; kk < g.kz; ++kk, ++k) {
         int32_t found = -1;
-        uint32_t r[4] = {rb, rx0 + (uint32_t)i, ry0 + (uint32_t)j, rz0 + (uint32_t)kk};
+        uint32_t r[4] = {rb, rx0 + (uint32_t)(i * g.dx), ry0 + (uint32_t)(j * g.dy), rz0 + (uint32_t)(kk * g.dz)};
         if (usable && r[1] <= L.span[1] && r[2] <= L.span[2] && r[3] <= L.span[3]) {
           const unsigned long long key = wcn_block_key(L, r);
           if (key != cached_key) {
@@ -427,23 +428,31 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
   }
 }
 
-bool make_geom(const int32_t ks[3], const int32_t st[3], KmapGeom* g) {
+bool make_geom(const int32_t ks[3], const int32_t st[3], const int32_t* dil, const int32_t* centre,
+               KmapGeom* g) {
   if (!ks || !st) return false;
   for (int d = 0; d < 3; ++d)
-    if (ks[d] < 1 || st[d] < 1) return false;
+    if (ks[d] < 1 || st[d] < 1 || (dil && dil[d] < 1)) return false;
   const int64_t K = (int64_t)ks[0] * ks[1] * ks[2];
   if (K > WCN_MAX_OFFSETS) return false;
   g->kx = ks[0]; g->ky = ks[1]; g->kz = ks[2];
   g->sx = st[0]; g->sy = st[1]; g->sz = st[2];
-  g->cx = (ks[0] % 2) ? ks[0] / 2 : 0;
-  g->cy = (ks[1] % 2) ? ks[1] / 2 : 0;
-  g->cz = (ks[2] % 2) ? ks[2] / 2 : 0;
+  g->cx = centre ? centre[0] : ((ks[0] % 2) ? ks[0] / 2 : 0);
+  g->cy = centre ? centre[1] : ((ks[1] % 2) ? ks[1] / 2 : 0);
+  g->cz = centre ? centre[2] : ((ks[2] % 2) ? ks[2] / 2 : 0);
+  g->dx = dil ? dil[0] : 1; g->dy = dil ? dil[1] : 1; g->dz = dil ? dil[2] : 1;
   g->K = (int32_t)K;
   return true;
 }
 
+// The compile-time-size probe kernels assume dilation 1 and the default centre.
+inline bool plain_geom(const KmapGeom& g) {
+  return g.dx == 1 && g.dy == 1 && g.dz == 1 && g.cx == ((g.kx % 2) ? g.kx / 2 : 0) &&
+         g.cy == ((g.ky % 2) ? g.ky / 2 : 0) && g.cz == ((g.kz % 2) ? g.kz / 2 : 0);
+}
+
 inline bool is_fixed_size(const KmapGeom& g, int x, int y, int z) {
-  return g.kx == x && g.ky == y && g.kz == z;
+  return plain_geom(g) && g.kx == x && g.ky == y && g.kz == z;
 }
 
 inline bool table_args_ok(const void* table, int64_t n_keys, int64_t capacity) {
@@ -594,11 +603,12 @@ size_t wcn_kmap_workspace_bytes(int64_t num_out, int32_t num_offsets) {
   return kmap_layout(nullptr, num_out, num_offsets, nullptr);
 }
 
-int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
-                   int64_t num_out, const int32_t host_kernel_size[3],
-                   const int32_t host_stride[3], void* workspace, void* stream) {
+static int kmap_count_impl(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
+                           int64_t num_out, const int32_t host_kernel_size[3],
+                           const int32_t host_stride[3], const int32_t* host_dilation,
+                           const int32_t* host_centre, void* workspace, void* stream) {
   KmapGeom g;
-  if (!make_geom(host_kernel_size, host_stride, &g)) return WCN_ERR_INVALID_ARGUMENT;
+  if (!make_geom(host_kernel_size, host_stride, host_dilation, host_centre, &g)) return WCN_ERR_INVALID_ARGUMENT;
   if (!table_args_ok(table, n_keys, capacity) || !workspace || num_out < 0 ||
       num_out >= (1ll << 31) || (num_out > 0 && !out_coords))
     return WCN_ERR_INVALID_ARGUMENT;
@@ -635,6 +645,22 @@ int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const in
   return WCN_OK;
 }
 
+int wcn_kmap_count(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
+                   int64_t num_out, const int32_t host_kernel_size[3],
+                   const int32_t host_stride[3], void* workspace, void* stream) {
+  return kmap_count_impl(table, n_keys, capacity, out_coords, num_out, host_kernel_size, host_stride,
+                         nullptr, nullptr, workspace, stream);
+}
+
+int wcn_kmap_count_dilated(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
+                           int64_t num_out, const int32_t host_kernel_size[3],
+                           const int32_t host_stride[3], const int32_t host_dilation[3],
+                           const int32_t host_centre[3], void* workspace, void* stream) {
+  if (!host_dilation || !host_centre) return WCN_ERR_INVALID_ARGUMENT;
+  return kmap_count_impl(table, n_keys, capacity, out_coords, num_out, host_kernel_size, host_stride,
+                         host_dilation, host_centre, workspace, stream);
+}
+
 int32_t wcn_kmap_last_table_flags(void) { return g_last_table_flags; }
 
 int wcn_kmap_read_result(const void* workspace, int64_t num_out, int32_t num_offsets,
@@ -665,7 +691,7 @@ int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int
                   const void* workspace, int64_t pair_capacity, int32_t* in_maps, int32_t* out_maps,
                   void* stream) {
   KmapGeom g;
-  if (!make_geom(host_kernel_size, host_stride, &g)) return WCN_ERR_INVALID_ARGUMENT;
+  if (!make_geom(host_kernel_size, host_stride, nullptr, nullptr, &g)) return WCN_ERR_INVALID_ARGUMENT;
   if (!table_args_ok(table, n_keys, capacity) || !workspace || num_out < 0 ||
       num_out >= (1ll << 31) || (num_out > 0 && !out_coords) || pair_capacity < 0)
     return WCN_ERR_INVALID_ARGUMENT;

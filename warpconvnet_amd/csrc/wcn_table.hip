@@ -9,7 +9,11 @@
 //
 // HBM traffic per key: 16 B read (bbox) + 16 B read (insert) + 4 B slot_of write + 4 B read +
 // 4 B perm write, plus 32 B per table slot to clear and one 32 B slot touched per key.
+#include <stdlib.h>
 #include <string.h>
+
+#include <chrono>
+#include <thread>
 
 #include "wcn_common.h"
 
@@ -243,11 +247,51 @@ int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView
   return WCN_OK;
 }
 
+// Host waits are polls (a blocking stream synchronisation wakes the host tens of microseconds
+// late) with an upper bound: WCN_WAIT_LIMIT_MS milliseconds (environment, default 60000), after
+// which the call gives up with WCN_ERR_LAUNCH instead of spinning for ever on a stream that is
+// stuck.  After a short spin the poll yields the core between looks.
+namespace {
+int64_t wait_limit_ns() {
+  static const int64_t limit = [] {
+    const char* e = getenv("WCN_WAIT_LIMIT_MS");
+    const long long ms = e ? atoll(e) : 0;
+    return (int64_t)(ms > 0 ? ms : 60000) * 1000000;
+  }();
+  return limit;
+}
+struct BoundedPoll {
+  std::chrono::steady_clock::time_point start = std::chrono::steady_clock::now();
+  unsigned looks = 0;
+  // false once the time limit has passed
+  bool again() {
+    if ((++looks & 0xFFu) != 0) return true;
+    const int64_t ns = std::chrono::duration_cast<std::chrono::nanoseconds>(
+                           std::chrono::steady_clock::now() - start).count();
+    if (ns > wait_limit_ns()) return false;
+    if (ns > 200000) std::this_thread::yield();
+    return true;
+  }
+};
+int wait_for_event(hipEvent_t ev) {
+  BoundedPoll poll;
+  for (;;) {
+    const hipError_t e = hipEventQuery(ev);
+    if (e == hipSuccess) return WCN_OK;
+    if (e != hipErrorNotReady || !poll.again()) return WCN_ERR_LAUNCH;
+  }
+}
+// per-thread pinned staging of wcn_read_small (released by wcn_thread_release)
+thread_local void* g_small_staging = nullptr;
+thread_local hipEvent_t g_small_done = nullptr;
+thread_local int g_small_device = -1;
+}  // namespace
+
 int wcn_read_small(void* host_dst, const void* device_src, size_t bytes, hipStream_t stream) {
   constexpr size_t kStaging = 16384;
-  thread_local void* staging = nullptr;
-  thread_local hipEvent_t done = nullptr;
-  thread_local int staging_device = -1;
+  void*& staging = g_small_staging;
+  hipEvent_t& done = g_small_done;
+  int& staging_device = g_small_device;
   if (bytes > kStaging) return WCN_ERR_INVALID_ARGUMENT;
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return WCN_ERR_LAUNCH;
@@ -268,11 +312,7 @@ int wcn_read_small(void* host_dst, const void* device_src, size_t bytes, hipStre
   if (hipMemcpyAsync(staging, device_src, bytes, hipMemcpyDeviceToHost, stream) != hipSuccess)
     return WCN_ERR_LAUNCH;
   if (hipEventRecord(done, stream) != hipSuccess) return WCN_ERR_LAUNCH;
-  for (;;) {
-    const hipError_t e = hipEventQuery(done);
-    if (e == hipSuccess) break;
-    if (e != hipErrorNotReady) return WCN_ERR_LAUNCH;
-  }
+  if (wait_for_event(done) != WCN_OK) return WCN_ERR_LAUNCH;
   memcpy(host_dst, staging, bytes);
   return WCN_OK;
 }
@@ -320,11 +360,7 @@ int wcn_read_early_end(void* host_dst, const void* device_src, size_t bytes, hip
   if (g_early_src != device_src || g_early_bytes != bytes)
     return wcn_read_small(host_dst, device_src, bytes, stream);
   g_early_src = nullptr;
-  for (;;) {
-    const hipError_t e = hipEventQuery(g_early_done);
-    if (e == hipSuccess) break;
-    if (e != hipErrorNotReady) return WCN_ERR_LAUNCH;
-  }
+  if (wait_for_event(g_early_done) != WCN_OK) return WCN_ERR_LAUNCH;
   memcpy(host_dst, g_early_staging, bytes);
   return WCN_OK;
 }
@@ -370,10 +406,14 @@ int wcn_mailbox_mark(hipStream_t stream) {
 int wcn_mailbox_end(void* host_dst, size_t payload_bytes, int64_t sequence) {
   if (!g_box || !g_box_done || payload_bytes + 8 > kMailboxBytes) return WCN_ERR_INVALID_ARGUMENT;
   volatile int64_t* word0 = g_box;
+  BoundedPoll poll;
   for (;;) {
     if (*word0 == sequence) break;
     const hipError_t e = hipEventQuery(g_box_done);
-    if (e == hipErrorNotReady) continue;
+    if (e == hipErrorNotReady) {
+      if (!poll.again()) return WCN_ERR_LAUNCH;
+      continue;
+    }
     if (e != hipSuccess) return WCN_ERR_LAUNCH;
     // the kernel is over: its write must be there by now, or it never happened
     if (*word0 == sequence) break;
@@ -392,7 +432,23 @@ int wcn_table_status_from_bits(int32_t bits) {
 
 extern "C" {
 
-int wcn_version(void) { return 100; }
+int wcn_version(void) { return 200; }
+
+int wcn_thread_release(void) {
+  int st = WCN_OK;
+  if (g_small_done && hipEventDestroy(g_small_done) != hipSuccess) st = WCN_ERR_LAUNCH;
+  if (g_early_done && hipEventDestroy(g_early_done) != hipSuccess) st = WCN_ERR_LAUNCH;
+  if (g_box_done && hipEventDestroy(g_box_done) != hipSuccess) st = WCN_ERR_LAUNCH;
+  if (g_small_staging && hipHostFree(g_small_staging) != hipSuccess) st = WCN_ERR_LAUNCH;
+  if (g_early_staging && hipHostFree(g_early_staging) != hipSuccess) st = WCN_ERR_LAUNCH;
+  if (g_box && hipHostFree(g_box) != hipSuccess) st = WCN_ERR_LAUNCH;
+  g_small_done = g_early_done = g_box_done = nullptr;
+  g_small_staging = g_early_staging = nullptr;
+  g_box = nullptr;
+  g_small_device = g_early_device = g_box_device = -1;
+  g_early_src = nullptr;
+  return st;
+}
 
 const char* wcn_status_string(int status) {
   switch (status) {

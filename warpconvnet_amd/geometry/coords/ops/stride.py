@@ -22,21 +22,28 @@ def stride_coords(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
     row count.  Output rows ascend in their representative's source row, so a batch-sorted input
     yields a batch-sorted output (the reference sorts by batch afterwards, stride.py:44-48, with an
     order inside a batch that depends on a thread race; as sets the results are identical).
-    Only the reference's default ordering is built.
+    Any other `order` sorts the coarse voxels of every batch item along that curve.
     """
     num_spatial_dims = batch_indexed_coords.shape[1] - 1
     assert len(stride) == num_spatial_dims, \
         (f"Stride must match the number of spatial dimensions. Got {len(stride)} spatial "
          f"dimensions for but coordinates with {num_spatial_dims} spatial dimensions.")
-    if str(getattr(order, "name", order)).lower() != "random":
-        raise NotImplementedError("only the default (unordered) output ordering is built")
     if all(s == 1 for s in stride):
         return batch_indexed_coords, offsets_from_batch_index(batch_indexed_coords[:, 0])
     out, count = unique_floor_div_rows(batch_indexed_coords, stride)
     unique_coords = out[:count, : num_spatial_dims + 1]
     if num_spatial_dims != 3:
         unique_coords = unique_coords.contiguous()
-    return unique_coords, offsets_from_batch_index(unique_coords[:, 0])
+    out_offsets = offsets_from_batch_index(unique_coords[:, 0])
+    if str(getattr(order, "name", order)).lower() not in ("random", "point_ordering.random"):
+        # The coarse voxels of every batch item along a space-filling curve.  (The reference hands
+        # the four-column rows to `encode`, whose code function accepts three columns and raises,
+        # stride.py:49-51; the evident intent is the ordering of the spatial columns per batch item.)
+        from .serialization import encode
+        code = encode(unique_coords[:, 1:].contiguous(), batch_offsets=out_offsets, order=order,
+                      return_perm=True)
+        unique_coords = unique_coords[code.perm].contiguous()
+    return unique_coords, out_offsets
 
 
 @torch.no_grad()

@@ -32,15 +32,22 @@ def kernel_offsets_from_size(kernel_size: Tuple[int, ...], kernel_dilation: Tupl
     for odd sizes and 0 for even ones, scaled by the dilation (reference: torch_discrete.py:44-77)."""
     assert len(kernel_size) == len(kernel_dilation)
     axes = []
-    for d, (size, dil) in enumerate(zip(kernel_size, kernel_dilation)):
-        centre = (size - 1) // 2 if size % 2 == 1 else 0
-        if center_offset is not None:
-            centre = centre + center_offset[d]
+    centres = _kernel_centres(kernel_size, center_offset)
+    for size, dil, centre in zip(kernel_size, kernel_dilation, centres):
         axes.append((torch.arange(size, dtype=torch.int32) - centre) * dil)
     grid = torch.meshgrid(*axes, indexing="ij")
     spatial = torch.stack([g.reshape(-1) for g in grid], dim=1)
     batch = torch.zeros(spatial.shape[0], 1, dtype=torch.int32)
     return torch.cat([batch, spatial], dim=1).to(device)
+
+
+def _kernel_centres(kernel_size, center_offset=None):
+    """Index of the zero offset per dimension: (s - 1) // 2 for odd sizes and 0 for even ones,
+    unless the caller names it (reference: torch_discrete.py:64-67)."""
+    if center_offset is None:
+        return [(int(s) - 1) // 2 if int(s) % 2 == 1 else 0 for s in kernel_size]
+    assert len(center_offset) == len(kernel_size)
+    return [int(c) for c in center_offset]
 
 
 def _pad_kernel_args(values: Sequence[int], fill: int):
@@ -52,7 +59,8 @@ def _pad_kernel_args(values: Sequence[int], fill: int):
 
 @torch.no_grad()
 def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_size, stride,
-                           identity_map_index: Optional[int]) -> IntSearchResult:
+                           identity_map_index: Optional[int], dilation=None,
+                           centres=None) -> IntSearchResult:
     """Count, read the offsets, fill.  Handles the device-reported table overflow by rebuilding
     the table with more slots and starting over."""
     device = out_coords.device
@@ -72,8 +80,14 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     out_buf = torch.empty(assumed, dtype=torch.int32, device=device)
     while True:
         raw, n_keys, slots = table._raw()
-        check(L.wcn_kmap_count(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws),
-                               stream_ptr(device)), "wcn_kmap_count")
+        if dilation is None:
+            check(L.wcn_kmap_count(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws),
+                                   stream_ptr(device)), "wcn_kmap_count")
+        else:
+            check(L.wcn_kmap_count_dilated(ptr(raw), n_keys, slots, ptr(out4), M, ks, st,
+                                           int3(_pad_kernel_args(dilation, 1)),
+                                           int3(_pad_kernel_args(centres, 0)), ptr(ws),
+                                           stream_ptr(device)), "wcn_kmap_count_dilated")
         check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), assumed,
                               ptr(in_buf), ptr(out_buf), stream_ptr(device)), "wcn_kmap_fill")
         status = L.wcn_kmap_read_result(ptr(ws), M, K, host_offsets, stream_ptr(device))
@@ -160,9 +174,6 @@ def generate_kernel_map(
             "Kernel dilation is not supported with method='size'. Use method='offset' instead."
         assert kernel_center_offset is None, \
             "Custom kernel_center_offset is not supported with method='size'. Use method='offset' instead."
-    elif (kernel_dilation is not None and any(s != 1 for s in kernel_dilation)) \
-            or kernel_center_offset is not None:
-        raise NotImplementedError("dilated or re-centred kernels are not built on this path")
     if num_spatial_dims > 3:
         raise NotImplementedError("more than 3 spatial dimensions are not supported")
 
@@ -173,13 +184,24 @@ def generate_kernel_map(
     identity_map_index = int(np.prod(kernel_size)) // 2 if (is_odd and same_count) else None
 
     stride = ntuple(in_to_out_stride_ratio, ndim=num_spatial_dims)
+    dilation = centres = None
+    if method == "offset":
+        # the reference probes a table of offsets here (torch_discrete.py:428-444); the same
+        # queries come out of the size-based probe with scaled and re-centred offsets
+        dilation = [1] * num_spatial_dims if kernel_dilation is None else [int(d) for d in kernel_dilation]
+        assert len(dilation) == num_spatial_dims and all(d >= 1 for d in dilation)
+        centres = _kernel_centres(kernel_size, kernel_center_offset)
+        if centres != _kernel_centres(kernel_size):
+            identity_map_index = None  # the offset at K // 2 is no longer the zero offset
+        elif all(d == 1 for d in dilation):
+            dilation = centres = None
     result = _kernel_map_from_table(table, batch_indexed_out_coords, kernel_size, stride,
-                                    identity_map_index)
+                                    identity_map_index, dilation, centres)
     same_set = (batch_indexed_in_coords.data_ptr() == batch_indexed_out_coords.data_ptr()
                 and batch_indexed_in_coords.shape == batch_indexed_out_coords.shape
                 and batch_indexed_in_coords.stride() == batch_indexed_out_coords.stride())
     result._symmetric = bool(same_set and is_odd and all(s == 1 for s in stride)
-                             and getattr(result, "_keys_unique", False))
+                             and centres is None and getattr(result, "_keys_unique", False))
     if skip_symmetric_kernel_map and is_odd:
         # only the offsets before the centre are kept (torch_discrete.py:286-296)
         half = int(np.prod(kernel_size)) // 2

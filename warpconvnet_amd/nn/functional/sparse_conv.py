@@ -287,20 +287,25 @@ def generate_output_coords_and_kernel_map(
         if kernel_map is not None:
             return out_coords, out_offsets, kernel_map
 
+    # dilated kernels take the offset-based probe (the size-based one asserts dilation 1, as in the
+    # reference: torch_discrete.py:445-448)
+    method = "offset" if any(int(d) != 1 for d in kernel_dilation) else "size"
     if transposed:
         forward_map = None
         if cache is not None:
             forward_map = cache.get(make_key(False, out_offsets, input_sparse_tensor.offsets))
         if forward_map is None:
             forward_map = generate_kernel_map(out_coords, in_coords, stride, kernel_size,
-                                              kernel_dilation, skip_symmetric_kernel_map=False)
+                                              kernel_dilation, method=method,
+                                              skip_symmetric_kernel_map=False)
         kernel_map = IntSearchResult(in_maps=forward_map.out_maps, out_maps=forward_map.in_maps,
                                      offsets=forward_map.offsets)
         kernel_map._in_ascend = forward_map._out_ascend
         kernel_map._in_group_start = forward_map._group_start
     else:
         kernel_map = generate_kernel_map(in_coords, out_coords, stride, kernel_size,
-                                         kernel_dilation, skip_symmetric_kernel_map=False)
+                                         kernel_dilation, method=method,
+                                         skip_symmetric_kernel_map=False)
 
     if input_sparse_tensor.cache is None:
         input_sparse_tensor._extra_attributes["_cache"] = IntSearchCache()
