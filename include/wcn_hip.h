@@ -226,6 +226,25 @@ int wcn_sparse_conv_fwd_static(const void* features, int64_t num_in, int32_t c_i
                                const int32_t* group_start_or_null, void* out, int64_t num_out,
                                void* stream);
 
+/* Re-orders the pair lists of a map so that out_maps ascends inside every offset, and writes the
+ * table group_start[k * (G + 1) + g] = number of pairs of offset k with out_maps < 64 g
+ * (G = ceil(num_out / 64); (K, G + 1) int32).  This is what wcn_sparse_conv_fwd does inside its
+ * workspace on every call with out_maps_ascend = 0; done once here, the results can be kept with
+ * the map and passed with out_maps_ascend = 1 and group_start on every later call (the map of a
+ * transposed convolution, or a forward map with its lists exchanged for the input gradient).  The
+ * reference keeps such a map as it is and pays nothing for its order because its per-offset GEMMs
+ * scatter with atomics (sparse_conv.py:1916-1939 builds the exchanged map; :495-544 uses it).
+ * Precondition: at most one pair per (offset, output row), which every kernel map satisfies; of
+ * several such pairs in a caller's lists only the one with the lowest input row is kept (and the
+ * tail of that offset's range in in_sorted / out_sorted is left unwritten, beyond the counts in
+ * group_start).  in_sorted / out_sorted have room for host_offsets[K] pairs.  Kernels only. */
+size_t wcn_pairs_sort_workspace_bytes(int64_t num_out, int32_t num_offsets, int64_t num_pairs);
+
+int wcn_pairs_sort_by_out(const int32_t* in_maps, const int32_t* out_maps, const int64_t* host_offsets,
+                          int32_t num_offsets, int64_t num_out, int32_t* in_sorted,
+                          int32_t* out_sorted, int32_t* group_start, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Gradients of the contraction.  Replace the per-offset loops of the reference backward
  * (sparse_conv.py:314-355 explicit, :418-492 implicit, :547-627 CUTLASS) and the native calls

@@ -134,6 +134,62 @@ def test_strided_then_transposed_pair(oracle, dtype):
     assert rel_err(back.feature_tensor.float().cpu().numpy(), want) <= TOL[dtype]
 
 
+def test_pair_lists_are_reordered_once_and_kept_on_the_map(oracle):
+    """The map of a transposed convolution does not ascend in output row: its re-ordered lists
+    are made on the first product and the very same tensors serve the second one."""
+    import ctypes
+    from warpconvnet_amd._lib import check, lib, ptr, stream_ptr, workspace
+    from warpconvnet_amd.nn.functional.sparse_conv import (generate_output_coords_and_kernel_map,
+                                                         spatially_sparse_conv)
+    items = [synthetic.random_cloud(40 + b, 6000, 32)[:, 1:] for b in range(2)]
+    bc = synthetic.batch_indexed(items)
+    x = normal_features(len(bc), 16, seed=11)
+    fine = _voxels(items, x)
+    w = kaiming_weight(8, 16, 32, seed=12)
+    coarse = spatially_sparse_conv(fine, w.to(DEV), 2, stride=2)
+    wt = kaiming_weight(8, 32, 16, seed=13).to(DEV)
+    first = spatially_sparse_conv(coarse, wt, 2, stride=2, transposed=True,
+                                  output_spatially_sparse_tensor=fine)
+    _, _, km = generate_output_coords_and_kernel_map(
+        coarse, (2, 2, 2), (1, 1, 1), (2, 2, 2), False, True, output_spatially_sparse_tensor=fine)
+    assert km._by_out is not None and not km._out_ascend
+    kept = km._by_out
+    second = spatially_sparse_conv(coarse, wt, 2, stride=2, transposed=True,
+                                   output_spatially_sparse_tensor=fine)
+    assert km._by_out is kept
+    assert torch.equal(first.feature_tensor, second.feature_tensor)
+    # the kept lists: same pairs per offset, ascending output rows, group starts by definition
+    K = len(km)
+    off = km.offsets.tolist()
+    gi, go, groups = (t.cpu().numpy() for t in kept[:3])
+    im, om = km.in_maps.cpu().numpy(), km.out_maps.cpu().numpy()
+    M = len(bc)
+    G = (M + 63) // 64
+    groups = groups.reshape(K, G + 1)
+    for k in range(K):
+        a, b = off[k], off[k + 1]
+        assert np.all(np.diff(go[a:b]) > 0)
+        order = np.argsort(om[a:b], kind="stable")
+        assert np.array_equal(go[a:b], om[a:b][order]) and np.array_equal(gi[a:b], im[a:b][order])
+        assert np.array_equal(groups[k], np.searchsorted(go[a:b], 64 * np.arange(G + 1)))
+
+    # direct call with duplicate (offset, output row) pairs: the lowest input row is kept
+    L = lib()
+    in_l = torch.tensor([9, 3, 7, 5, 1, 8], dtype=torch.int32, device=DEV)
+    out_l = torch.tensor([2, 2, 0, 2, 1, 1], dtype=torch.int32, device=DEV)  # offset 0: rows 2,2,0,2; offset 1: 1,1
+    host_off = (ctypes.c_int64 * 3)(0, 4, 6)
+    for _ in range(3):
+        ins = torch.full((6,), -7, dtype=torch.int32, device=DEV)
+        outs = torch.full((6,), -7, dtype=torch.int32, device=DEV)
+        gs = torch.empty(2 * 2, dtype=torch.int32, device=DEV)
+        ws = workspace(L.wcn_pairs_sort_workspace_bytes(3, 2, 6), torch.device(DEV))
+        check(L.wcn_pairs_sort_by_out(ptr(in_l), ptr(out_l), host_off, 2, 3, ptr(ins), ptr(outs), ptr(gs),
+                                      ptr(ws), ws.numel(), stream_ptr(torch.device(DEV))), "sort")
+        assert gs.tolist() == [0, 2, 0, 1]
+        assert ins.tolist()[:2] == [7, 3] and outs.tolist()[:2] == [0, 2]
+        assert ins.tolist()[4] == 1 and outs.tolist()[4] == 1
+
+
 def test_transposed_adjoint_identity():
     """<conv(x), y> == <x, conv_T(y)> when the transposed weights are W[k]^T on the same map."""
     from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv

@@ -42,6 +42,8 @@ SIGNATURES = {
                                            _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
     "wcn_sparse_conv_fwd_static": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                                   _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp]),
+    "wcn_pairs_sort_workspace_bytes": (_sz, [_i64, _i32, _i64]),
+    "wcn_pairs_sort_by_out": (ctypes.c_int, [_vp, _vp, _i64p, _i32, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "wcn_sparse_conv_dgrad": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                              _i64p, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
     "wcn_map_rows_workspace_bytes": (_sz, [_i64, _i32, _i64]),

@@ -905,10 +905,10 @@ __device__ __forceinline__ int offset_of_pair(const int64_t* __restrict__ offset
   return lo;
 }
 
-__global__ void __launch_bounds__(256) rows_clear(uint32_t* __restrict__ row_mask, int64_t n) {
+__global__ void __launch_bounds__(256) rows_clear(uint32_t* __restrict__ words, int64_t n, uint32_t value) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (int64_t)gridDim.x * blockDim.x)
-    row_mask[i] = 0u;
+    words[i] = value;
 }
 
 __global__ void __launch_bounds__(256) rows_mark(const int32_t* __restrict__ out_maps,
@@ -948,6 +948,9 @@ __global__ void __launch_bounds__(256) rows_fill(const int32_t* __restrict__ in_
                                                  const uint32_t* __restrict__ row_mask,
                                                  const int32_t* __restrict__ row_ptr,
                                                  int32_t* __restrict__ row_in) {
+  // row_in starts at INT32_MAX everywhere: of several pairs with the same (offset, output row),
+  // which a kernel map never holds but a caller's lists may, the lowest input row survives,
+  // whatever order the threads run in.
   const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= offsets[K]) return;
   const int k = offset_of_pair(offsets, K, p);
@@ -957,7 +960,7 @@ __global__ void __launch_bounds__(256) rows_fill(const int32_t* __restrict__ in_
   int rank = 0;
   for (int w = 0; w < (k >> 5); ++w) rank += __popc(mw[w]);
   rank += __popc(mw[k >> 5] & ((1u << (k & 31)) - 1u));
-  row_in[row_ptr[o] + rank] = in_maps[p];
+  atomicMin(&row_in[row_ptr[o] + rank], in_maps[p]);
 }
 
 // Output-row form -> pair lists that ascend in output row inside every offset, plus their
@@ -1193,7 +1196,10 @@ int wcn_rows_build(const int32_t* in_maps, const int32_t* out_maps, int num_offs
   const unsigned rows_grid = (unsigned)((num_out + 255) / 256);
   const int64_t mask_words = num_out * v.words;
   hipLaunchKernelGGL(rows_clear, dim3((unsigned)std::min<int64_t>(4096, (mask_words + 255) / 256)),
-                     dim3(256), 0, s, v.row_mask, mask_words);
+                     dim3(256), 0, s, v.row_mask, mask_words, 0u);
+  if (pairs > 0)
+    hipLaunchKernelGGL(rows_clear, dim3((unsigned)std::min<int64_t>(4096, (pairs + 255) / 256)),
+                       dim3(256), 0, s, (uint32_t*)v.row_in, pairs, 0x7fffffffu);
   if (pairs > 0)
     hipLaunchKernelGGL(rows_mark, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, s, out_maps,
                        (const int64_t*)v.offsets, num_offsets, v.words, num_out, v.row_mask);
@@ -1216,6 +1222,75 @@ int wcn_conv_set_timing_events(void* start_event, void* stop_event) {
   g_time_start = (hipEvent_t)start_event;
   g_time_stop = (hipEvent_t)stop_event;
   return WCN_OK;
+}
+
+// pair lists -> output-row form -> pair lists ascending in output row inside every offset, with
+// their group_start table.  Of several pairs with the same (offset, output row) one is kept.
+static void pairs_sort_by_out(const int32_t* in_maps, const int32_t* out_maps, const int64_t* offsets_dev,
+                              int K, int64_t num_out, int64_t L, uint32_t* row_mask, int32_t* row_ptr,
+                              int32_t* row_in, int32_t* groups, int64_t* row_total, int32_t* in_sorted,
+                              int32_t* out_sorted, int32_t* group_start, hipStream_t s) {
+  const int words = (K + 31) / 32;
+  const int64_t G = (num_out + 63) / 64;
+  const unsigned rows_grid = (unsigned)((num_out + 255) / 256);
+  const int64_t mask_words = num_out * words;
+  hipLaunchKernelGGL(rows_clear, dim3((unsigned)std::min<int64_t>(4096, (mask_words + 255) / 256)),
+                     dim3(256), 0, s, row_mask, mask_words, 0u);
+  if (L > 0) {
+    hipLaunchKernelGGL(rows_clear, dim3((unsigned)std::min<int64_t>(4096, (L + 255) / 256)), dim3(256),
+                       0, s, (uint32_t*)row_in, L, 0x7fffffffu);
+    hipLaunchKernelGGL(rows_mark, dim3((unsigned)((L + 255) / 256)), dim3(256), 0, s, out_maps,
+                       offsets_dev, K, words, num_out, row_mask);
+  }
+  hipLaunchKernelGGL(rows_count<false>, dim3(rows_grid), dim3(256), 0, s, (const uint32_t*)row_mask,
+                     words, num_out, groups, row_ptr);
+  wcn_scan_rows_launch(groups, G, 1, row_total, s);
+  hipLaunchKernelGGL(rows_count<true>, dim3(rows_grid), dim3(256), 0, s, (const uint32_t*)row_mask,
+                     words, num_out, groups, row_ptr);
+  if (L > 0)
+    hipLaunchKernelGGL(rows_fill, dim3((unsigned)((L + 255) / 256)), dim3(256), 0, s, in_maps, out_maps,
+                       offsets_dev, K, words, num_out, (const uint32_t*)row_mask,
+                       (const int32_t*)row_ptr, row_in);
+  hipLaunchKernelGGL(rows_to_pairs<false>, dim3(rows_grid), dim3(256), 0, s, (const uint32_t*)row_mask,
+                     (const int32_t*)row_ptr, (const int32_t*)row_in, K, words, num_out, offsets_dev,
+                     group_start, G, in_sorted, out_sorted);
+  wcn_scan_rows_launch(group_start, G, K, row_total, s);
+  hipLaunchKernelGGL(rows_to_pairs<true>, dim3(rows_grid), dim3(256), 0, s, (const uint32_t*)row_mask,
+                     (const int32_t*)row_ptr, (const int32_t*)row_in, K, words, num_out, offsets_dev,
+                     group_start, G, in_sorted, out_sorted);
+}
+
+struct SortWorkspace {
+  int64_t* offsets;
+  int64_t* row_total;
+  uint32_t* row_mask;
+  int32_t* row_ptr;
+  int32_t* row_in;
+  int32_t* groups;
+};
+
+inline size_t sort_layout(void* base, int64_t num_out, int K, int64_t L, SortWorkspace* w) {
+  char* p = (char*)base;
+  size_t off = 0;
+  const int64_t G = (num_out + 63) / 64;
+  const int words = (K + 31) / 32;
+  if (w) w->offsets = (int64_t*)(p + off);
+  off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
+  if (w) w->row_total = (int64_t*)(p + off);
+  off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
+  if (w) w->row_mask = (uint32_t*)(p + off);
+  off += wcn_align256(sizeof(uint32_t) * (size_t)num_out * words);
+  if (w) w->row_ptr = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)(num_out + 1));
+  if (w) w->row_in = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)L);
+  if (w) w->groups = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)(G + 1));
+  return off;
+}
+
+__global__ void offsets_store(OffsetsByValue ov, int n, int64_t* __restrict__ dst) {
+  if ((int)threadIdx.x < n) dst[threadIdx.x] = ov.v[threadIdx.x];
 }
 
 size_t wcn_conv_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_in, int32_t c_out,
@@ -1301,33 +1376,10 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   a.in_maps = in_maps;
   a.out_maps = out_maps;
   a.group_start = group_start_or_null;
-  const unsigned rows_grid = (unsigned)((num_out + 255) / 256);
   if (!out_maps_ascend) {
-    // pair lists -> output-row form -> pair lists ascending in output row, with group_start
-    const int64_t mask_words = num_out * w.words;
-    hipLaunchKernelGGL(rows_clear, dim3((unsigned)std::min<int64_t>(4096, (mask_words + 255) / 256)),
-                       dim3(256), 0, s, w.row_mask, mask_words);
-    if (L > 0)
-      hipLaunchKernelGGL(rows_mark, dim3((unsigned)((L + 255) / 256)), dim3(256), 0, s, out_maps,
-                         (const int64_t*)w.offsets, num_offsets, w.words, num_out, w.row_mask);
-    hipLaunchKernelGGL(rows_count<false>, dim3(rows_grid), dim3(256), 0, s,
-                       (const uint32_t*)w.row_mask, w.words, num_out, w.groups, w.row_ptr);
-    wcn_scan_rows_launch(w.groups, w.G, 1, w.row_total, s);
-    hipLaunchKernelGGL(rows_count<true>, dim3(rows_grid), dim3(256), 0, s,
-                       (const uint32_t*)w.row_mask, w.words, num_out, w.groups, w.row_ptr);
-    if (L > 0)
-      hipLaunchKernelGGL(rows_fill, dim3((unsigned)((L + 255) / 256)), dim3(256), 0, s, in_maps,
-                         out_maps, (const int64_t*)w.offsets, num_offsets, w.words, num_out,
-                         (const uint32_t*)w.row_mask, (const int32_t*)w.row_ptr, w.row_in);
-    hipLaunchKernelGGL(rows_to_pairs<false>, dim3(rows_grid), dim3(256), 0, s,
-                       (const uint32_t*)w.row_mask, (const int32_t*)w.row_ptr,
-                       (const int32_t*)w.row_in, num_offsets, w.words, num_out,
-                       (const int64_t*)w.offsets, w.group_start, w.G, w.in_sorted, w.out_sorted);
-    wcn_scan_rows_launch(w.group_start, w.G, num_offsets, w.row_total, s);
-    hipLaunchKernelGGL(rows_to_pairs<true>, dim3(rows_grid), dim3(256), 0, s,
-                       (const uint32_t*)w.row_mask, (const int32_t*)w.row_ptr,
-                       (const int32_t*)w.row_in, num_offsets, w.words, num_out,
-                       (const int64_t*)w.offsets, w.group_start, w.G, w.in_sorted, w.out_sorted);
+    pairs_sort_by_out(in_maps, out_maps, (const int64_t*)w.offsets, num_offsets, num_out, L, w.row_mask,
+                      w.row_ptr, w.row_in, w.groups, w.row_total, w.in_sorted, w.out_sorted,
+                      w.group_start, s);
     a.in_maps = w.in_sorted;
     a.out_maps = w.out_sorted;
     a.group_start = w.group_start;
@@ -1399,6 +1451,40 @@ int wcn_sparse_conv_fwd_static(const void* features, int64_t num_in, int32_t c_i
                   bias_or_null, in_maps, out_maps, host_offsets, identity_offset, out_maps_ascend,
                   group_start_or_null, out, num_out, ws, WCN_CONV_STATIC_SCRATCH_BYTES, 0, 0, true,
                   stream);
+}
+
+size_t wcn_pairs_sort_workspace_bytes(int64_t num_out, int32_t num_offsets, int64_t num_pairs) {
+  if (num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || num_pairs < 0) return 0;
+  return sort_layout(nullptr, num_out, num_offsets, num_pairs, nullptr);
+}
+
+int wcn_pairs_sort_by_out(const int32_t* in_maps, const int32_t* out_maps, const int64_t* host_offsets,
+                          int32_t num_offsets, int64_t num_out, int32_t* in_sorted,
+                          int32_t* out_sorted, int32_t* group_start, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  if (!host_offsets || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || num_out < 0 ||
+      num_out >= (1ll << 31) || !group_start || !workspace)
+    return WCN_ERR_INVALID_ARGUMENT;
+  const int64_t L = host_offsets[num_offsets];
+  if (host_offsets[0] != 0 || L < 0 || L > INT32_MAX) return WCN_ERR_INVALID_ARGUMENT;
+  for (int k = 0; k < num_offsets; ++k)
+    if (host_offsets[k + 1] < host_offsets[k]) return WCN_ERR_INVALID_ARGUMENT;
+  if (L > 0 && (!in_maps || !out_maps || !in_sorted || !out_sorted)) return WCN_ERR_INVALID_ARGUMENT;
+  if (workspace_bytes < sort_layout(nullptr, num_out, num_offsets, L, nullptr)) return WCN_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  SortWorkspace w;
+  sort_layout(workspace, num_out, num_offsets, L, &w);
+  if (num_offsets + 1 <= OFFSETS_BY_VALUE) {
+    OffsetsByValue ov;
+    for (int i = 0; i < OFFSETS_BY_VALUE; ++i) ov.v[i] = i <= num_offsets ? host_offsets[i] : 0;
+    hipLaunchKernelGGL(offsets_store, dim3(1), dim3(OFFSETS_BY_VALUE), 0, s, ov, num_offsets + 1, w.offsets);
+  } else if (hipMemcpyAsync(w.offsets, host_offsets, sizeof(int64_t) * (size_t)(num_offsets + 1),
+                            hipMemcpyHostToDevice, s) != hipSuccess) {
+    return WCN_ERR_LAUNCH;
+  }
+  pairs_sort_by_out(in_maps, out_maps, w.offsets, num_offsets, num_out, L, w.row_mask, w.row_ptr,
+                    w.row_in, w.groups, w.row_total, in_sorted, out_sorted, group_start, s);
+  return hipGetLastError() == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
 }
 
 int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,

@@ -217,7 +217,9 @@ __global__ void __launch_bounds__(256) table_query(const WcnTableHeader* __restr
 
 inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
 
-inline int grid_for(int64_t n, int block, int cap = 1 << 20) {
+// One-item-per-thread kernels take the uncapped grid (a grid's x extent reaches 2^31 - 1 blocks, and
+// item counts here stay below 2^31); a cap is for kernels that loop with a grid stride.
+inline int grid_for(int64_t n, int block, int cap = 0x7fffffff) {
   int64_t g = (n + block - 1) / block;
   if (g < 1) g = 1;
   if (g > cap) g = cap;

@@ -37,6 +37,13 @@ class IntSearchResult:
         self._in_ascend = False
         self._in_group_start = None
         self._symmetric = False
+        # The pair lists re-ordered once for the contraction, kept with the map: ascending in
+        # out_maps (`_by_out`, for the forward product over a map whose out_maps does not ascend:
+        # the map of a transposed convolution) and ascending in in_maps (`_by_in`, for the input
+        # gradient over a map that is not symmetric).  Each is (first list, second list,
+        # group-start table, row count) or None until first needed.
+        self._by_out = None
+        self._by_in = None
 
     @torch.no_grad()
     def __getitem__(self, idx: int) -> Tuple[Tensor, Tensor]:

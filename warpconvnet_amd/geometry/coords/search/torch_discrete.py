@@ -98,7 +98,10 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
         table._checked = True
         break
     total = int(host_offsets[K])
-    if total <= assumed:
+    if 2 * total <= assumed:
+        # far fewer pairs than assumed: exact copies, so the map does not hold the large buffers
+        in_maps, out_maps = in_buf[:total].clone(), out_buf[:total].clone()
+    elif total <= assumed:
         in_maps, out_maps = in_buf[:total], out_buf[:total]
     else:
         in_maps = torch.empty(total, dtype=torch.int32, device=device)
@@ -109,9 +112,13 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     result = IntSearchResult(in_maps, out_maps, offsets, identity_map_index=identity_map_index)
     result._host_offsets = host_offsets  # the contraction passes them on as they are
     # by-products the contraction reuses: pairs ascend in output row inside every offset, and
-    # the workspace (kept alive by the reference below) holds their per-64-row group starts
+    # the workspace holds their per-64-row group starts, (K, G + 1) int32.  Only that table is
+    # kept with the map (a copy of about K * M / 16 bytes); the workspace itself, whose probe
+    # results are K * M * 4 bytes, goes back to the allocator here.
     result._out_ascend = True
-    result._group_start = (ws, L.wcn_kmap_group_start(ptr(ws), M, K), (K, M))
+    begin = L.wcn_kmap_group_start(ptr(ws), M, K) - ws.data_ptr()
+    groups = ws[begin:begin + 4 * K * ((M + 63) // 64 + 1)].clone()
+    result._group_start = (groups, groups.data_ptr(), (K, M))
     result._keys_unique = (L.wcn_kmap_last_table_flags() & 1) == 0
     return result
 

@@ -77,6 +77,38 @@ def _host_offsets_of(km: IntSearchResult):
 
 
 @torch.no_grad()
+def _pairs_sorted(km: IntSearchResult, by: str, num_rows: int):
+    """The map's pair lists re-ordered so that the `by` side ("out" or "in") ascends inside every
+    offset, with the table of per-64-row group starts of that order: made by the library on first
+    use and kept on the map object, so a cached map pays for it once (the reference caches the
+    exchanged map of a transposed convolution the same way, sparse_conv.py:1916-1939).
+    Returns (gathered-side list, ascending-side list, group-start tensor)."""
+    kept = km._by_out if by == "out" else km._by_in
+    if kept is not None and kept[3] == num_rows:
+        return kept[:3]
+    gathered, ascending = (km.in_maps, km.out_maps) if by == "out" else (km.out_maps, km.in_maps)
+    K = len(km)
+    device = gathered.device
+    L = lib()
+    host_offsets = _host_offsets_of(km)
+    num_pairs = int(host_offsets[K])
+    g_sorted = torch.empty(num_pairs, dtype=torch.int32, device=device)
+    a_sorted = torch.empty(num_pairs, dtype=torch.int32, device=device)
+    groups = torch.empty(K * ((num_rows + 63) // 64 + 1), dtype=torch.int32, device=device)
+    ws = workspace(L.wcn_pairs_sort_workspace_bytes(num_rows, K, num_pairs), device)
+    check(L.wcn_pairs_sort_by_out(ptr(gathered.contiguous()), ptr(ascending.contiguous()),
+                                  host_offsets, K, num_rows, ptr(g_sorted), ptr(a_sorted),
+                                  ptr(groups), ptr(ws), ws.numel(), stream_ptr(device)),
+          "wcn_pairs_sort_by_out")
+    kept = (g_sorted, a_sorted, groups, num_rows)
+    if by == "out":
+        km._by_out = kept
+    else:
+        km._by_in = kept
+    return kept[:3]
+
+
+@torch.no_grad()
 def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSearchResult,
                         num_out_coords: int, bias: Optional[Tensor] = None,
                         compute_dtype: Optional[torch.dtype] = None) -> Tensor:
@@ -110,10 +142,16 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
     device = x.device
     out = torch.empty((num_out_coords, c_out), dtype=x.dtype, device=device)
     L = lib()
-    ascend = 1 if km._out_ascend else 0
+    in_maps, out_maps = km.in_maps, km.out_maps
     group_start = None
-    if ascend and km._group_start is not None and km._group_start[2] == (K, num_out_coords):
+    if not km._out_ascend and num_out_coords > 0:
+        # a map whose out_maps does not ascend (transposed convolution, caller-made lists) is
+        # re-ordered once and the result kept on the map object
+        in_maps, out_maps, groups = _pairs_sorted(km, "out", num_out_coords)
+        group_start = ptr(groups)
+    elif km._group_start is not None and km._group_start[2] == (K, num_out_coords):
         group_start = ctypes.c_void_p(km._group_start[1])
+    ascend = 1
     host_offsets = _host_offsets_of(km)
     num_pairs = int(host_offsets[K])
     nbytes = L.wcn_conv_workspace_bytes(num_out_coords, K, c_in, c_out, DTYPE_CODE[x.dtype],
@@ -121,8 +159,8 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
     ws = workspace(nbytes, device)
     iden = -1 if km.identity_map_index is None else int(km.identity_map_index)
     check(L.wcn_sparse_conv_fwd(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(w),
-                                DTYPE_CODE[w.dtype], K, c_out, ptr(b), ptr(km.in_maps),
-                                ptr(km.out_maps), host_offsets, iden, ascend, group_start,
+                                DTYPE_CODE[w.dtype], K, c_out, ptr(b), ptr(in_maps),
+                                ptr(out_maps), host_offsets, iden, ascend, group_start,
                                 ptr(out), num_out_coords, ptr(ws), ws.numel(), stream_ptr(device)),
           "wcn_sparse_conv_fwd")
     return out if out.dtype == in_features.dtype else out.to(in_features.dtype)
@@ -168,17 +206,23 @@ def sparse_conv_backward(grad_output: Tensor, in_features: Tensor, weight: Tenso
             grad_x = torch.zeros_like(x)
         else:
             symmetric = 1 if (km._symmetric and km._out_ascend and n_in == n_out) else 0
-            ascend = 1 if (symmetric or km._in_ascend) else 0
-            gs = km._group_start if symmetric else km._in_group_start
+            in_maps, out_maps = km.in_maps, km.out_maps
             group_start = None
-            if ascend and gs is not None and gs[2] == (K, n_in):
-                group_start = ctypes.c_void_p(gs[1])
+            if not symmetric and not km._in_ascend:
+                # general map: the lists ascending in input row are made once per map object
+                out_maps, in_maps, groups = _pairs_sorted(km, "in", n_in)
+                group_start = ptr(groups)
+            else:
+                gs = km._group_start if symmetric else km._in_group_start
+                if gs is not None and gs[2] == (K, n_in):
+                    group_start = ctypes.c_void_p(gs[1])
+            ascend = 1
             ws = workspace(L.wcn_conv_workspace_bytes(n_in, K, c_out, c_in, code, num_pairs, ascend),
                            device)
             grad_x = torch.empty((n_in, c_in), dtype=dtype, device=device)
             check(L.wcn_sparse_conv_dgrad(ptr(gy), n_out, c_out, code, ptr(w), DTYPE_CODE[w.dtype], K,
-                                          c_in, ptr(km.in_maps), ptr(km.out_maps), host_offsets, iden,
-                                          symmetric, 1 if km._in_ascend else 0, group_start,
+                                          c_in, ptr(in_maps), ptr(out_maps), host_offsets, iden,
+                                          symmetric, 1, group_start,
                                           ptr(grad_x), n_in, ptr(ws), ws.numel(), stream_ptr(device)),
                   "wcn_sparse_conv_dgrad")
         grad_x = grad_x.to(in_features.dtype)
