@@ -1,6 +1,7 @@
 """Compiles the HIP sources under csrc/ into warpconvnet_amd/libwcn_hip.so for gfx950."""
 import glob
 import os
+import re
 import shutil
 import subprocess
 
@@ -63,6 +64,47 @@ def _check_no_scratch(src, log):
         raise RuntimeError(f"{os.path.basename(src)}: no resource-usage remarks found; cannot vouch for its kernels")
 
 
+def _vgprs_in(text):
+    regs = set()
+    for m in re.finditer(r"v\[(\d+):(\d+)\]", text):
+        regs.update(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in re.finditer(r"(?<![\w\[])v(\d+)\b", text):
+        regs.add(int(m.group(1)))
+    return regs
+
+
+def _check_loads_not_copied(src, asm_text):
+    """The destination of a written-out load must not be read or moved before a vmcnt wait: a
+    copy the compiler inserts between the load and its wait (at a control-flow merge, say) would
+    carry the register's old contents.  Checked on the generated code, in program-text order,
+    over the copy-like instructions of the 400 lines after each such load."""
+    lines = asm_text.split("\n")
+    code = [l.split(";")[0].rstrip() for l in lines]
+    in_asm, bad = False, []
+    for i, raw in enumerate(lines):
+        if "#ASMSTART" in raw:
+            in_asm = True
+            continue
+        if "#ASMEND" in raw:
+            in_asm = False
+            continue
+        m = re.match(r"\s*global_load_dword(x2|x4)?\s+(\S+),", code[i])
+        if not (in_asm and m):
+            continue
+        dst = _vgprs_in(m.group(2))
+        for j in range(i + 1, min(len(code), i + 400)):
+            st = code[j].strip()
+            if "s_endpgm" in st or ("s_waitcnt" in st and "vmcnt" in st):
+                break
+            ops = st.split(None, 1)
+            if len(ops) > 1 and re.match(r"v_(mov|cndmask|accvgpr|perm|swap)", st) and _vgprs_in(ops[1]) & dst:
+                bad.append(f"line {i + 1}: {code[i].strip()}  ->  line {j + 1}: {st}")
+                break
+    if bad:
+        raise RuntimeError(f"{os.path.basename(src)}: the compiler moves registers that loads are still in flight "
+                           "into:\n  " + "\n  ".join(bad[:10]))
+
+
 def build_library(verbose: bool = False) -> str:
     """Every source file is compiled to an object of its own (in parallel), then linked."""
     from concurrent.futures import ThreadPoolExecutor
@@ -80,6 +122,13 @@ def build_library(verbose: bool = False) -> str:
         logs = list(pool.map(_run, cmds))
     for src, log in zip(sources, logs):
         _check_no_scratch(src, log)
+    for src in sources:
+        if os.path.basename(src) in NO_SCRATCH_SOURCES:
+            asm_path = os.path.join(objdir, os.path.basename(src)[:-4] + ".s")
+            _run([hipcc, *compile_flags, "-S", "--cuda-device-only", "-o", asm_path, src])
+            with open(asm_path) as f:
+                _check_loads_not_copied(src, f.read())
+            os.remove(asm_path)
     logs = [_without_remarks(log) for log in logs]
     logs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", LIB_PATH, *objects]))
     if verbose:

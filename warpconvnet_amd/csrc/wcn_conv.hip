@@ -1104,8 +1104,7 @@ int launch_conv(const ConvArgs& a, hipStream_t s) {
   constexpr int dtype = std::is_same<T, float>::value ? WCN_DTYPE_F32
                         : std::is_same<T, _Float16>::value ? WCN_DTYPE_F16 : WCN_DTYPE_BF16;
   // Rows of at most one k-slice go to the pair-packed kernel.  WCN_CONV_KERNEL=ring in the
-  // environment keeps them on the output-stationary kernels below, whose results are bitwise
-  // reproducible from run to run (no atomics).
+  // environment keeps them on the output-stationary kernels below (for comparisons).
   static const bool ring_only = [] {
     const char* e = getenv("WCN_CONV_KERNEL");
     return e && std::string(e) == "ring";
