@@ -25,12 +25,66 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
 
-# Bytes the contraction kernel moves between L2 and the memory fabric per launch on this workload,
-# from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch),
-# each scaled by what the same counter reads for the 1 GiB device copy of --calibrate-copy
-# (FETCH_SIZE reads 0.5 GiB for it -> x2.0; WRITE_SIZE reads 1 GiB -> x1.0).  Summary kept in
-# profiles/conv_fwd_cfg2_hbm_traffic.txt; to be re-measured whenever the kernel changes.
-CONV_FWD_TRAFFIC_BYTES = (282610 * 2.0 + 160171 * 1.0) * 1024
+# Bytes the contraction kernel moves between L2 and the memory fabric per launch on this workload
+# come from the committed counter summary (two `rocprofv3 --pmc` runs of this script: FETCH_SIZE,
+# then WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB device copy of
+# --calibrate-copy).  The summary names the kernel it was taken from; a line for another kernel
+# than the one this run launches is reported as stale (traffic: null).
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "conv_fwd_cfg2_hbm_traffic.txt")
+CONV_KERNEL = "conv_fwd_pack<f16, 512, 7, 4, 2, true>"  # what wcn_sparse_conv_fwd launches for 64 -> 64 fp16
+
+
+def measured_traffic():
+    """(bytes per launch or None, note) from the line `TRAFFIC_JSON: {...}` of the summary."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                if line.startswith("TRAFFIC_JSON:"):
+                    rec = json.loads(line[len("TRAFFIC_JSON:"):])
+                    if rec.get("kernel") != CONV_KERNEL or os.environ.get("WCN_CONV_KERNEL"):
+                        return None, f"stale: {os.path.basename(TRAFFIC_FILE)} holds {rec.get('kernel')}"
+                    total = (rec["fetch_kib"] * rec["fetch_factor"] + rec["write_kib"] * rec["write_factor"]) * 1024
+                    return float(total), f"{os.path.basename(TRAFFIC_FILE)} (tree {rec.get('tree', '?')})"
+    except (OSError, ValueError, KeyError):
+        pass
+    return None, "no counter summary found"
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def measured_peaks(dev):
+    """What this GPU reaches on two plain library operations, beside the published peaks: a 1 GiB
+    device copy (bytes read + written per second) and an 8192^3 fp16 GEMM."""
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    a = torch.randn(8192, 8192, device=dev, dtype=torch.float16)
+    b = torch.randn(8192, 8192, device=dev, dtype=torch.float16)
+    out = {}
+    for name, fn, work in (("stream_copy_GBps", lambda: dst.copy_(src), 2.0 * (1 << 30) / 1e9),
+                           ("fp16_gemm_8192_TFLOPs", lambda: torch.matmul(a, b), 2.0 * 8192 ** 3 / 1e12)):
+        for _ in range(3):
+            fn()
+        times = []
+        for _ in range(10):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) * 1e-3)
+        out[name] = work / float(np.median(times))
+    del src, dst, a, b
+    return out
+
 
 METRIC = "voxels/sec, 3x3x3 C64->64 fp16 conv @1M voxels; kernel-map build ms"
 
@@ -46,20 +100,53 @@ def make_workload(batch=4, per_item=250_000, c_in=64, c_out=64, seed=0):
     return bcoords, offsets, feats, weight
 
 
+def _cpu_kernel_map_by_item(bcoords, threads):
+    """The scalar C oracle's kernel map, one batch item per host thread (the items are independent:
+    a pair never crosses items), merged into one map."""
+    from concurrent.futures import ThreadPoolExecutor
+    from oracle import cpu_oracle
+    batch = bcoords[:, 0]
+    bounds = np.flatnonzero(np.diff(batch)) + 1
+    starts = np.concatenate([[0], bounds, [len(bcoords)]])
+    parts = [np.ascontiguousarray(bcoords[a:b]) for a, b in zip(starts[:-1], starts[1:])]
+    with ThreadPoolExecutor(max_workers=max(1, min(threads, len(parts)))) as pool:
+        maps = list(pool.map(lambda c: cpu_oracle.kernel_map(c, c, (3, 3, 3)), parts))
+    K = len(maps[0][2]) - 1
+    ins, outs, off = [], [], [0]
+    for k in range(K):
+        for (im, om, o, _), base in zip(maps, starts[:-1]):
+            ins.append(im[o[k]:o[k + 1]] + base)
+            outs.append(om[o[k]:o[k + 1]] + base)
+        off.append(off[-1] + sum(int(m[2][k + 1] - m[2][k]) for m in maps))
+    return (np.concatenate(ins).astype(np.int32), np.concatenate(outs).astype(np.int32),
+            np.asarray(off, dtype=np.int64), maps[0][3])
+
+
 def cpu_baseline(bcoords, feats, weight):
     """The reference's explicit gather-GEMM-scatter algorithm (torch-CPU restatement, computed in
     fp32 through the reference's own compute_dtype knob) on the host cores, with the kernel map
-    from the scalar C oracle.  Full workload, one pass each."""
+    from the scalar C oracle.  Full workload, one pass each, twice: on all host threads (the map
+    one batch item per thread) and on a single thread."""
     from oracle import cpu_oracle
     from oracle.explicit_conv import explicit_gemm_forward
     threads = os.cpu_count() or 1
     threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
-    torch.set_num_threads(threads)
+    n = len(bcoords)
+    # single thread
+    torch.set_num_threads(1)
     t0 = time.perf_counter()
     im, om, off, iden = cpu_oracle.kernel_map(bcoords, bcoords, (3, 3, 3))
-    t_map = time.perf_counter() - t0
+    t_map1 = time.perf_counter() - t0
     im_t, om_t = torch.as_tensor(im), torch.as_tensor(om)
-    n = len(bcoords)
+    t0 = time.perf_counter()
+    explicit_gemm_forward(feats, weight, im_t, om_t, off, iden, n, compute_dtype=torch.float32)
+    t_conv1 = time.perf_counter() - t0
+    # all threads
+    torch.set_num_threads(threads)
+    t0 = time.perf_counter()
+    im_p, om_p, off_p, iden_p = _cpu_kernel_map_by_item(bcoords, threads)
+    t_map = time.perf_counter() - t0
+    assert iden_p == iden and np.array_equal(off_p, off) and np.array_equal(im_p, im) and np.array_equal(om_p, om)
     explicit_gemm_forward(feats[:1000], weight, im_t[:0], om_t[:0], [0] * 28, None, 1000,
                           compute_dtype=torch.float32)  # warm the thread pool
     t0 = time.perf_counter()
@@ -70,11 +157,14 @@ def cpu_baseline(bcoords, feats, weight):
         "unit": "voxels/s",
         "cores": threads,
         "kind": "port",
+        "cpu": cpu_model(),
         "sample": (f"full workload once: {n} voxels, {int(off[-1])} pairs; kernel map by the scalar "
-                   f"C oracle on 1 thread ({t_map * 1e3:.0f} ms) + explicit gather-GEMM-scatter in "
-                   f"torch fp32 on {threads} threads ({t_conv * 1e3:.0f} ms)"),
+                   f"C oracle, one batch item per thread ({t_map * 1e3:.0f} ms) + explicit "
+                   f"gather-GEMM-scatter in torch fp32 on {threads} threads ({t_conv * 1e3:.0f} ms)"),
         "map_ms": t_map * 1e3,
         "conv_ms": t_conv * 1e3,
+        "single_thread": {"value": n / (t_map1 + t_conv1), "unit": "voxels/s", "cores": 1,
+                          "map_ms": t_map1 * 1e3, "conv_ms": t_conv1 * 1e3},
     }, out, (im, om, off)
 
 
@@ -390,9 +480,41 @@ def main():
         gc.enable()
 
     ms_per_step = elapsed * 1e3 / args.steps
-    map_ms = float(np.mean([s.elapsed_time(m) for s, m in zip(starts, mids)]))
-    conv_call_ms = float(np.mean([m.elapsed_time(e) for m, e in zip(mids, ends)]))
-    conv_kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in kernel_events]))
+    # medians over the steps (the wall-clock figure above is the mean of the same K steps)
+    map_ms = float(np.median([s.elapsed_time(m) for s, m in zip(starts, mids)]))
+    conv_call_ms = float(np.median([m.elapsed_time(e) for m, e in zip(mids, ends)]))
+    conv_kernel_ms = float(np.median([a.elapsed_time(b) for a, b in kernel_events]))
+    step_device_ms = float(np.median([s.elapsed_time(e) for s, e in zip(starts, ends)]))
+
+    # The same cold step through the module interface: SpatiallySparseConv.forward on a Voxels
+    # object made anew in every step (no cached table or map), as a caller of the reference does.
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d
+    module = SparseConv3d(64, 64, 3, bias=False).to(dev).half()
+    with torch.no_grad():
+        module.weight.copy_(weight_d)
+    offsets_t = torch.as_tensor(np.asarray(offsets, dtype=np.int64))
+    coords3 = coords_d[:, 1:].contiguous()
+
+    def module_step():
+        vox = Voxels(coords3.view(-1, 3), feats_d, offsets=offsets_t)
+        with torch.no_grad():
+            return module(vox)
+
+    for _ in range(min(args.warmup, 20)):
+        module_step()
+    torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            mod_out = module_step()
+        torch.cuda.synchronize()
+        module_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    finally:
+        gc.enable()
+    module_max_diff = float((mod_out.feature_tensor.float() - out.float()).abs().max())
     if os.environ.get("WCN_BENCH_TRACE"):  # per-step device times, for looking into an odd average
         for i in range(args.steps):
             print(f"step {i}: map {starts[i].elapsed_time(mids[i]):.3f} ms, contraction call "
@@ -406,6 +528,7 @@ def main():
     cap = 2 * n
     map_bytes = 24 * n + 8 * cap + 16 * n + 8 * K * n + 8 * num_pairs
     achieved = conv_bytes / (conv_kernel_ms * 1e-3) / 1e9
+    traffic_bytes, traffic_note = measured_traffic()
 
     result = {
         "metric": METRIC,
@@ -426,23 +549,31 @@ def main():
                          "map from scratch and runs the contraction"),
             "num_voxels": n,
             "num_pairs": num_pairs,
+            "timing": "ms_per_step: wall clock over the K steps / K; the *_ms fields below: medians over the steps of device-event intervals",
+            "step_device_ms": step_device_ms,
             "kernel_map_build_ms": map_ms,
             "contraction_call_ms": conv_call_ms,
             "contraction_kernel_ms": conv_kernel_ms,
+            "module_forward_ms": module_ms,
+            "module_forward_note": ("SparseConv3d.forward on a Voxels object made anew per step (cold table and "
+                                    "map, cache lookups, output Voxels); wall clock / K; max |difference| to the "
+                                    f"direct path's output: {module_max_diff:.3g}"),
             "kernel_map_algorithmic_GBps": map_bytes / (map_ms * 1e-3) / 1e9,
             "kernel_map_frac_of_hbm_peak": map_bytes / (map_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "contraction_TFLOPs": conv_flops / (conv_kernel_ms * 1e-3) / 1e12,
             "contraction_frac_of_mfma_peak": conv_flops / (conv_kernel_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
         },
         "roofline": {
-            "kernel": "conv_fwd_ring<f16, 6, false, 0>",
+            "kernel": CONV_KERNEL if not os.environ.get("WCN_CONV_KERNEL") else "conv_fwd_ring<f16, 6, false, 0>",
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": CONV_FWD_TRAFFIC_BYTES,
+            "traffic": traffic_bytes,
+            "traffic_source": traffic_note,
             "algorithmic_bytes": conv_bytes,
+            "measured_peaks": measured_peaks(dev),
         },
     }
 
