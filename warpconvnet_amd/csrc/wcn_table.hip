@@ -88,74 +88,46 @@ __global__ void __launch_bounds__(1024) table_bbox(const int4* __restrict__ keys
   }
 }
 
-// Keys that follow each other in the input and fall into the same 4x4x4 block (the rule for voxels
-// in scan order: neighbours along the last axis) are inserted together: the lanes of such a run
-// combine their bits, the first lane of the run finds or claims the block's slot and adds the
-// combined bits with one atomic per half of the mask, and hands the slot to the others.
 __global__ void __launch_bounds__(256) table_insert(const int4* __restrict__ keys, int64_t n_keys,
                                                     WcnTableHeader* __restrict__ hdr,
                                                     WcnSlot* __restrict__ slots, uint32_t cap_mask,
                                                     int32_t* __restrict__ slot_of) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int lane = wcn_lane();
+  if (i >= n_keys) return;
   const WcnLayout L = wcn_make_layout(hdr);
-  if (!L.ok) {  // uniform
+  if (!L.ok) {
     if (i == 0) atomicOr(&hdr->status, WCN_DEV_RANGE);
-    if (i < n_keys) slot_of[i] = -1;
+    slot_of[i] = -1;
     return;
   }
-  const bool active = i < n_keys;  // the inactive lanes are the last ones of the last wave
-  unsigned long long key = 0ull, bits = 0ull;
-  if (active) {
-    const int4 c = keys[i];
-    uint32_t r[4];
-    wcn_relative(L, c.x, c.y, c.z, c.w, r);  // always inside: the box was built from these keys
-    key = wcn_block_key(L, r);
-    bits = 1ull << wcn_block_bit(r);
-  }
-  const unsigned long long prev = __shfl_up(key, 1, 64);
-  const bool head = active && (lane == 0 || prev != key);
-  const unsigned long long heads = __ballot(head);
-  const int n_active = __popcll(__ballot(active));
-  // the run this lane belongs to: [my_head, run_end)
-  const unsigned long long upto = heads & (lane == 63 ? ~0ull : ((2ull << lane) - 1ull));
-  const int my_head = 63 - __clzll((long long)upto);  // active lanes always have a head at or below them
-  const unsigned long long above = lane == 63 ? 0ull : (heads >> (lane + 1));
-  int run_end = above != 0ull ? lane + 1 + (__ffsll((long long)above) - 1) : 64;
-  run_end = run_end < n_active ? run_end : n_active;
-  // OR of the bits of lanes lane .. run_end - 1 (doubling): the head ends up with the whole run's
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const unsigned long long other = __shfl_down(bits, d, 64);
-    if (lane + d < run_end) bits |= other;
-  }
+  const int4 c = keys[i];
+  uint32_t r[4];
+  wcn_relative(L, c.x, c.y, c.z, c.w, r);  // always inside: the box was built from these keys
+  const unsigned long long key = wcn_block_key(L, r);
+  const uint32_t bit_index = wcn_block_bit(r);
+  const uint32_t bit = 1u << (bit_index & 31u);  // within the 32-bit half of the mask that holds it
+  uint32_t h = wcn_mix(key, cap_mask);
   int32_t placed = -1;
-  if (head) {
-    uint32_t h = wcn_mix(key, cap_mask);
-    for (int p = 0; p < WCN_MAX_PROBE; ++p) {
-      // cheap pre-read: most keys find their block already present
-      // (a stale EMPTY from the vector cache only costs the CAS below; a non-empty key is final)
-      unsigned long long seen = *reinterpret_cast<const volatile unsigned long long*>(&slots[h].key);
-      if (seen == WCN_EMPTY_KEY) {
-        seen = atomicCAS(&slots[h].key, WCN_EMPTY_KEY, key);
-        if (seen == WCN_EMPTY_KEY) seen = key;  // this thread claimed the slot
-      }
-      if (seen == key) {
-        // the results of the atomics are not used, so they are issued without waiting for a reply;
-        // repeated keys show up later as fewer set bits than keys
-        uint32_t* half = reinterpret_cast<uint32_t*>(&slots[h].mask);
-        const uint32_t lo = (uint32_t)bits, hi = (uint32_t)(bits >> 32);
-        if (lo) atomicOr(half, lo);
-        if (hi) atomicOr(half + 1, hi);
-        placed = (int32_t)h;
-        break;
-      }
-      h = (h + 1) & cap_mask;
+  for (int p = 0; p < WCN_MAX_PROBE; ++p) {
+    // cheap pre-read: most keys find their block already present
+    // (a stale EMPTY from the vector cache only costs the CAS below; a non-empty key is final)
+    unsigned long long seen = *reinterpret_cast<const volatile unsigned long long*>(&slots[h].key);
+    if (seen == WCN_EMPTY_KEY) {
+      seen = atomicCAS(&slots[h].key, WCN_EMPTY_KEY, key);
+      if (seen == WCN_EMPTY_KEY) seen = key;  // this thread claimed the slot
     }
-    if (placed < 0) atomicOr(&hdr->status, WCN_DEV_OVERFLOW);
+    if (seen == key) {
+      // the result of the atomic is not used, so it is issued without waiting for a reply;
+      // repeated keys show up later as fewer set bits than keys
+      uint32_t* half = reinterpret_cast<uint32_t*>(&slots[h].mask) + (bit_index >> 5);
+      atomicOr(half, bit);
+      placed = (int32_t)h;
+      break;
+    }
+    h = (h + 1) & cap_mask;
   }
-  placed = __shfl(placed, my_head < 0 ? 0 : my_head, 64);
-  if (active) slot_of[i] = placed;
+  if (placed < 0) atomicOr(&hdr->status, WCN_DEV_OVERFLOW);
+  slot_of[i] = placed;
 }
 
 // base of every occupied slot = running sum of block populations.  A 1024-thread workgroup owns
