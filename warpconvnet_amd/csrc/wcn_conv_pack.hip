@@ -542,19 +542,26 @@ int launch_instance(const ConvArgs& a, hipStream_t s) {
 #define WCN_PACK_NW 7
 #endif
 
+// Tile height: R rows for column groups of 64 channels, 2 R for 32 (same LDS).  Maps with fewer
+// such tiles than the GPU has CUs take tiles of half the height, so that more CUs have work.
+template <typename T, int NL, bool FULL>
+int launch_shaped(const ConvArgs& a, hipStream_t s) {
+  constexpr int R = WCN_PACK_R, NW = WCN_PACK_NW;
+  const bool wide_out = a.c_out > 32;
+  const int64_t ny = wide_out ? (a.c_out + 63) / 64 : 1;
+  const int64_t tiles = (a.num_out + (wide_out ? R : 2 * R) - 1) / (wide_out ? R : 2 * R) * ny;
+  const bool few = tiles < 224;
+  if (wide_out) return few ? launch_instance<T, R / 2, NW, 4, NL, FULL>(a, s) : launch_instance<T, R, NW, 4, NL, FULL>(a, s);
+  return few ? launch_instance<T, R, NW, 2, NL, FULL>(a, s) : launch_instance<T, 2 * R, NW, 2, NL, FULL>(a, s);
+}
+
 template <typename T>
 int launch_typed(const ConvArgs& a, hipStream_t s) {
-  constexpr int R = WCN_PACK_R, NW = WCN_PACK_NW;
   const uint32_t row_bytes = (uint32_t)a.c_in * (uint32_t)sizeof(T);
-  const bool wide_out = a.c_out > 32;
-  if (row_bytes == 128) return wide_out ? launch_instance<T, R, NW, 4, 2, true>(a, s)
-                                        : launch_instance<T, 2 * R, NW, 2, 2, true>(a, s);
-  if (row_bytes == 64) return wide_out ? launch_instance<T, R, NW, 4, 1, true>(a, s)
-                                       : launch_instance<T, 2 * R, NW, 2, 1, true>(a, s);
-  if (row_bytes > 64) return wide_out ? launch_instance<T, R, NW, 4, 2, false>(a, s)
-                                      : launch_instance<T, 2 * R, NW, 2, 2, false>(a, s);
-  return wide_out ? launch_instance<T, R, NW, 4, 1, false>(a, s)
-                  : launch_instance<T, 2 * R, NW, 2, 1, false>(a, s);
+  if (row_bytes == 128) return launch_shaped<T, 2, true>(a, s);
+  if (row_bytes == 64) return launch_shaped<T, 1, true>(a, s);
+  if (row_bytes > 64) return launch_shaped<T, 2, false>(a, s);
+  return launch_shaped<T, 1, false>(a, s);
 }
 
 }  // namespace
