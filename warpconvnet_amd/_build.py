@@ -34,7 +34,7 @@ def _run(cmd):
 # Sources whose kernels issue loads in inline assembly and wait for them by count: a register the
 # compiler spills (or otherwise moves) while such a load is still in flight would be overwritten
 # later by the landing data.  These files must compile without any scratch memory.
-NO_SCRATCH_SOURCES = ("wcn_conv_pack.hip",)
+NO_SCRATCH_SOURCES = ("wcn_conv_pack_f16.hip", "wcn_conv_pack_bf16.hip", "wcn_conv_pack_f32.hip")
 _REMARK = "-Rpass-analysis=kernel-resource-usage"
 
 
@@ -122,13 +122,15 @@ def build_library(verbose: bool = False) -> str:
         logs = list(pool.map(_run, cmds))
     for src, log in zip(sources, logs):
         _check_no_scratch(src, log)
-    for src in sources:
-        if os.path.basename(src) in NO_SCRATCH_SOURCES:
-            asm_path = os.path.join(objdir, os.path.basename(src)[:-4] + ".s")
-            _run([hipcc, *compile_flags, "-S", "--cuda-device-only", "-o", asm_path, src])
-            with open(asm_path) as f:
-                _check_loads_not_copied(src, f.read())
-            os.remove(asm_path)
+    checked = [src for src in sources if os.path.basename(src) in NO_SCRATCH_SOURCES]
+    asm_paths = [os.path.join(objdir, os.path.basename(src)[:-4] + ".s") for src in checked]
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(checked)))) as pool:
+        list(pool.map(_run, [[hipcc, *compile_flags, "-S", "--cuda-device-only", "-o", asm, src]
+                             for src, asm in zip(checked, asm_paths)]))
+    for src, asm in zip(checked, asm_paths):
+        with open(asm) as f:
+            _check_loads_not_copied(src, f.read())
+        os.remove(asm)
     logs = [_without_remarks(log) for log in logs]
     logs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", LIB_PATH, *objects]))
     if verbose:

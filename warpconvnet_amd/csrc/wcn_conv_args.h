@@ -26,7 +26,8 @@ struct ConvArgs {
 };
 
 
-// The pair-packed contraction (wcn_conv_pack.hip): whether it takes a problem, and its launch.
+// The pair-packed contraction (wcn_conv_pack*.hip): whether it takes a problem, and its launch.
+constexpr int WCN_PACK_MAX_BIAS = 1024;  // output channels (padded) whose bias fits the kernel's LDS copy
 bool wcn_conv_pack_takes(const ConvArgs& a, int dtype);
 int wcn_conv_pack_launch(const ConvArgs& a, int dtype, hipStream_t stream);
 
