@@ -68,7 +68,22 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, three, three, fake, 100, null, null, null) == -1
     assert L.wcn_kmap_fill(fake, 10, 1024, fake, 5, three, three, fake, -1, fake, fake, null) == -1
     assert L.wcn_stride_unique(fake, 10, bad, fake, 1024, fake, fake, null) == -1
+    one = (ctypes.c_int32 * 3)(1, 1, 1)
+    zero = (ctypes.c_int32 * 3)(0, 0, 0)
+    assert L.wcn_kmap_count_dilated(fake, 10, 1024, fake, 5, three, three, zero, one, fake, null) == -1  # dilation 0
+    assert L.wcn_kmap_count_dilated(fake, 10, 1024, fake, 5, bad, three, one, one, fake, null) == -1
+    assert L.wcn_kmap_count_dilated(fake, 10, 1024, fake, 5, three, three, one, one, null, null) == -1
     offs = (ctypes.c_int64 * 28)(*([0] * 28))
+    assert L.wcn_pairs_sort_workspace_bytes(1000, 27, 5000) >= 4 * 1000 + 4 * 5000
+    assert L.wcn_pairs_sort_workspace_bytes(1000, 0, 5000) == 0
+    assert L.wcn_pairs_sort_by_out(fake, fake, offs, 27, 10, fake, fake, null, fake, 1 << 20, null) == -1   # no group table
+    assert L.wcn_pairs_sort_by_out(fake, fake, None, 27, 10, fake, fake, fake, fake, 1 << 20, null) == -1
+    assert L.wcn_pairs_sort_by_out(fake, fake, offs, 27, 10, fake, fake, fake, fake, 16, null) == -6         # workspace too small
+    too_many = (ctypes.c_int64 * 201)(*([0] * 201))
+    assert L.wcn_sparse_conv_fwd_static(fake, 10, 64, 1, fake, 1, 200, 64, null, fake, fake, too_many, -1, 1,
+                                        null, fake, 10, null) == -1                                       # > 127 offsets
+    assert L.wcn_sparse_conv_fwd_static(fake, 10, 64, 1, fake, 1, 27, 64, null, fake, fake, offs, -1, 1,
+                                        null, fake, 10_000_000, null) == -6                               # beyond the 4 MiB array
 
     def conv(dtype=1, wdtype=1, ws_bytes=1 << 30, ascend=1, gs=null, offsets=offs):
         return L.wcn_sparse_conv_fwd(fake, 10, 64, dtype, fake, wdtype, 27, 64, null, fake, fake,
