@@ -100,24 +100,32 @@ struct PackMma<float> {
 // have landed" is a fixed count for s_waitcnt vmcnt (loads retire in order).  The compiler's own
 // bookkeeping merges the loop's many paths and ends up waiting for nearly everything in every step.
 // The waits name the registers they vouch for, so that no use can move ahead of them.
-__device__ __forceinline__ void load_dword(int32_t& dst, const int32_t* p) {
-  asm volatile("global_load_dword %0, %1, off" : "=&v"(dst) : "v"(p));
-}
 template <int NL>
 __device__ __forceinline__ void load_row(u32x4 (&dst)[NL], const char* p0, const char* p1) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst[0]) : "v"(p0));
   if (NL == 2) asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst[NL - 1]) : "v"(p1));
+}
+// The same loads with the address as a uniform base (a scalar register pair) plus an unsigned
+// 32-bit byte offset per lane: one vector instruction makes the offset, against three or four for
+// a 64-bit address per lane.
+__device__ __forceinline__ void load_dword_at(int32_t& dst, const int32_t* base, uint32_t off) {
+  asm volatile("global_load_dword %0, %1, %2" : "=&v"(dst) : "v"(off), "s"(base));
+}
+template <int NL>
+__device__ __forceinline__ void load_row_at(u32x4 (&dst)[NL], const char* base, uint32_t off) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(dst[0]) : "v"(off), "s"(base));
+  if (NL == 2) asm volatile("global_load_dwordx4 %0, %1, %2 offset:64" : "=&v"(dst[NL - 1]) : "v"(off), "s"(base));
 }
 template <int N>
 __device__ __forceinline__ void wait_loads(int32_t& a, int32_t& b) {
   asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
 }
 template <int N, int NL>
-__device__ __forceinline__ void wait_loads(u32x4 (&r)[NL], int32_t& b) {
+__device__ __forceinline__ void wait_rows(u32x4 (&r)[NL]) {
   if (NL == 2)
-    asm volatile("s_waitcnt vmcnt(%3)" : "+v"(r[0]), "+v"(r[NL - 1]), "+v"(b) : "n"(N));
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(r[0]), "+v"(r[NL - 1]) : "n"(N));
   else
-    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(r[0]), "+v"(b) : "n"(N));
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r[0]) : "n"(N));
 }
 
 // LDS traffic is ordered by lgkmcnt alone; a plain s_barrier (no wait for the loads in flight).
@@ -303,6 +311,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
       const int row = cb * 16 + c;
       w_opnd[cb][l] = row * WPARTS + ((l * 4 + g) ^ ((row >> 1) & (WPARTS - 1)));
     }
+  const uint32_t c4 = (uint32_t)c * 4u;
   uint32_t col_off[NL];
   bool col_ok[NL];
 #pragma unroll
@@ -377,10 +386,10 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
     const bool use = n > 0 && !(d.w0 & F_IDENT);
     const int32_t* pin = use ? a.in_maps + d.p0 : zidx;
     const int32_t* pout = use ? a.out_maps + d.p0 : zidx;
-    const int last = use ? n - 1 : 0;  // slots past the block's pairs repeat its last pair
-    const int slot = c < last ? c : last;
-    load_dword(in_raw[u], pin + slot);
-    load_dword(out_raw[u], pout + slot);
+    const uint32_t last4 = use ? (uint32_t)(n - 1) * 4u : 0u;  // slots past the block's pairs repeat its last pair
+    const uint32_t slot4 = c4 < last4 ? c4 : last4;
+    load_dword_at(in_raw[u], pin, slot4);
+    load_dword_at(out_raw[u], pout, slot4);
   };
   auto issue_gather = [&](int u) {
     const Step d = ring[u];
@@ -392,6 +401,10 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
     if ((uint32_t)in >= (uint32_t)a.num_in) {  // malformed map: the pair contributes nothing
       in = 0;
       out_raw[u] = -1;
+    }
+    if (FULL) {  // rows of NL * 64 bytes, all of X within 4 GiB of its start (the launch checks)
+      load_row_at<NL>(A[u], xbase, ((uint32_t)in << (NL == 2 ? 7 : 6)) + col_off[0]);
+      return;
     }
     const char* p = xbase + (uint64_t)(uint32_t)in * row_bytes;
     const char* q[2];
@@ -451,29 +464,41 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
             for (int l = 0; l < NL; ++l) Wop[cb][l] = wbuf[(phase & 1) * WTILE + w_opnd[cb][l]];
         }
       }
-      // The step's rows were requested DG steps ago: that step's two pair-list loads and DG - 1
-      // whole steps of loads came after them.  Waited for in every step, also the empty ones: a
-      // register is free for other values only once the load into it has landed.
-      wait_loads<2 + (DG - 1) * (NL + 2), NL>(A[u], out_raw[u]);
+      // The sums this block adds to (the pair-list entries landed DG steps ago, when the rows were
+      // requested): read now and handed to the MFMAs as their starting value, so that the read's
+      // latency and that of the weight operands pass while the next steps are prepared below.
+      const int orow = (d.w0 & F_IDENT) ? d.p0 + c : out_raw[u] - d.m0;
+      const bool mine = c < n && (uint32_t)orow < (uint32_t)tile_rows;
+      f32x4* sums[NB];
+      f32x4 P[NB];
+      {
+        const int row = mine ? orow : 0;  // lanes without a pair read along (and write nothing)
+        float* const rowp = acc + row * RS;
+        const int sw = row & 7;  // 16-byte granule cb * 4 + g of the row is stored at granule ^ (row % 8)
+#pragma unroll
+        for (int cb = 0; cb < NB; ++cb) sums[cb] = reinterpret_cast<f32x4*>(rowp + (((cb * 4 + g) ^ sw) << 2));
+      }
+      if (n > 0) {
+#pragma unroll
+        for (int cb = 0; cb < NB; ++cb) P[cb] = *sums[cb];
+      }
+      const bool tile_end = (d.w0 & F_TILE_END) != 0;
+      issue_gather((u + DG) % U);
+      issue_idx(u);  // from here on ring[u], in_raw[u] and out_raw[u] belong to a later step
+      // The step's rows were requested DG steps ago: that step's two pair-list loads, DG - 1 whole
+      // steps of loads and this step's own came after them.  Waited for in every step, also the
+      // empty ones: a register is free for other values only once the load into it has landed.
+      wait_rows<2 + DG * (NL + 2), NL>(A[u]);
       if (n > 0) {
         // products: lane (c, g) gets channels cb * 16 + 4 g .. + 3 of pair c
-        f32x4 P[NB];
 #pragma unroll
-        for (int cb = 0; cb < NB; ++cb)
-          P[cb] = PackMma<T>::template run<NL>(Wop[cb], A[u], (f32x4){0.f, 0.f, 0.f, 0.f});
-        const int orow = (d.w0 & F_IDENT) ? d.p0 + c : out_raw[u] - d.m0;
-        if (c < n && (uint32_t)orow < (uint32_t)tile_rows) {
-          // 16-byte granule cb * 4 + g of the row, stored at granule ^ (row % 8)
-          float* const rowp = acc + orow * RS;
-          const int sw = orow & 7;
+        for (int cb = 0; cb < NB; ++cb) P[cb] = PackMma<T>::template run<NL>(Wop[cb], A[u], P[cb]);
+        if (mine) {
 #pragma unroll
-          for (int cb = 0; cb < NB; ++cb) {
-            f32x4* const q = reinterpret_cast<f32x4*>(rowp + (((cb * 4 + g) ^ sw) << 2));
-            *q = *q + P[cb];
-          }
+          for (int cb = 0; cb < NB; ++cb) *sums[cb] = P[cb];
         }
       }
-      if (d.w0 & F_TILE_END) {
+      if (tile_end) {
         // ---- the tile is complete: bias, one rounding, whole 16-byte stores; sums back to zero ----
         lds_barrier();
         T* __restrict__ out = (T*)a.out;
@@ -522,8 +547,6 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
         // instead of turning every later wait of the ring into a full one.
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
       }
-      issue_gather((u + DG) % U);
-      issue_idx(u);
     }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the ring's last loads land before the registers are given up
@@ -590,8 +613,10 @@ int launch_sized(const ConvArgs& a, hipStream_t s) {
 template <typename T>
 int launch_typed(const ConvArgs& a, hipStream_t s) {
   const uint32_t row_bytes = (uint32_t)a.c_in * (uint32_t)sizeof(T);
-  if (row_bytes == 128) return launch_sized<T, 2, true>(a, s);
-  if (row_bytes == 64) return launch_sized<T, 1, true>(a, s);
+  // the instances for whole rows address X with 32-bit byte offsets
+  const bool near = (uint64_t)a.num_in * row_bytes < (1ull << 32);
+  if (row_bytes == 128 && near) return launch_sized<T, 2, true>(a, s);
+  if (row_bytes == 64 && near) return launch_sized<T, 1, true>(a, s);
   if (row_bytes > 64) return launch_sized<T, 2, false>(a, s);
   return launch_sized<T, 1, false>(a, s);
 }
