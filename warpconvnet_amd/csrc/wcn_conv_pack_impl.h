@@ -41,8 +41,8 @@ namespace {
 using namespace wcn_mma;
 
 constexpr int PB = 16;  // pairs per block (rows of one MFMA)
-constexpr int U = 8;    // steps in the ring (unroll factor of the step loop)
-constexpr int DG = 4;   // gathered rows are requested DG steps before they are multiplied
+constexpr int U = 4;    // steps in the ring (unroll factor of the step loop)
+constexpr int DG = 2;   // gathered rows are requested DG steps before they are multiplied
 
 // Step descriptor (wave-uniform).
 constexpr uint32_t F_PHASE = 1u << 16;     // first step of a phase
@@ -589,7 +589,7 @@ int launch_instance(const ConvArgs& a, hipStream_t s) {
 #define WCN_PACK_R 512
 #endif
 #ifndef WCN_PACK_NW
-#define WCN_PACK_NW 7
+#define WCN_PACK_NW 11  // 12 waves: three per SIMD, 168 registers each; a 512-row tile's run of ~160 pairs is one step
 #endif
 
 // Tile height: R rows for column groups of 64 channels, 2 R for 32 (same LDS).  Maps with fewer
