@@ -45,12 +45,12 @@ constexpr int U = 4;    // steps in the ring (unroll factor of the step loop)
 constexpr int DG = 2;   // gathered rows are requested DG steps before they are multiplied
 
 // Step descriptor (wave-uniform).
-constexpr uint32_t F_PHASE = 1u << 16;     // first step of a phase
+constexpr uint32_t F_NEW_TILE = 1u << 16;  // this wave's first step of a tile
 constexpr uint32_t F_TILE_END = 2u << 16;  // last step of a tile
 constexpr uint32_t F_END = 4u << 16;       // no work left: leave the loop
 constexpr uint32_t F_IDENT = 8u << 16;     // identity offset: pair i of the block is (m0 + p0 + i, p0 + i)
 struct Step {
-  uint32_t w0;  // pairs of this wave's block (0..16) | k << 8 | flags
+  uint32_t w0;  // pairs of this wave's block (0..16) | k << 8 | flags | phase barriers to pass before the step << 24
   int32_t p0;   // first pair of the block (index into the pair lists; tile row for F_IDENT)
   int32_t m0;   // first output row of the step's tile
 };
@@ -321,28 +321,32 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
   }
 
   // ---- the step generator (runs U steps ahead of the multiplications) -----------------------------
+  // A wave's steps are the blocks it has to multiply, plus one step (empty if need be) in a tile's
+  // last phase, where the tile is written out by all waves together.  Phases in which the wave has
+  // no block cost it a barrier each and nothing else: the step that follows says how many.
   // lane k % 64 holds the run of offset k in the generator's tile (offsets below 64 in [0], the
-  // others in [1]): pairs, first pair, steps
-  int plan_cnt[2] = {0, 0}, plan_start[2] = {0, 0}, plan_steps[2] = {1, 1};
+  // others in [1]): pairs, first pair, this wave's steps
+  int plan_cnt[2] = {0, 0}, plan_start[2] = {0, 0}, plan_mine[2] = {0, 0};
+  unsigned long long plan_work[2] = {0ull, 0ull};  // the offsets in which this wave has a step
   int gen_iter = -1;                 // tiles this generator has entered, minus one
-  int gen_k = K - 1, gen_sip = 0, gen_steps = 1;  // "just past the last step of a tile": the first advance enters tile 0
+  int gen_k = K - 1, gen_sip = 0, gen_mine = 0;  // "past the last step of a tile": the first advance enters tile 0
   int gen_cnt = 0, gen_start = 0, gen_ident = 0;
   int64_t gen_m0 = 0;
   bool gen_live = true;              // false once the tiles are used up
   auto next_step = [&]() -> Step {
     Step d = {F_END, 0, 0};
     if (!gen_live) return d;
-    uint32_t flags = 0;
-    if (++gen_sip >= gen_steps) {  // next phase
+    uint32_t flags = 0, bars = 0;
+    if (gen_sip >= gen_mine) {     // this wave's steps of the phase are used up
       gen_sip = 0;
-      flags |= F_PHASE;
-      if (++gen_k >= K) {          // next tile
-        gen_k = 0;
+      if (gen_k == K - 1) {        // next tile
+        gen_k = -1;
         ++gen_iter;
         if (tile_of(gen_iter) >= num_vtiles) {
           gen_live = false;
           return d;
         }
+        flags |= F_NEW_TILE;
         gen_m0 = (int64_t)(tile_of(gen_iter) / ny) * R;
         const int32_t* slot = s_plan + (gen_iter % PLAN_SLOTS) * 256;
 #pragma unroll
@@ -350,26 +354,42 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
           plan_cnt[h] = slot[64 * h + lane];
           plan_start[h] = slot[128 + 64 * h + lane];
           const int nb = (plan_cnt[h] + PB - 1) / PB;
-          plan_steps[h] = nb > 0 ? (nb + NW - 1) / NW : 1;
+          int mine = nb > wave ? (nb - wave + NW - 1) / NW : 0;
+          if (64 * h + lane == K - 1 && mine == 0) mine = 1;  // the step that ends the tile
+          plan_mine[h] = mine;
+          plan_work[h] = __ballot(mine > 0);
         }
       }
+      // the next offset with a step of this wave (the last offset always has one)
+      const int from = gen_k + 1;
+      int nk;
+      const unsigned long long w0m = from < 64 ? plan_work[0] & (~0ull << from) : 0ull;
+      if (!K2 || w0m != 0ull) {
+        nk = (int)__builtin_ctzll(w0m);
+      } else {
+        const int f1 = from > 64 ? from - 64 : 0;
+        nk = 64 + (int)__builtin_ctzll(plan_work[1] & (~0ull << f1));
+      }
+      bars = (uint32_t)(nk - gen_k);
+      gen_k = nk;
       if (!K2 || gen_k < 64) {
         gen_cnt = __builtin_amdgcn_readlane(plan_cnt[0], gen_k);
         gen_start = __builtin_amdgcn_readlane(plan_start[0], gen_k);
-        gen_steps = __builtin_amdgcn_readlane(plan_steps[0], gen_k);
+        gen_mine = __builtin_amdgcn_readlane(plan_mine[0], gen_k);
       } else {
         gen_cnt = __builtin_amdgcn_readlane(plan_cnt[1], gen_k - 64);
         gen_start = __builtin_amdgcn_readlane(plan_start[1], gen_k - 64);
-        gen_steps = __builtin_amdgcn_readlane(plan_steps[1], gen_k - 64);
+        gen_mine = __builtin_amdgcn_readlane(plan_mine[1], gen_k - 64);
       }
       gen_ident = gen_k == a.identity ? 1 : 0;
     }
     const int j = gen_sip * NW + wave;  // this wave's block of the run
     int n = gen_cnt - j * PB;
     n = n < 0 ? 0 : (n > PB ? PB : n);
-    if (gen_k == K - 1 && gen_sip == gen_steps - 1) flags |= F_TILE_END;
+    if (gen_k == K - 1 && gen_sip == gen_mine - 1) flags |= F_TILE_END;
     if (gen_ident) flags |= F_IDENT;
-    d.w0 = (uint32_t)n | ((uint32_t)gen_k << 8) | flags;
+    ++gen_sip;
+    d.w0 = (uint32_t)n | ((uint32_t)gen_k << 8) | flags | (bars << 24);
     d.p0 = gen_start + j * PB;
     d.m0 = (int32_t)gen_m0;
     return d;
@@ -445,11 +465,13 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
         break;
       }
       const int n = (int)(d.w0 & 0xFFu);
-      if (d.w0 & F_PHASE) {
-        // everybody is done with the previous phase: its additions and its reads of the weight tile
-        lds_barrier();
-        ++phase;
-        if (((d.w0 >> 8) & 0xFFu) == 0u) {  // a new tile
+      const int bars = (int)(d.w0 >> 24);
+      if (bars > 0) {
+        // a barrier per phase: everybody is done with the phase before, its additions and its reads
+        // of the weight tile
+        for (int i = 0; i < bars; ++i) lds_barrier();
+        phase += bars;
+        if (d.w0 & F_NEW_TILE) {
           ++cmp_iter;
           const int vt = tile_of(cmp_iter);
           m0 = (int64_t)(vt / ny) * R;
