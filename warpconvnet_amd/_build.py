@@ -73,35 +73,85 @@ def _vgprs_in(text):
     return regs
 
 
-def _check_loads_not_copied(src, asm_text):
-    """The destination of a written-out load must not be read or moved before a vmcnt wait: a
-    copy the compiler inserts between the load and its wait (at a control-flow merge, say) would
-    carry the register's old contents.  Checked on the generated code, in program-text order,
-    over the copy-like instructions of the 400 lines after each such load."""
-    lines = asm_text.split("\n")
+def _loads_in_flight_touched(name, lines):
+    """One kernel's listing: every use of a written-out load's destination before a wait that covers it."""
     code = [l.split(";")[0].rstrip() for l in lines]
-    in_asm, bad = False, []
+    in_asm, asm_load = False, {}
     for i, raw in enumerate(lines):
         if "#ASMSTART" in raw:
             in_asm = True
-            continue
-        if "#ASMEND" in raw:
+        elif "#ASMEND" in raw:
             in_asm = False
-            continue
-        m = re.match(r"\s*global_load_dword(x2|x4)?\s+(\S+),", code[i])
-        if not (in_asm and m):
-            continue
-        dst = _vgprs_in(m.group(2))
-        for j in range(i + 1, min(len(code), i + 400)):
+        else:
+            m = re.match(r"\s*global_load_dword(x2|x4)?\s+(\S+),", code[i])
+            if in_asm and m:
+                asm_load[i] = _vgprs_in(m.group(2))
+    if not asm_load:
+        return []
+    first, last = min(asm_load), max(asm_load)
+    labels = {}
+    for i, c in enumerate(code):
+        m = re.match(r"^(\.LBB\d+_\d+):", c)
+        if m:
+            labels[m.group(1)] = i
+    # the loop around the loads: the last backward branch that spans all of them
+    head, back = None, None
+    for i, c in enumerate(code):
+        m = re.match(r"\s*s_c?branch\w*\s+(\.LBB\d+_\d+)", c)
+        if m and i > last and labels.get(m.group(1), 1 << 30) < first and (back is None or i > back):
+            head, back = labels[m.group(1)], i
+    # blocks that only leave the loop (label ... unconditional branch beyond the back edge) are not walked
+    skip, starts = set(), sorted(labels.values())
+    for n, start in enumerate(starts):
+        end = starts[n + 1] if n + 1 < len(starts) else len(code)
+        body = [k for k in range(start + 1, end) if code[k].strip()]
+        m = re.match(r"\s*s_branch\s+(\.LBB\d+_\d+)", code[body[-1]]) if body else None
+        if m and back is not None and labels.get(m.group(1), -1) > back:
+            skip.update(range(start, end))
+    bad = []
+    for i, dst in asm_load.items():
+        if back is not None and head <= i <= back:
+            order = list(range(i + 1, back + 1)) + list(range(head, i))  # once around the loop
+        else:
+            order = list(range(i + 1, len(code)))
+        issued = 0  # written-out loads issued after this one (they are issued on every path)
+        for j in order:
             st = code[j].strip()
-            if "s_endpgm" in st or ("s_waitcnt" in st and "vmcnt" in st):
+            if not st or j in skip or st.startswith((".", "#")):
+                continue
+            if j in asm_load:
+                if asm_load[j] & dst:
+                    break
+                issued += 1
+                continue
+            if "s_endpgm" in st:
                 break
+            m = re.search(r"s_waitcnt.*vmcnt\((\d+)\)", st)
+            if m:  # loads retire in order: all but the last N have landed (vmcnt(0) sits on side paths only)
+                if 1 <= int(m.group(1)) <= issued:
+                    break
+                continue
             ops = st.split(None, 1)
-            if len(ops) > 1 and re.match(r"v_(mov|cndmask|accvgpr|perm|swap)", st) and _vgprs_in(ops[1]) & dst:
-                bad.append(f"line {i + 1}: {code[i].strip()}  ->  line {j + 1}: {st}")
+            if len(ops) > 1 and _vgprs_in(ops[1]) & dst:
+                bad.append(f"{name}: line {i + 1}: {code[i].strip()}  ->  line {j + 1}: {st}")
                 break
+    return bad
+
+
+def _check_loads_not_copied(src, asm_text):
+    """The destination of a written-out load must not be read, moved or overwritten before a vmcnt
+    wait that covers the load: a copy the compiler inserts between the load and its wait (at a
+    control-flow merge or at the loop's back edge, say) would carry the register's old contents.
+    Checked on the generated code of every kernel, walking the program text from each such load
+    once around the loop that holds it, counting the written-out loads issued since."""
+    lines = asm_text.split("\n")
+    starts = [(i, m.group(1)) for i, l in enumerate(lines) for m in [re.match(r"^(_Z\w+):", l)] if m]
+    bad = []
+    for n, (begin, name) in enumerate(starts):
+        end = starts[n + 1][0] if n + 1 < len(starts) else len(lines)
+        bad += _loads_in_flight_touched(name, lines[begin:end])
     if bad:
-        raise RuntimeError(f"{os.path.basename(src)}: the compiler moves registers that loads are still in flight "
+        raise RuntimeError(f"{os.path.basename(src)}: the compiler touches registers that loads are still in flight "
                            "into:\n  " + "\n  ".join(bad[:10]))
 
 
