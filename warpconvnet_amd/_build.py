@@ -74,67 +74,74 @@ def _vgprs_in(text):
 
 
 def _loads_in_flight_touched(name, lines):
-    """One kernel's listing: every use of a written-out load's destination before a wait that covers it."""
-    code = [l.split(";")[0].rstrip() for l in lines]
-    in_asm, asm_load = False, {}
+    """One kernel's listing: every use of a written-out load's destination that some path reaches
+    before a wait that covers the load."""
+    code = [l.split(";")[0].strip() for l in lines]
+    in_asm, asm_load, labels = False, {}, {}
     for i, raw in enumerate(lines):
         if "#ASMSTART" in raw:
             in_asm = True
         elif "#ASMEND" in raw:
             in_asm = False
         else:
-            m = re.match(r"\s*global_load_dword(x2|x4)?\s+(\S+),", code[i])
+            m = re.match(r"global_load_dword(x2|x4)?\s+(\S+),", code[i])
             if in_asm and m:
                 asm_load[i] = _vgprs_in(m.group(2))
+            m = re.match(r"(\.LBB\d+_\d+):", code[i])
+            if m:
+                labels[m.group(1)] = i
     if not asm_load:
         return []
-    first, last = min(asm_load), max(asm_load)
-    labels = {}
-    for i, c in enumerate(code):
-        m = re.match(r"^(\.LBB\d+_\d+):", c)
+    n = len(code)
+    load_lines, last_load = sorted(asm_load), max(asm_load)
+
+    def successors(i):
+        st = code[i]
+        m = re.match(r"s_(c?)branch\w*\s+(\.LBB\d+_\d+)", st)
         if m:
-            labels[m.group(1)] = i
-    # the loop around the loads: the last backward branch that spans all of them
-    head, back = None, None
-    for i, c in enumerate(code):
-        m = re.match(r"\s*s_c?branch\w*\s+(\.LBB\d+_\d+)", c)
-        if m and i > last and labels.get(m.group(1), 1 << 30) < first and (back is None or i > back):
-            head, back = labels[m.group(1)], i
-    # blocks that only leave the loop (label ... unconditional branch beyond the back edge) are not walked
-    skip, starts = set(), sorted(labels.values())
-    for n, start in enumerate(starts):
-        end = starts[n + 1] if n + 1 < len(starts) else len(code)
-        body = [k for k in range(start + 1, end) if code[k].strip()]
-        m = re.match(r"\s*s_branch\s+(\.LBB\d+_\d+)", code[body[-1]]) if body else None
-        if m and back is not None and labels.get(m.group(1), -1) > back:
-            skip.update(range(start, end))
+            target = labels.get(m.group(2))
+            nxt = [target] if target is not None else []
+            # Every step issues its loads on every path, so a jump forward over some of them to a
+            # place that is still among the steps is either the way out of the loop spelled as a
+            # chain of tests or a path that cannot be taken: not walked.
+            if target is not None and i < target <= last_load and any(i < l < target for l in load_lines):
+                nxt = []
+            # likewise a jump from among the steps back to before the first of them: the loop is left
+            # (its condition is tested up there), not entered again
+            if target is not None and target < load_lines[0] and i < last_load:
+                nxt = []
+            return nxt + ([i + 1] if m.group(1) and i + 1 < n else [])
+        if st.startswith("s_endpgm"):
+            return []
+        return [i + 1] if i + 1 < n else []
+
     bad = []
-    for i, dst in asm_load.items():
-        if back is not None and head <= i <= back:
-            order = list(range(i + 1, back + 1)) + list(range(head, i))  # once around the loop
-        else:
-            order = list(range(i + 1, len(code)))
-        issued = 0  # written-out loads issued after this one (they are issued on every path)
-        for j in order:
-            st = code[j].strip()
-            if not st or j in skip or st.startswith((".", "#")):
+    for start, dst in asm_load.items():
+        # states: (instruction, written-out loads issued since `start`); they are issued on every path
+        seen, todo, hit = set(), [(s, 0) for s in successors(start)], None
+        while todo and hit is None:
+            i, issued = todo.pop()
+            if (i, issued) in seen:
                 continue
-            if j in asm_load:
-                if asm_load[j] & dst:
-                    break
-                issued += 1
-                continue
-            if "s_endpgm" in st:
-                break
-            m = re.search(r"s_waitcnt.*vmcnt\((\d+)\)", st)
-            if m:  # loads retire in order: all but the last N have landed (vmcnt(0) sits on side paths only)
-                if 1 <= int(m.group(1)) <= issued:
-                    break
-                continue
-            ops = st.split(None, 1)
-            if len(ops) > 1 and _vgprs_in(ops[1]) & dst:
-                bad.append(f"{name}: line {i + 1}: {code[i].strip()}  ->  line {j + 1}: {st}")
-                break
+            seen.add((i, issued))
+            st = code[i]
+            if i in asm_load:
+                if asm_load[i] & dst:
+                    continue  # the register takes its next load: this path is done
+                issued = min(issued + 1, 63)
+            elif st and not st.startswith((".", "#")):
+                m = re.search(r"s_waitcnt.*vmcnt\((\d+)\)", st)
+                if m:  # loads retire in order: all but the last N have landed
+                    if int(m.group(1)) <= issued:
+                        continue
+                else:
+                    ops = st.split(None, 1)
+                    if len(ops) > 1 and _vgprs_in(ops[1]) & dst:
+                        hit = f"{name}: line {start + 1}: {code[start]}  ->  line {i + 1}: {st}"
+                        break
+            todo.extend((s, issued) for s in successors(i))
+        if hit:
+            bad.append(hit)
     return bad
 
 
@@ -142,8 +149,8 @@ def _check_loads_not_copied(src, asm_text):
     """The destination of a written-out load must not be read, moved or overwritten before a vmcnt
     wait that covers the load: a copy the compiler inserts between the load and its wait (at a
     control-flow merge or at the loop's back edge, say) would carry the register's old contents.
-    Checked on the generated code of every kernel, walking the program text from each such load
-    once around the loop that holds it, counting the written-out loads issued since."""
+    Checked on the generated code of every kernel: from each such load along every path of the
+    control flow, counting the written-out loads issued since, up to a wait that covers it."""
     lines = asm_text.split("\n")
     starts = [(i, m.group(1)) for i, l in enumerate(lines) for m in [re.match(r"^(_Z\w+):", l)] if m]
     bad = []

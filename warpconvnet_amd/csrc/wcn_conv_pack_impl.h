@@ -50,7 +50,7 @@ constexpr uint32_t F_TILE_END = 2u << 16;  // last step of a tile
 constexpr uint32_t F_END = 4u << 16;       // no work left: leave the loop
 constexpr uint32_t F_IDENT = 8u << 16;     // identity offset: pair i of the block is (m0 + p0 + i, p0 + i)
 struct Step {
-  uint32_t w0;  // pairs of this wave's block (0..16) | k << 8 | flags | phase barriers to pass before the step << 24
+  uint32_t w0;  // pairs of this wave's block (0..16) | k << 8 | flags | slice << 20 | phase barriers to pass before the step << 24
   int32_t p0;   // first pair of the block (index into the pair lists; tile row for F_IDENT)
   int32_t m0;   // first output row of the step's tile
 };
@@ -188,8 +188,14 @@ __device__ __forceinline__ void runs_finish(const ConvArgs& a, int vt, int num_v
 // multiplying waves' load stream (whose waits are counts of loads still in flight, and loads retire
 // in order: one slow or oddly timed load in that stream stalls the ring): it brings W[k]^T of the
 // coming phases into LDS and publishes the runs of the coming tiles there.
-template <typename T, int R, int NW, int NB, int NL, bool FULL, bool K2>
+//
+// WIDE: feature rows of several 128-byte slices (up to four).  A phase is then one slice of one
+// offset -- K * NS phases per tile, the weight tile of a phase is the slice's 64 x 64 part of W[k]^T,
+// the gathered rows are the slice's 128 bytes -- and everything else stays as it is: the sums stay
+// in LDS across the slices.
+template <typename T, int R, int NW, int NB, int NL, bool FULL, bool K2, bool WIDE>
 __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int num_vtiles, int ny) {
+  static_assert(!WIDE || (NL == 2 && !K2), "slices are 128 bytes; the barrier count of a step has 8 bits");
   constexpr int KH = K2 ? 2 : 1;  // offsets a lane looks after: lane (and lane + 64 for maps of more than 64 offsets)
   extern __shared__ __attribute__((aligned(16))) float smem[];
   constexpr int THREADS = NW * 64;           // multiplying threads
@@ -206,6 +212,8 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int K = a.K;
+  const int NS = WIDE ? (int)((size_t)a.c_in_pad * sizeof(T) / (NL * 64)) : 1;  // slices of a row
+  const int KP = K * NS;                                                       // phases of a tile
   auto tile_of = [&](int iter) -> int { return (int)blockIdx.x + iter * (int)gridDim.x; };
 
   if (wave == NW) {
@@ -221,10 +229,10 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
       w_dst[j] = row * WPARTS + (part ^ ((row >> 1) & (WPARTS - 1)));
     }
     auto w_load = [&](int i, u32x4 (&regs)[WPL]) {  // the tile of phase i (counted over all tiles)
-      const int it = i / K, k = i - it * K;
+      const int it = i / KP, q = i - it * KP, k = WIDE ? q / NS : q, sl = WIDE ? q - k * NS : 0;
       const int vt = tile_of(it);
       const int n0 = vt < num_vtiles ? (vt % ny) * RS : 0;
-      const char* p = (const char*)a.Wt + (size_t)k * w_tile_bytes + (size_t)n0 * w_row_bytes;
+      const char* p = (const char*)a.Wt + (size_t)k * w_tile_bytes + (size_t)n0 * w_row_bytes + (size_t)sl * (NL * 64);
 #pragma unroll
       for (int j = 0; j < WPL; ++j) regs[j] = *reinterpret_cast<const u32x4*>(p + w_src[j]);
     };
@@ -266,8 +274,8 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
     lds_barrier();  // start: plans, bias and the first weight tile are published
     int num_iters = 0;
     while (tile_of(num_iters) < num_vtiles) ++num_iters;
-    const int num_phases = num_iters * K;
-    int k = 0, iter = 0;
+    const int num_phases = num_iters * KP;
+    int k = 0, iter = 0;  // k: the phase inside the tile
     for (int i0 = 0; i0 < num_phases; i0 += LW) {
 #pragma unroll
       for (int j = 0; j < LW; ++j) {
@@ -275,14 +283,14 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
         if (i >= num_phases) break;
         lds_barrier();  // phase i begins: the buffer of phase i - 1 is free
         // the tile of phase i + 1 (requested LW phases ago) goes to LDS, its registers take phase i + 1 + LW
-        if (k == K - 1 && K > 1) plan_store(iter + PLAN_AHEAD, pending);
+        if (k == KP - 1 && KP > 1) plan_store(iter + PLAN_AHEAD, pending);
         w_store((i + 1) & 1, wr[(j + 1) % LW]);
         w_load(i + 1 + LW, wr[(j + 1) % LW]);
         if (k == 0) {
           pending = plan_request(iter + PLAN_AHEAD);
-          if (K == 1) plan_store(iter + PLAN_AHEAD, pending);
+          if (KP == 1) plan_store(iter + PLAN_AHEAD, pending);
         }
-        if (++k == K) {
+        if (++k == KP) {
           k = 0;
           ++iter;
           lds_barrier();  // the tile's sums are complete (the multiplying waves write them out)
@@ -329,7 +337,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
   int plan_cnt[2] = {0, 0}, plan_start[2] = {0, 0}, plan_mine[2] = {0, 0};
   unsigned long long plan_work[2] = {0ull, 0ull};  // the offsets in which this wave has a step
   int gen_iter = -1;                 // tiles this generator has entered, minus one
-  int gen_k = K - 1, gen_sip = 0, gen_mine = 0;  // "past the last step of a tile": the first advance enters tile 0
+  int gen_k = K - 1, gen_sl = NS - 1, gen_sip = 0, gen_mine = 0;  // "past the last step of a tile": the first advance enters tile 0
   int gen_cnt = 0, gen_start = 0, gen_ident = 0;
   int64_t gen_m0 = 0;
   bool gen_live = true;              // false once the tiles are used up
@@ -337,8 +345,13 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
     Step d = {F_END, 0, 0};
     if (!gen_live) return d;
     uint32_t flags = 0, bars = 0;
-    if (gen_sip >= gen_mine) {     // this wave's steps of the phase are used up
+    if (gen_sip >= gen_mine && WIDE && gen_sl + 1 < NS) {  // the same blocks, next slice
       gen_sip = 0;
+      ++gen_sl;
+      bars = 1;
+    } else if (gen_sip >= gen_mine) {  // this wave's steps of the offset are used up
+      gen_sip = 0;
+      gen_sl = 0;
       if (gen_k == K - 1) {        // next tile
         gen_k = -1;
         ++gen_iter;
@@ -370,7 +383,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
         const int f1 = from > 64 ? from - 64 : 0;
         nk = 64 + (int)__builtin_ctzll(plan_work[1] & (~0ull << f1));
       }
-      bars = (uint32_t)(nk - gen_k);
+      bars = (uint32_t)((nk - gen_k - 1) * NS + 1);  // from the last slice of gen_k to the first of nk
       gen_k = nk;
       if (!K2 || gen_k < 64) {
         gen_cnt = __builtin_amdgcn_readlane(plan_cnt[0], gen_k);
@@ -386,10 +399,10 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
     const int j = gen_sip * NW + wave;  // this wave's block of the run
     int n = gen_cnt - j * PB;
     n = n < 0 ? 0 : (n > PB ? PB : n);
-    if (gen_k == K - 1 && gen_sip == gen_mine - 1) flags |= F_TILE_END;
+    if (gen_k == K - 1 && gen_sl == NS - 1 && gen_sip == gen_mine - 1) flags |= F_TILE_END;
     if (gen_ident) flags |= F_IDENT;
     ++gen_sip;
-    d.w0 = (uint32_t)n | ((uint32_t)gen_k << 8) | flags | (bars << 24);
+    d.w0 = (uint32_t)n | ((uint32_t)gen_k << 8) | flags | ((uint32_t)gen_sl << 20) | (bars << 24);
     d.p0 = gen_start + j * PB;
     d.m0 = (int32_t)gen_m0;
     return d;
@@ -422,16 +435,21 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
       in = 0;
       out_raw[u] = -1;
     }
-    if (FULL) {  // rows of NL * 64 bytes, all of X within 4 GiB of its start (the launch checks)
-      load_row_at<NL>(A[u], xbase, ((uint32_t)in << (NL == 2 ? 7 : 6)) + col_off[0]);
+    const uint32_t sl_off = WIDE ? ((d.w0 >> 20) & 3u) * (uint32_t)(NL * 64) : 0u;  // the step's slice of the row
+    if (FULL) {  // whole slices; all of X within 4 GiB of its start, fewer than 2^24 rows (the launch checks)
+      if (WIDE)
+        load_row_at<NL>(A[u], xbase, __umul24((uint32_t)in, row_bytes) + (sl_off + col_off[0]));
+      else
+        load_row_at<NL>(A[u], xbase, ((uint32_t)in << (NL == 2 ? 7 : 6)) + col_off[0]);
       return;
     }
-    const char* p = xbase + (uint64_t)(uint32_t)in * row_bytes;
+    const char* p = xbase + (uint64_t)(uint32_t)in * row_bytes + sl_off;
     const char* q[2];
 #pragma unroll
     for (int l = 0; l < NL; ++l) {
       q[l] = p + col_off[l];
-      if (!FULL) q[l] = col_ok[l] ? q[l] : zsrc + lane * 16;
+      const bool ok = WIDE ? sl_off + col_off[l] < row_bytes : col_ok[l];
+      if (!FULL) q[l] = ok ? q[l] : zsrc + lane * 16;
     }
     load_row<NL>(A[u], q[0], q[NL - 1]);
   };
@@ -574,11 +592,11 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the ring's last loads land before the registers are given up
 }
 
-template <typename T, int R, int NW, int NB, int NL, bool FULL, bool K2>
+template <typename T, int R, int NW, int NB, int NL, bool FULL, bool K2, bool WIDE>
 int launch_instance(const ConvArgs& a, hipStream_t s) {
   constexpr int lds = R * NB * 16 * 4 + 2 * NB * 16 * NL * 64 + PLAN_SLOTS * 1024 + MAX_BIAS * 4;
   static_assert(lds <= 160 * 1024, "LDS of one workgroup");
-  const void* fn = (const void*)conv_fwd_pack<T, R, NW, NB, NL, FULL, K2>;
+  const void* fn = (const void*)conv_fwd_pack<T, R, NW, NB, NL, FULL, K2, WIDE>;
   // more than 64 KiB of dynamic LDS has to be allowed once per device and kernel
   static std::mutex mu;
   static bool allowed[64] = {};
@@ -602,7 +620,7 @@ int launch_instance(const ConvArgs& a, hipStream_t s) {
   if (vtiles <= 0 || vtiles > INT32_MAX) return WCN_ERR_INVALID_ARGUMENT;
   const int per_cu = lds * 2 <= 160 * 1024 ? 2 : 1;  // workgroups resident per CU
   const unsigned grid = (unsigned)std::min<int64_t>(vtiles, (int64_t)cus[device] * per_cu);
-  hipLaunchKernelGGL((conv_fwd_pack<T, R, NW, NB, NL, FULL, K2>), dim3(grid), dim3((NW + 1) * 64), lds, s, a,
+  hipLaunchKernelGGL((conv_fwd_pack<T, R, NW, NB, NL, FULL, K2, WIDE>), dim3(grid), dim3((NW + 1) * 64), lds, s, a,
                      (int)vtiles, ny);
   return hipGetLastError() == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
 }
@@ -616,20 +634,21 @@ int launch_instance(const ConvArgs& a, hipStream_t s) {
 
 // Tile height: R rows for column groups of 64 channels, 2 R for 32 (same LDS).  Maps with fewer
 // such tiles than the GPU has CUs take tiles of half the height, so that more CUs have work.
-template <typename T, int NL, bool FULL, bool K2>
+template <typename T, int NL, bool FULL, bool K2, bool WIDE>
 int launch_shaped(const ConvArgs& a, hipStream_t s) {
   constexpr int R = WCN_PACK_R, NW = WCN_PACK_NW;
   const bool wide_out = a.c_out > 32;
   const int64_t ny = wide_out ? (a.c_out + 63) / 64 : 1;
   const int64_t tiles = (a.num_out + (wide_out ? R : 2 * R) - 1) / (wide_out ? R : 2 * R) * ny;
   const bool few = tiles < 224;
-  if (wide_out) return few ? launch_instance<T, R / 2, NW, 4, NL, FULL, K2>(a, s) : launch_instance<T, R, NW, 4, NL, FULL, K2>(a, s);
-  return few ? launch_instance<T, R, NW, 2, NL, FULL, K2>(a, s) : launch_instance<T, 2 * R, NW, 2, NL, FULL, K2>(a, s);
+  if (wide_out)
+    return few ? launch_instance<T, R / 2, NW, 4, NL, FULL, K2, WIDE>(a, s) : launch_instance<T, R, NW, 4, NL, FULL, K2, WIDE>(a, s);
+  return few ? launch_instance<T, R, NW, 2, NL, FULL, K2, WIDE>(a, s) : launch_instance<T, 2 * R, NW, 2, NL, FULL, K2, WIDE>(a, s);
 }
 
 template <typename T, int NL, bool FULL>
 int launch_sized(const ConvArgs& a, hipStream_t s) {
-  return a.K > 64 ? launch_shaped<T, NL, FULL, true>(a, s) : launch_shaped<T, NL, FULL, false>(a, s);
+  return a.K > 64 ? launch_shaped<T, NL, FULL, true, false>(a, s) : launch_shaped<T, NL, FULL, false, false>(a, s);
 }
 
 template <typename T>
@@ -637,6 +656,10 @@ int launch_typed(const ConvArgs& a, hipStream_t s) {
   const uint32_t row_bytes = (uint32_t)a.c_in * (uint32_t)sizeof(T);
   // the instances for whole rows address X with 32-bit byte offsets
   const bool near = (uint64_t)a.num_in * row_bytes < (1ull << 32);
+  if (row_bytes > 128) {  // several slices (wcn_conv_pack_takes has checked the limits)
+    const bool whole = row_bytes % 128 == 0 && near && a.num_in < (1 << 24);
+    return whole ? launch_shaped<T, 2, true, false, true>(a, s) : launch_shaped<T, 2, false, false, true>(a, s);
+  }
   if (row_bytes == 128 && near) return launch_sized<T, 2, true>(a, s);
   if (row_bytes == 64 && near) return launch_sized<T, 1, true>(a, s);
   if (row_bytes > 64) return launch_sized<T, 2, false>(a, s);
