@@ -1352,6 +1352,7 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   a.out = out;
   a.num_in = num_in;
   a.num_out = num_out;
+  a.num_pairs = L;
   a.G = w.G;
   a.K = num_offsets;
   a.c_in = c_in;

@@ -14,6 +14,7 @@ struct ConvArgs {
   const int32_t* group_start;  // (K, G + 1): pairs of offset k below output row 64 * g
   void* out;
   int64_t num_in, num_out, G;
+  int64_t num_pairs;           // all offsets together (known on the host)
   int32_t K, c_in, c_out, c_in_pad, c_out_pad, identity;
   int32_t vec_in;   // feature rows are 16-byte aligned and a whole number of 16-byte vectors
   int32_t vec_out;  // same for output rows

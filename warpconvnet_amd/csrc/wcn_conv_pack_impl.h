@@ -30,6 +30,7 @@
 #ifndef WCN_CONV_PACK_IMPL_H_
 #define WCN_CONV_PACK_IMPL_H_
 #include <algorithm>
+#include <cmath>
 #include <mutex>
 
 #include "wcn_common.h"
@@ -632,18 +633,54 @@ int launch_instance(const ConvArgs& a, hipStream_t s) {
 #define WCN_PACK_NW 11  // 12 waves: three per SIMD, 168 registers each; a 512-row tile's run of ~160 pairs is one step
 #endif
 
-// Tile height: R rows for column groups of 64 channels, 2 R for 32 (same LDS).  Maps with fewer
-// such tiles than the GPU has CUs take tiles of half the height, so that more CUs have work.
+// CUs of the current device (asked once per device).
+inline int device_cus() {
+  static std::mutex mu;
+  static int cus[64] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+  std::lock_guard<std::mutex> hold(mu);
+  if (cus[device] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n < 1) n = 256;
+    cus[device] = n;
+  }
+  return cus[device];
+}
+
+// Tile height: R, 3/4 R or 1/2 R rows for column groups of 64 channels, twice that for 32 (same
+// LDS), whichever an estimate of the run time likes best: rounds of the persistent grid times the
+// phases of a tile, a phase costing its barrier, weight tile and set-up (about one step's worth)
+// plus its steps.  Small tiles put more CUs to work on small maps; tall ones need fewer phases.
 template <typename T, int NL, bool FULL, bool K2, bool WIDE>
 int launch_shaped(const ConvArgs& a, hipStream_t s) {
   constexpr int R = WCN_PACK_R, NW = WCN_PACK_NW;
   const bool wide_out = a.c_out > 32;
   const int64_t ny = wide_out ? (a.c_out + 63) / 64 : 1;
-  const int64_t tiles = (a.num_out + (wide_out ? R : 2 * R) - 1) / (wide_out ? R : 2 * R) * ny;
-  const bool few = tiles < 224;
-  if (wide_out)
-    return few ? launch_instance<T, R / 2, NW, 4, NL, FULL, K2, WIDE>(a, s) : launch_instance<T, R, NW, 4, NL, FULL, K2, WIDE>(a, s);
-  return few ? launch_instance<T, R, NW, 2, NL, FULL, K2, WIDE>(a, s) : launch_instance<T, 2 * R, NW, 2, NL, FULL, K2, WIDE>(a, s);
+  const int cus = device_cus();
+  const double rows = (double)std::max<int64_t>(a.num_out, 1);
+  const bool has_identity = a.identity >= 0 && a.identity < a.K;
+  const double others = std::max(1, a.K - (has_identity ? 1 : 0));
+  const double per_row = std::max(0.0, (double)a.num_pairs - (has_identity ? rows : 0.0)) / (others * rows);
+  auto cost = [&](int r) {
+    const int64_t tiles = (a.num_out + r - 1) / r * ny;
+    const double rounds = (double)((tiles + cus - 1) / cus);
+    const double steps = std::max(1.0, std::ceil(r * per_row / PB / NW));
+    const double centre = has_identity ? 1.0 + std::ceil((double)r / PB / NW) : 0.0;
+    return rounds * (others * (1.0 + steps) + centre);
+  };
+  const int unit = wide_out ? R / 4 : R / 2;  // candidates: 2, 3, 4 units
+  int best = 4;
+  for (int q = 3; q >= 2; --q)
+    if (cost(q * unit) < cost(best * unit)) best = q;
+  if (wide_out) {
+    if (best == 2) return launch_instance<T, R / 2, NW, 4, NL, FULL, K2, WIDE>(a, s);
+    if (best == 3) return launch_instance<T, R / 4 * 3, NW, 4, NL, FULL, K2, WIDE>(a, s);
+    return launch_instance<T, R, NW, 4, NL, FULL, K2, WIDE>(a, s);
+  }
+  if (best == 2) return launch_instance<T, R, NW, 2, NL, FULL, K2, WIDE>(a, s);
+  if (best == 3) return launch_instance<T, R / 2 * 3, NW, 2, NL, FULL, K2, WIDE>(a, s);
+  return launch_instance<T, 2 * R, NW, 2, NL, FULL, K2, WIDE>(a, s);
 }
 
 template <typename T, int NL, bool FULL>
