@@ -31,7 +31,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
 # --calibrate-copy).  The summary names the kernel it was taken from; a line for another kernel
 # than the one this run launches is reported as stale (traffic: null).
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "conv_fwd_cfg2_hbm_traffic.txt")
-CONV_KERNEL = "conv_fwd_pack<f16, 512, 11, 4, 2, true, false>"  # what wcn_sparse_conv_fwd launches for 64 -> 64 fp16
+CONV_KERNEL = "conv_fwd_pack<f16, 512, 11, 4, 2, true, false, false>"  # what wcn_sparse_conv_fwd launches for 64 -> 64 fp16
 
 
 def measured_traffic():
