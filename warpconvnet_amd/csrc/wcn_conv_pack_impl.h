@@ -1,6 +1,6 @@
 // Pair-packed feature contraction (gfx950, MFMA): the kernel behind wcn_sparse_conv_fwd / _dgrad
-// for feature rows of at most one k-slice (64 channels of 16-bit data, 32 of fp32) and maps of at
-// most 128 offsets.
+// for feature rows of one to four 128-byte slices (64 channels of 16-bit data, 32 of fp32, per
+// slice) and maps of at most 128 offsets (64 when a row has several slices).
 //
 //   out[m, :] = bias + sum_k sum_{p in offset k, out_maps[p] == m} X[in_maps[p], :] @ W[k]
 //
@@ -14,10 +14,11 @@
 //     (out_maps ascends inside an offset; the run's bounds come from the group_start table); a run
 //     is cut into blocks of 16 pairs, block j goes to wave j % NW: every MFMA multiplies 16 real
 //     gathered rows (but for the last block of a run);
-//   * the tile is worked through one offset after the other (a "phase" per offset, one barrier
-//     between phases).  Inside a phase every output row occurs at most once, so the waves add
-//     their 16 x C_out products into the sums with plain LDS reads and writes: no atomics, and
-//     the order of the additions is fixed (k ascending), so results are bitwise reproducible;
+//   * the tile is worked through one offset after the other (a "phase" per offset -- per offset and
+//     slice for rows of several slices -- one barrier between phases).  Inside a phase every output
+//     row occurs at most once, so the waves add their 16 x C_out products into the sums with plain
+//     LDS reads and writes: no atomics, and the order of the additions is fixed (k ascending), so
+//     results are bitwise reproducible;
 //   * W[k]^T of the next phases travels memory -> registers -> LDS (two buffers) while the
 //     current phase runs; a wave reads the tile into registers once per phase;
 //   * a wave fetches the 16 gathered rows of a block straight from memory into registers in MFMA
@@ -25,8 +26,9 @@
 //     wave by a ring of U steps: while step s is multiplied, the rows of steps s+1 .. s+DG and
 //     the pair-list entries of steps up to s+U are in flight, across phase and tile boundaries.
 //
-// Every wave walks the same sequence of steps (phase k of a tile has max(1, ceil(blocks_k / NW))
-// steps; a step is empty for the waves beyond the run's last block), so the barriers line up.
+// A wave's steps are the blocks it has, plus one step (empty if need be) in a tile's last phase;
+// a step says how many phase barriers the wave passes before it, so every wave passes every barrier
+// and the phases line up although the waves walk different sequences of steps.
 #ifndef WCN_CONV_PACK_IMPL_H_
 #define WCN_CONV_PACK_IMPL_H_
 #include <algorithm>
