@@ -47,6 +47,13 @@ CONV_CASES = [
     ("f16_16_13", torch.float16, 16, 13, 3000, 1, (3, 3, 3)),
     ("f16_3_32", torch.float16, 3, 32, 3000, 1, (3, 3, 3)),      # network stem
     ("f16_256_256", torch.float16, 256, 256, 1500, 1, (3, 3, 3)),
+    # rows of several 128-byte slices: fp32 slices of 32 channels, a last slice that is partly there,
+    # a map of a single tile, and column groups of 32 output channels
+    ("f32_128_64", torch.float32, 128, 64, 3000, 2, (3, 3, 3)),
+    ("f16_160_96", torch.float16, 160, 96, 3000, 1, (3, 3, 3)),
+    ("f32_40_24", torch.float32, 40, 24, 2500, 1, (3, 3, 3)),
+    ("bf16_192_32_tiny", torch.bfloat16, 192, 32, 40, 1, (3, 3, 3)),
+    ("f16_128_128_k2", torch.float16, 128, 128, 3000, 1, (2, 2, 2)),
     ("f16_16_16_k5", torch.float16, 16, 16, 3000, 1, (5, 5, 5)),
     ("bf16_40_72_k2", torch.bfloat16, 40, 72, 3000, 1, (2, 2, 2)),
 ]
@@ -219,6 +226,11 @@ def test_conv_linearity_and_determinism():
     assert rel_err((2 * fa - 3 * fb).cpu().numpy(), fab.cpu().numpy()) <= 1e-5
     again = spatially_sparse_conv(_voxels(items, a), w, 3).feature_tensor
     assert torch.equal(fa, again)  # no atomics: bitwise reproducible
+    # the same for rows of several slices (their products are added slice by slice, in order)
+    wide = normal_features(n, 192, seed=4, dtype=torch.float16)
+    ww = kaiming_weight(27, 192, 64, seed=5, dtype=torch.float16).to(DEV)
+    first = spatially_sparse_conv(_voxels(items, wide), ww, 3).feature_tensor
+    assert torch.equal(first, spatially_sparse_conv(_voxels(items, wide), ww, 3).feature_tensor)
 
 
 def test_one_by_one_shortcut_and_errors():
