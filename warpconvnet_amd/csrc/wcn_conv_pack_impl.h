@@ -217,7 +217,22 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
   const int K = a.K;
   const int NS = WIDE ? (int)((size_t)a.c_in_pad * sizeof(T) / (NL * 64)) : 1;  // slices of a row
   const int KP = K * NS;                                                       // phases of a tile
-  auto tile_of = [&](int iter) -> int { return (int)blockIdx.x + iter * (int)gridDim.x; };
+  // Tiles of a workgroup: tile0, tile0 + gridDim.x, ...  With several column groups (ny > 1) the
+  // tiles of one row tile gather the same rows, so they should meet in one L2: workgroups go to the
+  // eight XCDs in turn (blockIdx.x % 8), and the ny workgroups that are neighbours on an XCD
+  // (blockIdx.x / 8 = ny * set + column group) take the column groups of row tile 8 * set + XCD.
+  // A permutation of [0, gridDim.x) when the grid divides that way; blockIdx.x itself otherwise.
+  int tile0 = (int)blockIdx.x;
+  {
+    const int grid = (int)gridDim.x, per_xcd = grid / 8;
+    if (ny > 1 && grid % 8 == 0 && per_xcd % ny == 0) {
+      const int xcd = (int)blockIdx.x % 8, q = (int)blockIdx.x / 8;
+      tile0 = ((q / ny) * 8 + xcd) * ny + q % ny;
+    }
+  }
+  tile0 = __builtin_amdgcn_readfirstlane(tile0);
+  const int tile_step = __builtin_amdgcn_readfirstlane((int)gridDim.x);
+  auto tile_of = [&](int iter) -> int { return tile0 + iter * tile_step; };
 
   if (wave == NW) {
     // ================= supplier wave =================
