@@ -350,19 +350,22 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
   // A wave's steps are the blocks it has to multiply, plus one step (empty if need be) in a tile's
   // last phase, where the tile is written out by all waves together.  Phases in which the wave has
   // no block cost it a barrier each and nothing else: the step that follows says how many.
-  // lane k % 64 holds the run of offset k in the generator's tile (offsets below 64 in [0], the
-  // others in [1]): pairs, first pair, this wave's steps
-  int plan_cnt[2] = {0, 0}, plan_start[2] = {0, 0}, plan_mine[2] = {0, 0};
+  // Per tile, lane k % 64 prepares what the wave's steps in offset k need (offsets below 64 in [0],
+  // the others in [1]): the descriptor word and the first pair of its first block there, the number
+  // of its blocks, the run's pairs; a step then takes its descriptor out of these registers.
+  uint32_t plan_w0[2] = {0u, 0u};
+  int plan_p0[2] = {0, 0}, plan_mine[2] = {0, 0}, plan_cnt[2] = {0, 0};
   unsigned long long plan_work[2] = {0ull, 0ull};  // the offsets in which this wave has a step
   int gen_iter = -1;                 // tiles this generator has entered, minus one
   int gen_k = K - 1, gen_sl = NS - 1, gen_sip = 0, gen_mine = 0;  // "past the last step of a tile": the first advance enters tile 0
-  int gen_cnt = 0, gen_start = 0, gen_ident = 0;
+  uint32_t gen_w0 = 0u;              // the first block of the wave in offset gen_k: descriptor word,
+  int gen_p0 = 0;                    //   first pair
   int64_t gen_m0 = 0;
   bool gen_live = true;              // false once the tiles are used up
   auto next_step = [&]() -> Step {
     Step d = {F_END, 0, 0};
     if (!gen_live) return d;
-    uint32_t flags = 0, bars = 0;
+    uint32_t extra = 0, bars = 0;
     if (gen_sip >= gen_mine && WIDE && gen_sl + 1 < NS) {  // the same blocks, next slice
       gen_sip = 0;
       ++gen_sl;
@@ -377,17 +380,25 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
           gen_live = false;
           return d;
         }
-        flags |= F_NEW_TILE;
+        extra |= F_NEW_TILE;
         gen_m0 = (int64_t)(tile_of(gen_iter) / ny) * R;
         const int32_t* slot = s_plan + (gen_iter % PLAN_SLOTS) * 256;
 #pragma unroll
         for (int h = 0; h < KH; ++h) {
-          plan_cnt[h] = slot[64 * h + lane];
-          plan_start[h] = slot[128 + 64 * h + lane];
-          const int nb = (plan_cnt[h] + PB - 1) / PB;
+          const int off = 64 * h + lane;
+          const int cnt = slot[off], start = slot[128 + off];
+          const int nb = (cnt + PB - 1) / PB;
           int mine = nb > wave ? (nb - wave + NW - 1) / NW : 0;
-          if (64 * h + lane == K - 1 && mine == 0) mine = 1;  // the step that ends the tile
+          if (off == K - 1 && mine == 0) mine = 1;  // the step that ends the tile
+          int n1 = cnt - wave * PB;                 // pairs of the wave's first block
+          n1 = n1 < 0 ? 0 : (n1 > PB ? PB : n1);
+          uint32_t w0 = (uint32_t)n1 | ((uint32_t)off << 8);
+          if (off == a.identity) w0 |= F_IDENT;
+          if (off == K - 1 && mine == 1) w0 |= F_TILE_END;
+          plan_w0[h] = w0;
+          plan_p0[h] = start + wave * PB;
           plan_mine[h] = mine;
+          plan_cnt[h] = cnt;
           plan_work[h] = __ballot(mine > 0);
         }
       }
@@ -404,24 +415,30 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
       bars = (uint32_t)((nk - gen_k - 1) * NS + 1);  // from the last slice of gen_k to the first of nk
       gen_k = nk;
       if (!K2 || gen_k < 64) {
-        gen_cnt = __builtin_amdgcn_readlane(plan_cnt[0], gen_k);
-        gen_start = __builtin_amdgcn_readlane(plan_start[0], gen_k);
+        gen_w0 = __builtin_amdgcn_readlane(plan_w0[0], gen_k);
+        gen_p0 = __builtin_amdgcn_readlane(plan_p0[0], gen_k);
         gen_mine = __builtin_amdgcn_readlane(plan_mine[0], gen_k);
       } else {
-        gen_cnt = __builtin_amdgcn_readlane(plan_cnt[1], gen_k - 64);
-        gen_start = __builtin_amdgcn_readlane(plan_start[1], gen_k - 64);
+        gen_w0 = __builtin_amdgcn_readlane(plan_w0[1], gen_k - 64);
+        gen_p0 = __builtin_amdgcn_readlane(plan_p0[1], gen_k - 64);
         gen_mine = __builtin_amdgcn_readlane(plan_mine[1], gen_k - 64);
       }
-      gen_ident = gen_k == a.identity ? 1 : 0;
     }
-    const int j = gen_sip * NW + wave;  // this wave's block of the run
-    int n = gen_cnt - j * PB;
-    n = n < 0 ? 0 : (n > PB ? PB : n);
-    if (gen_k == K - 1 && gen_sl == NS - 1 && gen_sip == gen_mine - 1) flags |= F_TILE_END;
-    if (gen_ident) flags |= F_IDENT;
+    uint32_t w0 = gen_w0;
+    int p0 = gen_p0;
+    if (gen_sip > 0) {  // a run of more than NW blocks: the wave's further blocks in the offset
+      const int cnt = (!K2 || gen_k < 64) ? __builtin_amdgcn_readlane(plan_cnt[0], gen_k)
+                                          : __builtin_amdgcn_readlane(plan_cnt[1], gen_k - 64);
+      int n = cnt - (gen_sip * NW + wave) * PB;
+      n = n < 0 ? 0 : (n > PB ? PB : n);
+      w0 = (uint32_t)n | (gen_w0 & (0xFF00u | F_IDENT));
+      p0 = gen_p0 + gen_sip * NW * PB;
+      if (gen_k == K - 1 && gen_sip == gen_mine - 1) w0 |= F_TILE_END;
+    }
+    if (WIDE && gen_sl != NS - 1) w0 &= ~F_TILE_END;  // the tile ends with the last slice
     ++gen_sip;
-    d.w0 = (uint32_t)n | ((uint32_t)gen_k << 8) | flags | ((uint32_t)gen_sl << 20) | (bars << 24);
-    d.p0 = gen_start + j * PB;
+    d.w0 = w0 | extra | ((uint32_t)gen_sl << 20) | (bars << 24);
+    d.p0 = p0;
     d.m0 = (int32_t)gen_m0;
     return d;
   };
