@@ -531,6 +531,7 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
           n0 = (vt % ny) * RS;
           tile_rows = (int)(a.num_out - m0 < R ? a.num_out - m0 : R);
         }
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): nothing pending after the barrier (said so that the compiler knows)
         // this phase's tile -> operand registers (only if this wave has a block in the phase)
         if (n > 0) {
 #pragma unroll
