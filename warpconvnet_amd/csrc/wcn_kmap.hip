@@ -4,7 +4,8 @@
 // passes (torch_discrete.py:80-157).  Here one thread owns one output voxel and resolves its K
 // offsets in registers; a wave's 64 voxels form a "group".  The probe pass stores, per offset and
 // group, the 64-bit mask of lanes that hit and its popcount, and the hit lanes park the input
-// rows they found, packed in lane order, in the (offset, group) cell of a scratch table.  A row-wise
+// rows they found in the group's stretch of a scratch table, packed offset by offset and in lane
+// order (one contiguous piece per group, for the emit pass to read back).  A row-wise
 // exclusive scan turns the counts into start positions; the emit pass then reads masks, starts
 // and parked rows -- no table probes -- and every hit lane writes its pair at start + (number of
 // hits in lower lanes).  Because groups are 64 consecutive output rows and lanes ascend within a
@@ -33,7 +34,7 @@ struct KmapWorkspace {  // host-computed addresses inside a kmap workspace
   int32_t* groups;      // (K+1, G+1): rows 0..K-1 per-offset hit counts of each 64-row group, row K
                         // all hits of the group; after the scan, exclusive prefix sums
   unsigned long long* hits;  // (G, K): lanes of the group that hit, per offset
-  int32_t* found;       // (K, 64 G): input rows found by the hit lanes of (offset, group), packed
+  int32_t* found;       // (G, 64 K): input rows found by the hit lanes of a group, packed offset by offset
   int64_t G;            // number of 64-row groups
 };
 
@@ -114,13 +115,13 @@ __global__ void __launch_bounds__(256) kmap_pass(const WcnTableHeader* __restric
         }
         const unsigned long long hits = __ballot(found >= 0);
         const int cnt = __popcll(hits);
-        group_hits += cnt;
         if (lane == 0) {
           groups[(int64_t)k * (G + 1) + group] = cnt;
           o.hits[group * g.K + k] = hits;
         }
-        if (found >= 0)  // hits of a group are parked contiguously, in lane order
-          o.found[(int64_t)k * (G * 64) + group * 64 + __popcll(hits & ((1ull << lane) - 1ull))] = found;
+        if (found >= 0)  // hits of a group are parked contiguously: offset by offset, in lane order
+          o.found[group * (64 * (int64_t)g.K) + group_hits + __popcll(hits & ((1ull << lane) - 1ull))] = found;
+        group_hits += cnt;
       }
     }
   }
@@ -254,13 +255,13 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
       const bool hit = (hm >> q) & 1u;
       const unsigned long long hits = __ballot(hit);
       const int cnt = __popcll(hits);
-      group_hits += cnt;
       if (lane == 0) {
         groups[(int64_t)k * (G + 1) + group] = cnt;
         o.hits[group * K + k] = hits;
       }
-      if (hit)  // hits of a group are parked contiguously, in lane order
-        o.found[(int64_t)k * (G * 64) + group * 64 + __popcll(hits & ((1ull << lane) - 1ull))] = found[q];
+      if (hit)  // hits of a group are parked contiguously: offset by offset, in lane order
+        o.found[group * (64 * (int64_t)K) + group_hits + __popcll(hits & ((1ull << lane) - 1ull))] = found[q];
+      group_hits += cnt;
     }
   }
   if (lane == 0) groups[(int64_t)K * (G + 1) + group] = group_hits;
@@ -286,6 +287,8 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
   if (offsets[K] > pair_capacity || offsets[K + 1] != 0) return;
   const int lane = wcn_lane();
   const unsigned long long below = (1ull << lane) - 1ull;
+  const int32_t* parked = found + group * (64 * (int64_t)K);  // the group's rows, offset by offset
+  int parked_before = 0;                                       // rows of the offsets walked so far
   for (int k0 = 0; k0 < K; k0 += 64) {
     unsigned long long h = 0ull;
     long long st = 0;
@@ -299,7 +302,8 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
 #pragma unroll
       for (int j = 0; j < KFIX; ++j) {
         const unsigned long long hj = __shfl(h, j, 64);
-        row[j] = ((hj >> lane) & 1ull) ? found[(int64_t)j * (G * 64) + group * 64 + __popcll(hj & below)] : -1;
+        row[j] = ((hj >> lane) & 1ull) ? parked[parked_before + __popcll(hj & below)] : -1;
+        parked_before += __popcll(hj);  // the same in every lane
       }
 #pragma unroll
       for (int j = 0; j < KFIX; ++j) {
@@ -317,9 +321,10 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
         const long long sj = __shfl(st, j, 64);
         if ((hj >> lane) & 1ull) {
           const long long p = sj + __popcll(hj & below);
-          in_maps[p] = found[(int64_t)(k0 + j) * (G * 64) + group * 64 + __popcll(hj & below)];
+          in_maps[p] = parked[parked_before + __popcll(hj & below)];
           out_maps[p] = (int32_t)m;
         }
+        parked_before += __popcll(hj);  // the same in every lane
       }
     }
   }
