@@ -52,12 +52,21 @@ __global__ void __launch_bounds__(1024) table_bbox(const int4* __restrict__ keys
   int mn[4] = {INT32_MAX, INT32_MAX, INT32_MAX, INT32_MAX};
   int mx[4] = {INT32_MIN, INT32_MIN, INT32_MIN, INT32_MIN};
   const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_keys; i += nthreads) {
-    const int4 c = keys[i];
-    mn[0] = min(mn[0], c.x); mx[0] = max(mx[0], c.x);
-    mn[1] = min(mn[1], c.y); mx[1] = max(mx[1], c.y);
-    mn[2] = min(mn[2], c.z); mx[2] = max(mx[2], c.z);
-    mn[3] = min(mn[3], c.w); mx[3] = max(mx[3], c.w);
+  constexpr int PER = 8;  // keys a thread has in flight together
+  for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i0 < n_keys; i0 += nthreads * PER) {
+    int4 c[PER];
+#pragma unroll
+    for (int t = 0; t < PER; ++t) {
+      const int64_t i = i0 + t * nthreads;
+      c[t] = keys[i < n_keys ? i : i0];  // past the end: the thread's first key again
+    }
+#pragma unroll
+    for (int t = 0; t < PER; ++t) {
+      mn[0] = min(mn[0], c[t].x); mx[0] = max(mx[0], c[t].x);
+      mn[1] = min(mn[1], c[t].y); mx[1] = max(mx[1], c[t].y);
+      mn[2] = min(mn[2], c[t].z); mx[2] = max(mx[2], c[t].z);
+      mn[3] = min(mn[3], c[t].w); mx[3] = max(mx[3], c[t].w);
+    }
   }
 #pragma unroll
   for (int d = 0; d < 4; ++d) {
