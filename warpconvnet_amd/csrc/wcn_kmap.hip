@@ -330,6 +330,81 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
   }
 }
 
+// Emit pass for maps of at most 64 offsets, a lane per PAIR: the parked rows of a group already lie
+// in the order of its pairs (offset by offset, in lane order), so lane p of a round takes pair
+// p, p + 64, ... of the group, finds the offset it belongs to (binary search over the running counts
+// the lanes hold), its rank there, and from rank and mask the output row.  A group's ~270 pairs cost
+// five rounds of one load and two stores where a walk over the offsets costs one load and two
+// stores of a few lanes each per offset.
+__device__ __forceinline__ int kmap_nth_set_bit(unsigned long long mask, int r) {  // position of the r-th set bit (r counts from 0)
+  uint32_t w = (uint32_t)mask;
+  int pos = 0;
+  int c = __popc(w);
+  if (r >= c) {
+    r -= c;
+    w = (uint32_t)(mask >> 32);
+    pos = 32;
+  }
+#pragma unroll
+  for (int half = 16; half >= 1; half >>= 1) {
+    const uint32_t low = w & ((1u << half) - 1u);
+    c = __popc(low);
+    if (r >= c) {
+      r -= c;
+      w >>= half;
+      pos += half;
+    } else {
+      w = low;
+    }
+  }
+  return pos;
+}
+
+__global__ void __launch_bounds__(256) kmap_emit_flat(const unsigned long long* __restrict__ hits,
+                                                      const int32_t* __restrict__ found,
+                                                      const int32_t* __restrict__ groups,
+                                                      const int64_t* __restrict__ offsets, int K,
+                                                      int64_t G, int64_t pair_capacity,
+                                                      int32_t* __restrict__ in_maps,
+                                                      int32_t* __restrict__ out_maps) {
+  const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t group = m >> 6;  // wave-uniform
+  if (group >= G) return;
+  if (offsets[K] > pair_capacity || offsets[K + 1] != 0) return;  // see kmap_emit
+  const int lane = wcn_lane();
+  const int32_t* parked = found + group * (64 * (int64_t)K);
+  unsigned long long h = 0ull;
+  long long st = 0;
+  if (lane < K) {
+    h = hits[group * K + lane];
+    st = offsets[lane] + groups[(int64_t)lane * (G + 1) + group];
+  }
+  const int cnt = __popcll(h);
+  const int incl = wcn_wave_inclusive_sum(cnt);  // pairs of the offsets up to and including this lane's
+  const int total = __shfl(incl, 63, 64);
+  for (int p0 = 0; p0 < total; p0 += 64) {
+    const int p = p0 + lane;
+    const bool live = p < total;
+    // first offset whose running count exceeds p (the lanes past K hold the total: never chosen by a live p)
+    int lo = 0, hi = 63;
+#pragma unroll
+    for (int step = 0; step < 6; ++step) {
+      const int mid = (lo + hi) >> 1;
+      const int v = __shfl(incl, mid, 64);
+      if (v <= p) lo = mid + 1; else hi = mid;
+    }
+    const int k = lo;
+    const unsigned long long hk = __shfl(h, k, 64);
+    const long long sk = __shfl(st, k, 64);
+    const int rank = p - (__shfl(incl, k, 64) - __popcll(hk));
+    if (live) {
+      const long long dst = sk + rank;
+      in_maps[dst] = parked[p];
+      out_maps[dst] = (int32_t)(group * 64 + kmap_nth_set_bit(hk, rank));
+    }
+  }
+}
+
 // In-place exclusive prefix sum of each row of `groups` (one workgroup per row, G+1 entries; the
 // last entry receives the row total).
 __global__ void kmap_zero_ticket(int32_t* ticket) { *ticket = 0; }
@@ -488,7 +563,10 @@ void launch_emit(int64_t num_out, const KmapGeom& g, const KmapWorkspace& w, int
                  int32_t* in_maps, int32_t* out_maps, hipStream_t s) {
   const dim3 grid(grid_for(num_out, 256)), block(256);
   const int64_t* offsets = (const int64_t*)w.result;
-  if (g.K == 27) {
+  if (g.K <= 64) {
+    hipLaunchKernelGGL(kmap_emit_flat, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
+                       w.G, pair_capacity, in_maps, out_maps);
+  } else if (g.K == 27) {
     hipLaunchKernelGGL(kmap_emit<27>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
                        w.G, pair_capacity, in_maps, out_maps);
   } else if (g.K == 8) {
