@@ -267,18 +267,16 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
   if (lane == 0) groups[(int64_t)K * (G + 1) + group] = group_hits;
 }
 
-// Emit pass: pair lists from the masks, scanned counts and parked rows of the probe pass.  Lane j
-// fetches mask and start of offset k0 + j for the whole group; the lanes then walk the offsets
-// together.
-template <int KFIX>
+// Emit pass: pair lists from the masks, scanned counts and parked rows of the probe pass.  This
+// kernel takes maps of any size (the launch uses it for more than 64 offsets): lane j fetches mask
+// and start of offset k0 + j for the whole group; the lanes then walk the offsets together.
 __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __restrict__ hits,
                                                  const int32_t* __restrict__ found,
                                                  const int32_t* __restrict__ groups,
-                                                 const int64_t* __restrict__ offsets, int K_runtime,
+                                                 const int64_t* __restrict__ offsets, int K,
                                                  int64_t G, int64_t pair_capacity,
                                                  int32_t* __restrict__ in_maps,
                                                  int32_t* __restrict__ out_maps) {
-  const int K = KFIX > 0 ? KFIX : K_runtime;
   const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t group = m >> 6;  // wave-uniform
   if (group >= G) return;
@@ -297,35 +295,15 @@ __global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __res
       st = offsets[k0 + lane] + groups[(int64_t)(k0 + lane) * (G + 1) + group];
     }
     const int n = K - k0 < 64 ? K - k0 : 64;
-    if (KFIX > 0) {
-      int32_t row[KFIX > 0 ? KFIX : 1];
-#pragma unroll
-      for (int j = 0; j < KFIX; ++j) {
-        const unsigned long long hj = __shfl(h, j, 64);
-        row[j] = ((hj >> lane) & 1ull) ? parked[parked_before + __popcll(hj & below)] : -1;
-        parked_before += __popcll(hj);  // the same in every lane
+    for (int j = 0; j < n; ++j) {
+      const unsigned long long hj = __shfl(h, j, 64);
+      const long long sj = __shfl(st, j, 64);
+      if ((hj >> lane) & 1ull) {
+        const long long p = sj + __popcll(hj & below);
+        in_maps[p] = parked[parked_before + __popcll(hj & below)];
+        out_maps[p] = (int32_t)m;
       }
-#pragma unroll
-      for (int j = 0; j < KFIX; ++j) {
-        const unsigned long long hj = __shfl(h, j, 64);
-        const long long sj = __shfl(st, j, 64);
-        if ((hj >> lane) & 1ull) {
-          const long long p = sj + __popcll(hj & below);
-          in_maps[p] = row[j];
-          out_maps[p] = (int32_t)m;
-        }
-      }
-    } else {
-      for (int j = 0; j < n; ++j) {
-        const unsigned long long hj = __shfl(h, j, 64);
-        const long long sj = __shfl(st, j, 64);
-        if ((hj >> lane) & 1ull) {
-          const long long p = sj + __popcll(hj & below);
-          in_maps[p] = parked[parked_before + __popcll(hj & below)];
-          out_maps[p] = (int32_t)m;
-        }
-        parked_before += __popcll(hj);  // the same in every lane
-      }
+      parked_before += __popcll(hj);  // the same in every lane
     }
   }
 }
@@ -566,14 +544,8 @@ void launch_emit(int64_t num_out, const KmapGeom& g, const KmapWorkspace& w, int
   if (g.K <= 64) {
     hipLaunchKernelGGL(kmap_emit_flat, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
                        w.G, pair_capacity, in_maps, out_maps);
-  } else if (g.K == 27) {
-    hipLaunchKernelGGL(kmap_emit<27>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
-                       w.G, pair_capacity, in_maps, out_maps);
-  } else if (g.K == 8) {
-    hipLaunchKernelGGL(kmap_emit<8>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
-                       w.G, pair_capacity, in_maps, out_maps);
   } else {
-    hipLaunchKernelGGL(kmap_emit<0>, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
+    hipLaunchKernelGGL(kmap_emit, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
                        w.G, pair_capacity, in_maps, out_maps);
   }
 }

@@ -70,7 +70,9 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     out4 = _four_columns(out_coords)
     M = out4.shape[0]
     ws = workspace(L.wcn_kmap_workspace_bytes(M, K), device)
-    host_offsets = (ctypes.c_int64 * (K + 1))()
+    # the library writes the result into this host tensor; the ctypes array is a view of it
+    offsets64 = torch.empty(K + 1, dtype=torch.int64)
+    host_offsets = (ctypes.c_int64 * (K + 1)).from_address(offsets64.data_ptr())
     # The pairs are emitted into buffers of assumed size while the pair count is still on its way
     # to the host (a voxel of a surface-like scene has a handful of neighbours, far from K); the
     # lists handed out are views of these buffers.  More pairs than assumed: the emit pass has
@@ -90,6 +92,13 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
                                            stream_ptr(device)), "wcn_kmap_count_dilated")
         check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), assumed,
                               ptr(in_buf), ptr(out_buf), stream_ptr(device)), "wcn_kmap_fill")
+        # By-product the contraction reuses: the per-64-row group starts of every offset, (K, G + 1)
+        # int32, final once the count call's kernels have run.  Only this table is kept with the
+        # map (a copy of about K * M / 16 bytes; the workspace, whose probe results are K * M * 4
+        # bytes, goes back to the allocator).  The copy is enqueued here, before the wait for the
+        # result, so that nothing stands between that wait and what the caller launches next.
+        begin = L.wcn_kmap_group_start(ptr(ws), M, K) - ws.data_ptr()
+        groups = ws[begin:begin + 4 * K * ((M + 63) // 64 + 1)].clone()
         status = L.wcn_kmap_read_result(ptr(ws), M, K, host_offsets, stream_ptr(device))
         if status == ERR_TABLE_OVERFLOW:
             table._grow()
@@ -108,16 +117,11 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
         out_maps = torch.empty(total, dtype=torch.int32, device=device)
         check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), total,
                               ptr(in_maps), ptr(out_maps), stream_ptr(device)), "wcn_kmap_fill")
-    offsets = torch.from_numpy(np.ctypeslib.as_array(host_offsets).astype(np.int32))
+    offsets = offsets64.to(torch.int32)
     result = IntSearchResult(in_maps, out_maps, offsets, identity_map_index=identity_map_index)
     result._host_offsets = host_offsets  # the contraction passes them on as they are
-    # by-products the contraction reuses: pairs ascend in output row inside every offset, and
-    # the workspace holds their per-64-row group starts, (K, G + 1) int32.  Only that table is
-    # kept with the map (a copy of about K * M / 16 bytes); the workspace itself, whose probe
-    # results are K * M * 4 bytes, goes back to the allocator here.
-    result._out_ascend = True
-    begin = L.wcn_kmap_group_start(ptr(ws), M, K) - ws.data_ptr()
-    groups = ws[begin:begin + 4 * K * ((M + 63) // 64 + 1)].clone()
+    result._offsets64 = offsets64        # the memory behind that array
+    result._out_ascend = True  # pairs ascend in output row inside every offset
     result._group_start = (groups, groups.data_ptr(), (K, M))
     result._keys_unique = (L.wcn_kmap_last_table_flags() & 1) == 0
     return result
