@@ -56,6 +56,14 @@ CONV_CASES = [
     ("f16_128_128_k2", torch.float16, 128, 128, 3000, 1, (2, 2, 2)),
     ("f16_16_16_k5", torch.float16, 16, 16, 3000, 1, (5, 5, 5)),
     ("bf16_40_72_k2", torch.bfloat16, 40, 72, 3000, 1, (2, 2, 2)),
+    # wide rows on both sides and at least 96 tiles of 256 output rows: the output-stationary kernel
+    # (sums in registers), with and without an identity offset, last tile partly filled; tiles of
+    # 192 rows (four 48-row waves, whose rows span two 64-row groups) and, for the map of 51,000
+    # rows, of 256 rows (eight 32-row waves)
+    ("f16_128_128_rows", torch.float16, 128, 128, 13000, 2, (3, 3, 3)),
+    ("bf16_256_128_rows", torch.bfloat16, 256, 128, 12500, 2, (3, 3, 3)),
+    ("f16_128_256_rows_k2", torch.float16, 128, 256, 13000, 2, (2, 2, 2)),
+    ("bf16_128_128_rows_tall", torch.bfloat16, 128, 128, 17000, 3, (3, 3, 3)),
 ]
 
 

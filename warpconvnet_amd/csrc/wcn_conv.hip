@@ -1103,12 +1103,21 @@ template <typename T>
 int launch_conv(const ConvArgs& a, hipStream_t s) {
   constexpr int dtype = std::is_same<T, float>::value ? WCN_DTYPE_F32
                         : std::is_same<T, _Float16>::value ? WCN_DTYPE_F16 : WCN_DTYPE_BF16;
-  // Rows of at most one k-slice go to the pair-packed kernel.  WCN_CONV_KERNEL=ring in the
-  // environment keeps them on the output-stationary kernels below (for comparisons).
-  static const bool ring_only = [] {
+  // Wide rows on both sides go to the output-stationary kernel of wcn_conv_dense.hip, rows of up to
+  // four k-slices to the pair-packed kernel.  WCN_CONV_KERNEL=ring in the environment keeps
+  // everything on the kernels below, WCN_CONV_KERNEL=pack skips the first of the two (for comparisons).
+  static const int only = [] {
     const char* e = getenv("WCN_CONV_KERNEL");
-    return e && std::string(e) == "ring";
+    return !e ? 0 : std::string(e) == "ring" ? 1 : std::string(e) == "pack" ? 2 : 0;
   }();
+  const bool ring_only = only == 1;
+  if (only == 0 && wcn_conv_dense_takes(a, dtype)) {
+    if (g_time_start) (void)hipEventRecord(g_time_start, s);
+    const int st = wcn_conv_dense_launch(a, dtype, s);
+    if (g_time_stop) (void)hipEventRecord(g_time_stop, s);
+    g_time_start = g_time_stop = nullptr;
+    return st;
+  }
   if (!ring_only && wcn_conv_pack_takes(a, dtype)) {
     if (g_time_start) (void)hipEventRecord(g_time_start, s);
     const int st = wcn_conv_pack_launch(a, dtype, s);

@@ -32,4 +32,9 @@ constexpr int WCN_PACK_MAX_BIAS = 1024;  // output channels (padded) whose bias 
 bool wcn_conv_pack_takes(const ConvArgs& a, int dtype);
 int wcn_conv_pack_launch(const ConvArgs& a, int dtype, hipStream_t stream);
 
+// The output-stationary contraction for wide rows (wcn_conv_dense.hip): whether it takes a problem,
+// and its launch.
+bool wcn_conv_dense_takes(const ConvArgs& a, int dtype);
+int wcn_conv_dense_launch(const ConvArgs& a, int dtype, hipStream_t stream);
+
 #endif  // WCN_CONV_ARGS_H_
