@@ -115,14 +115,16 @@ __global__ void __launch_bounds__(DENSE_WAVES * 64) conv_fwd_dense(ConvArgs a, i
     // the entries of offset k's run, NE per lane (requested an offset ahead)
     auto request = [&](int k, int32_t (&e_in)[NE], int32_t (&e_out)[NE]) {
       const int lo = __builtin_amdgcn_readlane(run_lo, k), cnt = __builtin_amdgcn_readlane(run_cnt, k);
+      // no branches (the loads sit between the MFMAs of a chunk): lanes past the run read its last
+      // entry, an empty run reads zeros; settle() looks at the count again
+      const int32_t* pin = cnt > 0 ? a.in_maps + lo : (const int32_t*)a.zeros;
+      const int32_t* pout = cnt > 0 ? a.out_maps + lo : (const int32_t*)a.zeros;
+      const int last = cnt > 0 ? cnt - 1 : 0;
 #pragma unroll
       for (int h = 0; h < NE; ++h) {
-        e_in[h] = -1;
-        e_out[h] = -1;
-        if (lane + 64 * h < cnt) {
-          e_in[h] = a.in_maps[lo + lane + 64 * h];
-          e_out[h] = a.out_maps[lo + lane + 64 * h];
-        }
+        const int i = lane + 64 * h < last ? lane + 64 * h : last;
+        e_in[h] = pin[i];
+        e_out[h] = pout[i];
       }
     };
     // ... turned into the input row of each of the wave's output rows (lane (c, *): rows c, 16 + c, 32 + c, 48 + c)
@@ -136,10 +138,11 @@ __global__ void __launch_bounds__(DENSE_WAVES * 64) conv_fwd_dense(ConvArgs a, i
         return;
       }
       if (lane < WROWS_OUT) mytab[lane] = -1;
+      const int cnt = __builtin_amdgcn_readlane(run_cnt, k);
 #pragma unroll
       for (int h = 0; h < NE; ++h) {
         const uint32_t slot = (uint32_t)(e_out[h] - base);
-        if (e_in[h] >= 0 && slot < (uint32_t)WROWS_OUT && (uint32_t)e_in[h] < (uint32_t)a.num_in &&
+        if (lane + 64 * h < cnt && e_in[h] >= 0 && slot < (uint32_t)WROWS_OUT && (uint32_t)e_in[h] < (uint32_t)a.num_in &&
             (int64_t)e_out[h] < a.num_out)
           mytab[slot] = e_in[h];
       }
@@ -174,18 +177,14 @@ __global__ void __launch_bounds__(DENSE_WAVES * 64) conv_fwd_dense(ConvArgs a, i
       const int nchunk = chunk + 1 < NC ? chunk + 1 : 0;
       const int nk = (nchunk == 0 && k + 1 < K) ? k + 1 : k;
       // Every step issues the same loads in the same order, needed or not (the last step of a tile
-      // fetches its own chunk again, every step of an offset fetches the next offset's entries):
-      // the wait for the rows of the current chunk is then the same count of younger loads on
-      // every path into the multiplication below, and nothing loaded in a step is used in it.
+      // fetches its own chunk again, every step of an offset fetches the next offset's entries),
+      // and nothing loaded in a step is used in it: the waits for loaded data are then the same
+      // counts on every path.  The loads are issued between the first MFMAs of the chunk, whose
+      // operands are at hand, so that their address arithmetic runs beside the multiplications.
       if (nchunk == 0 && more) settle(nk, e_in, e_out, in_next);  // entries requested a step ago
-      load_w(nk, nchunk, wr);
-      request(k + 1 < K ? k + 1 : k, e_in, e_out);
-      {
-        int32_t in_sel[RB];
+      int32_t in_sel[RB];
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) in_sel[rb] = nchunk == 0 ? in_next[rb] : in_cur[rb];
-        load_rows(in_sel, nchunk, a_next);
-      }
+      for (int rb = 0; rb < RB; ++rb) in_sel[rb] = nchunk == 0 ? in_next[rb] : in_cur[rb];
       // ---- multiply the current chunk: the operands of the 16-channel blocks to come are read
       //      AHEAD blocks before they are multiplied ----
       constexpr int AHEAD = 3;
@@ -207,8 +206,14 @@ __global__ void __launch_bounds__(DENSE_WAVES * 64) conv_fwd_dense(ConvArgs a, i
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb)
             acc[rb][cb] = Mma<T>::mma(__builtin_bit_cast(V, wq[cb % (AHEAD + 1)][l]), a_cur[rb][l], acc[rb][cb]);
+        if (cb == 0) load_w(nk, nchunk, wr);
+        if (cb == 1) request(k + 1 < K ? k + 1 : k, e_in, e_out);
+        if (cb == 2) load_rows(in_sel, nchunk, a_next);
         __builtin_amdgcn_sched_group_barrier(0x008, 2 * RB, 0);  // this block's MFMAs
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);       // the operands AHEAD blocks on
+        if (cb == 0) __builtin_amdgcn_sched_group_barrier(0x020, WPT, 0);     // the next chunk's weights
+        if (cb == 1) __builtin_amdgcn_sched_group_barrier(0x020, 2 * NE, 0);  // the next offset's entries
+        if (cb == 2) __builtin_amdgcn_sched_group_barrier(0x020, 2 * RB, 0);  // the next chunk's rows
       }
       if (more) store_w(buf ^ 1, wr);
       __syncthreads();  // everybody has read this chunk's buffer and written the next one's
