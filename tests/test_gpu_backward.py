@@ -41,6 +41,10 @@ CASES = [
     ("f16_3_32", torch.float16, 3, 32, 2500, 1, (3, 3, 3)),
     ("f16_16_16_k5", torch.float16, 16, 16, 2500, 1, (5, 5, 5)),
     ("bf16_40_72_k2", torch.bfloat16, 40, 72, 2500, 1, (2, 2, 2)),
+    # wide rows and enough of them for the output-stationary kernel: forward 128 -> 256 and, for the
+    # input gradient, the same kernel over 256 -> 128 (odd kernel: symmetric map; even: re-ordered map)
+    ("f16_128_256_rows", torch.float16, 128, 256, 13000, 2, (3, 3, 3)),
+    ("bf16_128_128_rows_k2", torch.bfloat16, 128, 128, 13000, 2, (2, 2, 2)),
 ]
 
 
