@@ -564,7 +564,7 @@ def main():
             "contraction_frac_of_mfma_peak": conv_flops / (conv_kernel_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
         },
         "roofline": {
-            "kernel": CONV_KERNEL if not os.environ.get("WCN_CONV_KERNEL") else "conv_fwd_ring<f16, 6, false, 0>",
+            "kernel": CONV_KERNEL if os.environ.get("WCN_CONV_KERNEL") != "ring" else "conv_fwd_ring<f16, 6, false, 0>",
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
