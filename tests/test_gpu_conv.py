@@ -64,6 +64,7 @@ CONV_CASES = [
     ("bf16_256_128_rows", torch.bfloat16, 256, 128, 12500, 2, (3, 3, 3)),
     ("f16_128_256_rows_k2", torch.float16, 128, 256, 13000, 2, (2, 2, 2)),
     ("bf16_128_128_rows_tall", torch.bfloat16, 128, 128, 17000, 3, (3, 3, 3)),
+    ("f16_256_128_rows_k1", torch.float16, 256, 128, 13000, 2, (1, 1, 1)),   # pointwise: the identity offset alone
 ]
 
 
