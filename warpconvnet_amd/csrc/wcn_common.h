@@ -30,32 +30,69 @@ struct __attribute__((aligned(32))) WcnSlot {
 struct WcnTableHeader {  // first 256 bytes of a table workspace
   int32_t mn[4];         // bounding box of the keys, per column
   int32_t mx[4];
-  int32_t num_blocks;    // occupied slots
+  int32_t num_blocks;    // occupied slots (valid after table_sum_stats)
   int32_t status;        // WCN_DEV_* bits
-  int32_t total;         // running sum of block populations (ends at the number of distinct keys)
+  int32_t total;         // number of distinct keys (valid after table_sum_stats)
   int32_t num_keys;      // keys inserted; more keys than set bits (`total`) means some key came twice
-  int32_t reserved[52];
+  int32_t bins;          // bins of the build
+  int32_t pad;
+  int64_t stats_offset;  // bytes from the header to the bins' (voxels, blocks) counts
+  int32_t reserved[48];
 };
 static_assert(sizeof(WcnTableHeader) == 256, "header is 256 bytes");
 
-// Valid once the populations have been summed (table_base): every distinct key set one bit.
+// Valid once the bins' counts have been summed into the header: every distinct key set one bit.
 #define WCN_HAS_DUPLICATES(hdr) ((hdr)->total != (hdr)->num_keys)
 
 struct WcnTableView {  // host-computed addresses inside a table workspace
   WcnTableHeader* hdr;
   WcnSlot* slots;
   int32_t* perm;        // n_keys
-  int32_t* slot_of;     // n_keys (slot of each key; build scratch)
+  int32_t* slot_of;     // n_keys (slot of each key; written on request)
+  // The keys in block order: every key once, the keys of one block next to each other, the blocks
+  // of one bin next to each other.  Queries walked in this order meet their neighbours' slots and
+  // `perm` entries in the caches.
+  int32_t* order_coords;  // (n_keys, 4)
+  int32_t* order_row;     // n_keys: input row of each entry
+  // build scratch
+  int32_t* bin_coords;    // (n_keys, 4) keys grouped by bin
+  int32_t* bin_row;       // n_keys
+  int32_t* hist;          // (bins, parts) keys of part w in bin b, then their exclusive prefix sums
+  int32_t* bin_total;     // bins: keys per bin
+  int32_t* bin_start;     // bins + 1
+  int32_t* bin_stats;     // (bins, 2): distinct keys and blocks of each bin
+  int32_t* part_box;      // (parts, 8) bounding box of each part's keys
   int64_t n_keys;
   int64_t capacity;
+  int32_t bins;           // power of two
+  int32_t parts;          // workgroups of the histogram and scatter passes
 };
 
 static inline size_t wcn_align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// Keys are first grouped into bins of one to two thousand (a bin is a hash of the key's 16x16x16-voxel
+// cell, so the 4x4x4 blocks of a cell stay together); the bin count follows the slot count, so a
+// rebuild with more slots also re-deals the bins.
+#define WCN_BIN_SLOTS 4096      // distinct blocks a bin can hold (its table in LDS)
+#define WCN_PART_KEYS 4096      // keys per workgroup of the histogram and scatter passes
+static inline int32_t wcn_table_bins(int64_t capacity) {
+  int64_t b = capacity / 2048;
+  if (b < 16) b = 16;
+  if (b > 4096) b = 4096;
+  return (int32_t)b;
+}
+static inline int32_t wcn_table_parts(int64_t n_keys) {
+  int64_t w = (n_keys + WCN_PART_KEYS - 1) / WCN_PART_KEYS;
+  if (w < 1) w = 1;
+  if (w > 256) w = 256;
+  return (int32_t)w;
+}
 
 static inline size_t wcn_table_layout(void* base, int64_t n_keys, int64_t capacity,
                                       WcnTableView* v) {
   char* p = (char*)base;
   size_t off = 0;
+  const int32_t bins = wcn_table_bins(capacity), parts = wcn_table_parts(n_keys);
   if (v) v->hdr = (WcnTableHeader*)(p + off);
   off += 256;
   if (v) v->slots = (WcnSlot*)(p + off);
@@ -64,9 +101,29 @@ static inline size_t wcn_table_layout(void* base, int64_t n_keys, int64_t capaci
   off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
   if (v) v->slot_of = (int32_t*)(p + off);
   off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
+  if (v) v->order_coords = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * 4 * (size_t)n_keys);
+  if (v) v->order_row = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
+  if (v) v->bin_coords = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * 4 * (size_t)n_keys);
+  if (v) v->bin_row = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
+  if (v) v->hist = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)bins * (size_t)parts);
+  if (v) v->bin_total = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)bins);
+  if (v) v->bin_start = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)(bins + 1));
+  if (v) v->bin_stats = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * 2 * (size_t)bins);
+  if (v) v->part_box = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * 8 * (size_t)parts);
   if (v) {
     v->n_keys = n_keys;
     v->capacity = capacity;
+    v->bins = bins;
+    v->parts = parts;
   }
   return off;
 }

@@ -14,7 +14,7 @@
 #include "wcn_common.h"
 
 int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView& v,
-                         hipStream_t s);
+                         bool want_slot_of, hipStream_t s);
 int wcn_table_status_from_bits(int32_t bits);
 
 namespace {
@@ -465,9 +465,24 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
     }
     run += __shfl(v, 63, 64);
   }
+  // occupied slots and distinct keys of the table: the sums of the bins' counts
+  int voxels = 0, occupied = 0;
+  {
+    const int32_t bins = fin.hdr->bins;
+    const int32_t* stats = reinterpret_cast<const int32_t*>(reinterpret_cast<const char*>(fin.hdr) + fin.hdr->stats_offset);
+    for (int i = lane; i < bins; i += 64) {
+      voxels += stats[2 * i];
+      occupied += stats[2 * i + 1];
+    }
+#pragma unroll
+    for (int sft = 32; sft > 0; sft >>= 1) {
+      voxels += __shfl_xor(voxels, sft, 64);
+      occupied += __shfl_xor(occupied, sft, 64);
+    }
+  }
   if (lane == 0) {
     const int64_t status = fin.hdr->status;
-    const int64_t blocks = (int64_t)fin.hdr->num_blocks | ((int64_t)(WCN_HAS_DUPLICATES(fin.hdr) ? 1 : 0) << 32);
+    const int64_t blocks = (int64_t)occupied | ((int64_t)(voxels != fin.hdr->num_keys ? 1 : 0) << 32);
     fin.result[0] = 0;
     fin.result[fin.K + 1] = status;
     fin.result[fin.K + 2] = blocks;
@@ -790,7 +805,7 @@ int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_strid
     hipLaunchKernelGGL(stride_divide, dim3(grid_for(n, 256)), dim3(256), 0, s, (const int4*)coords,
                        n, host_stride[0], host_stride[1], host_stride[2], (int4*)w.coarse);
   }
-  const int rc = wcn_table_build_impl(w.coarse, n, v, s);
+  const int rc = wcn_table_build_impl(w.coarse, n, v, true, s);
   if (rc != WCN_OK) return rc;
   if (n > 0) {
     hipLaunchKernelGGL(stride_pick<false>, dim3(grid_for(n, 256)), dim3(256), 0, s,

@@ -1,72 +1,92 @@
 // Coordinate table of 4x4x4-voxel blocks: build and point queries (gfx950).
 //
-// Build pipeline (all on the caller's stream, no host round trip):
-//   table_clear   header, slots and perm to their empty values
-//   table_bbox    bounding box of the keys (LDS reduction, one atomic min/max per workgroup)
-//   table_insert  per key: claim / find the block slot with a 64-bit CAS, OR the voxel bit in
-//   table_base    per slot: base = running sum of block populations (one atomic per 1024 slots)
-//   table_perm    per key: perm[base + rank of its bit] = min(row index)
+// Build pipeline (all on the caller's stream, no host round trip).  The keys are first grouped into
+// bins of one to two thousand (a bin is a hash of the key's 16x16x16-voxel cell, so every 4x4x4
+// block lies in exactly one bin); one workgroup per bin then sees all voxels of its blocks and
+// builds their masks with LDS atomics:
+//   table_hist     per part of the keys (a workgroup): keys per bin (LDS counters) and the part's
+//                  bounding box
+//   table_colscan  per bin (a wave): prefix sums over the parts; the last workgroup to finish turns
+//                  the bin totals into bin starts, merges the boxes and initialises the header
+//   table_scatter  per part: every key and its row to its place in its bin; clears the slots
+//   table_bins     per bin: block masks and entry counts in an LDS table, their prefix sums, one
+//                  64-bit CAS per BLOCK to claim a slot of the table in memory (mask and base are
+//                  plain stores), then per key: its place in block order and perm[base + rank] = row
 //
-// HBM traffic per key: 16 B read (bbox) + 16 B read (insert) + 4 B slot_of write + 4 B read +
-// 4 B perm write, plus 32 B per table slot to clear and one 32 B slot touched per key.
+// HBM traffic per key: 16 B read twice (histogram, scatter), 20 B written and read (binned entry),
+// 20 B written (entry in block order) + 4 B (perm), plus 32 B per table slot to clear.
 #include <stdlib.h>
 #include <string.h>
 
 #include <chrono>
+#include <mutex>
 #include <thread>
 
 #include "wcn_common.h"
 
 namespace {
 
-__global__ void __launch_bounds__(256) table_clear(WcnTableHeader* __restrict__ hdr,
-                                                   WcnSlot* __restrict__ slots, int64_t capacity,
-                                                   int32_t* __restrict__ perm, int64_t n_keys) {
-  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
-  if (tid == 0) {
-    for (int d = 0; d < 4; ++d) {
-      hdr->mn[d] = INT32_MAX;
-      hdr->mx[d] = INT32_MIN;
-    }
-    hdr->num_blocks = 0;
-    hdr->status = 0;
-    hdr->total = 0;
-    hdr->num_keys = (int32_t)n_keys;
-  }
-  // each slot is two 16-byte stores: {EMPTY, 0} and {0, 0, 0, 0}
-  uint4* raw = reinterpret_cast<uint4*>(slots);
-  for (int64_t i = tid; i < 2 * capacity; i += nthreads) {
-    uint4 v = (i & 1) ? make_uint4(0u, 0u, 0u, 0u) : make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0u, 0u);
-    raw[i] = v;
-  }
-  for (int64_t i = tid; i < n_keys; i += nthreads) perm[i] = INT32_MAX;
+// Bin of a key: a hash of (batch, x >> 4, y >> 4, z >> 4).  Block boundaries are multiples of four
+// in absolute coordinates (the table's origin is rounded down to one), so a block never straddles
+// two cells.
+__device__ __forceinline__ uint32_t bin_of(const int4 c, uint32_t bin_mask) {
+  const unsigned long long a = ((unsigned long long)(uint32_t)c.x << 32) | (uint32_t)(c.y >> 4);
+  const unsigned long long b = ((unsigned long long)(uint32_t)(c.z >> 4) << 32) | (uint32_t)(c.w >> 4);
+  return wcn_mix(a * 0x9E3779B97F4A7C15ull + b, bin_mask);
 }
 
-// Bounding box of the keys.  Few, wide workgroups: the eight atomics a workgroup ends with all
-// land on the same eight words and serialise, so their number decides the run time.
-__global__ void __launch_bounds__(1024) table_bbox(const int4* __restrict__ keys, int64_t n_keys,
-                                                   WcnTableHeader* __restrict__ hdr) {
+struct PartRange {
+  int64_t lo, hi;
+};
+__device__ __forceinline__ PartRange part_range(int64_t n_keys) {
+  const int64_t chunk = (n_keys + gridDim.x - 1) / gridDim.x;
+  PartRange r;
+  r.lo = (int64_t)blockIdx.x * chunk;
+  r.hi = r.lo + chunk < n_keys ? r.lo + chunk : n_keys;
+  return r;
+}
+
+constexpr int MAX_BINS = 4096;
+
+// Keys per bin of one part of the keys, the part's bounding box; the part's share of the slots is
+// set to empty on the way (each slot is two 16-byte stores, {EMPTY, 0} and {0, 0, 0, 0}).
+__global__ void __launch_bounds__(1024) table_hist(const int4* __restrict__ keys, int64_t n_keys,
+                                                   int32_t bins, int32_t* __restrict__ hist,
+                                                   int32_t* __restrict__ part_box,
+                                                   WcnSlot* __restrict__ slots, int64_t capacity) {
+  __shared__ int s_cnt[MAX_BINS];
   __shared__ int s_mn[16][4];
   __shared__ int s_mx[16][4];
+  const int tid = threadIdx.x, parts = gridDim.x, part = blockIdx.x;
+  for (int b = tid; b < bins; b += 1024) s_cnt[b] = 0;
+  __syncthreads();
   int mn[4] = {INT32_MAX, INT32_MAX, INT32_MAX, INT32_MAX};
   int mx[4] = {INT32_MIN, INT32_MIN, INT32_MIN, INT32_MIN};
-  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
-  constexpr int PER = 8;  // keys a thread has in flight together
-  for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i0 < n_keys; i0 += nthreads * PER) {
+  const PartRange r = part_range(n_keys);
+  const uint32_t bin_mask = (uint32_t)bins - 1u;
+  constexpr int PER = 4;  // keys a thread has in flight together
+  for (int64_t i0 = r.lo + tid; i0 < r.hi; i0 += 1024 * PER) {
     int4 c[PER];
 #pragma unroll
     for (int t = 0; t < PER; ++t) {
-      const int64_t i = i0 + t * nthreads;
-      c[t] = keys[i < n_keys ? i : i0];  // past the end: the thread's first key again
+      const int64_t i = i0 + t * 1024;
+      c[t] = keys[i < r.hi ? i : i0];
     }
 #pragma unroll
     for (int t = 0; t < PER; ++t) {
+      if (i0 + t * 1024 < r.hi) atomicAdd(&s_cnt[bin_of(c[t], bin_mask)], 1);
       mn[0] = min(mn[0], c[t].x); mx[0] = max(mx[0], c[t].x);
       mn[1] = min(mn[1], c[t].y); mx[1] = max(mx[1], c[t].y);
       mn[2] = min(mn[2], c[t].z); mx[2] = max(mx[2], c[t].z);
       mn[3] = min(mn[3], c[t].w); mx[3] = max(mx[3], c[t].w);
     }
+  }
+  {
+    uint4* raw = reinterpret_cast<uint4*>(slots);
+    const int64_t items = 2 * capacity, chunk = (items + parts - 1) / parts;
+    const int64_t lo = (int64_t)part * chunk, hi = lo + chunk < items ? lo + chunk : items;
+    for (int64_t i = lo + tid; i < hi; i += 1024)
+      raw[i] = (i & 1) ? make_uint4(0u, 0u, 0u, 0u) : make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0u, 0u);
   }
 #pragma unroll
   for (int d = 0; d < 4; ++d) {
@@ -76,7 +96,7 @@ __global__ void __launch_bounds__(1024) table_bbox(const int4* __restrict__ keys
       mx[d] = max(mx[d], __shfl_xor(mx[d], s, 64));
     }
   }
-  const int wave = threadIdx.x >> 6;
+  const int wave = tid >> 6;
   if (wcn_lane() == 0) {
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
@@ -85,121 +105,406 @@ __global__ void __launch_bounds__(1024) table_bbox(const int4* __restrict__ keys
     }
   }
   __syncthreads();
-  if (threadIdx.x < 4) {
-    const int d = threadIdx.x;
-    int a = s_mn[0][d], b = s_mx[0][d];
-    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) {
-      a = min(a, s_mn[w][d]);
-      b = max(b, s_mx[w][d]);
+  for (int b = tid; b < bins; b += 1024) hist[(int64_t)b * parts + part] = s_cnt[b];
+  if (tid < 4) {
+    int a = s_mn[0][tid], b = s_mx[0][tid];
+    for (int w = 1; w < 16; ++w) {
+      a = min(a, s_mn[w][tid]);
+      b = max(b, s_mx[w][tid]);
     }
-    atomicMin(&hdr->mn[d], a);
-    atomicMax(&hdr->mx[d], b);
+    part_box[part * 8 + tid] = a;
+    part_box[part * 8 + 4 + tid] = b;
   }
 }
 
-__global__ void __launch_bounds__(256) table_insert(const int4* __restrict__ keys, int64_t n_keys,
-                                                    WcnTableHeader* __restrict__ hdr,
-                                                    WcnSlot* __restrict__ slots, uint32_t cap_mask,
-                                                    int32_t* __restrict__ slot_of) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n_keys) return;
-  const WcnLayout L = wcn_make_layout(hdr);
-  if (!L.ok) {
-    if (i == 0) atomicOr(&hdr->status, WCN_DEV_RANGE);
-    slot_of[i] = -1;
-    return;
+// One wave per bin: hist[bin][0..parts) becomes its exclusive prefix sum, bin_total[bin] its sum.
+// All loads of a column are issued before the first is used (parts <= 256: four per lane).
+__global__ void __launch_bounds__(256) table_colscan(int32_t* __restrict__ hist, int32_t bins,
+                                                     int32_t parts, int32_t* __restrict__ bin_total) {
+  const int lane = wcn_lane(), wave = threadIdx.x >> 6;
+  const int bin = blockIdx.x * 4 + wave;
+  if (bin >= bins) return;
+  int32_t* col = hist + (int64_t)bin * parts;
+  int v[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) v[t] = t * 64 + lane < parts ? col[t * 64 + lane] : 0;
+  int carry = 0;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int incl = wcn_wave_inclusive_sum(v[t]);
+    if (t * 64 + lane < parts) col[t * 64 + lane] = carry + incl - v[t];
+    carry += __shfl(incl, 63, 64);
   }
-  const int4 c = keys[i];
-  uint32_t r[4];
-  wcn_relative(L, c.x, c.y, c.z, c.w, r);  // always inside: the box was built from these keys
-  const unsigned long long key = wcn_block_key(L, r);
-  const uint32_t bit_index = wcn_block_bit(r);
-  const uint32_t bit = 1u << (bit_index & 31u);  // within the 32-bit half of the mask that holds it
-  uint32_t h = wcn_mix(key, cap_mask);
-  int32_t placed = -1;
-  for (int p = 0; p < WCN_MAX_PROBE; ++p) {
-    // cheap pre-read: most keys find their block already present
-    // (a stale EMPTY from the vector cache only costs the CAS below; a non-empty key is final)
-    unsigned long long seen = *reinterpret_cast<const volatile unsigned long long*>(&slots[h].key);
+  if (lane == 0) bin_total[bin] = carry;
+}
+
+// Every key and its row to its place in its bin.  Each workgroup scans the bin totals into bin
+// starts for itself (at most MAX_BINS numbers); workgroup 0 also stores them for the next pass,
+// merges the parts' bounding boxes and writes the header.
+__global__ void __launch_bounds__(1024) table_scatter(const int4* __restrict__ keys, int64_t n_keys,
+                                                      int32_t bins, const int32_t* __restrict__ hist,
+                                                      const int32_t* __restrict__ bin_total,
+                                                      int32_t* __restrict__ bin_start,
+                                                      const int32_t* __restrict__ part_box,
+                                                      WcnTableHeader* __restrict__ hdr,
+                                                      int64_t stats_offset,
+                                                      int4* __restrict__ bin_coords,
+                                                      int32_t* __restrict__ bin_row) {
+  __shared__ int s_cur[MAX_BINS];
+  __shared__ int s_wave[16];
+  const int tid = threadIdx.x, lane = wcn_lane(), wave = tid >> 6;
+  const int parts = gridDim.x, part = blockIdx.x;
+  const PartRange r = part_range(n_keys);
+  constexpr int PER = 4;
+  int4 c[PER];  // the first keys are requested before anything else
+#pragma unroll
+  for (int t = 0; t < PER; ++t) {
+    const int64_t i = r.lo + tid + t * 1024;
+    c[t] = i < r.hi ? keys[i] : make_int4(0, 0, 0, 0);
+  }
+  int v[4], mine[4], sum = 0;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int b = tid * 4 + t;
+    v[t] = b < bins ? bin_total[b] : 0;
+    mine[t] = b < bins ? hist[(int64_t)b * parts + part] : 0;
+    sum += v[t];
+  }
+  const int incl = wcn_wave_inclusive_sum(sum);
+  if (lane == 63) s_wave[wave] = incl;
+  __syncthreads();
+  int run = incl - sum;
+  for (int w = 0; w < wave; ++w) run += s_wave[w];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int b = tid * 4 + t;
+    if (b < bins) {
+      s_cur[b] = run + mine[t];
+      if (part == 0) bin_start[b] = run;
+    }
+    run += v[t];
+  }
+  if (part == 0) {
+    if (tid == 0) bin_start[bins] = (int32_t)n_keys;
+    if (wave == 1) {  // the boxes: lane d + 8 j merges column d of parts j, j + 8, ...
+      const int d = lane & 7;
+      int acc = d < 4 ? INT32_MAX : INT32_MIN;
+      for (int p = lane >> 3; p < parts; p += 8) {
+        const int x = part_box[p * 8 + d];
+        acc = d < 4 ? min(acc, x) : max(acc, x);
+      }
+#pragma unroll
+      for (int s = 8; s < 64; s <<= 1) {
+        const int o = __shfl_xor(acc, s, 64);
+        acc = d < 4 ? min(acc, o) : max(acc, o);
+      }
+      if (lane < 4) hdr->mn[lane] = acc;
+      else if (lane < 8) hdr->mx[lane - 4] = acc;
+      if (lane == 8) {
+        hdr->num_blocks = 0;
+        hdr->status = 0;
+        hdr->total = 0;
+        hdr->num_keys = (int32_t)n_keys;
+        hdr->bins = bins;
+        hdr->stats_offset = stats_offset;
+      }
+    }
+  }
+  __syncthreads();
+  const uint32_t bin_mask = (uint32_t)bins - 1u;
+  for (int64_t i0 = r.lo + tid; i0 < r.hi; i0 += 1024 * PER) {
+    if (i0 != r.lo + tid) {
+#pragma unroll
+      for (int t = 0; t < PER; ++t) {
+        const int64_t i = i0 + t * 1024;
+        c[t] = keys[i < r.hi ? i : i0];
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < PER; ++t) {
+      const int64_t i = i0 + t * 1024;
+      if (i < r.hi) {
+        const int pos = atomicAdd(&s_cur[bin_of(c[t], bin_mask)], 1);
+        bin_coords[pos] = c[t];
+        bin_row[pos] = (int32_t)i;
+      }
+    }
+  }
+}
+
+// One workgroup per bin.  LDS holds an open-addressing table of the bin's blocks: key, occupancy
+// mask, number of entries (keys, duplicates included), later their prefix sums.
+struct BinLds {
+  unsigned long long key[WCN_BIN_SLOTS];
+  unsigned long long mask[WCN_BIN_SLOTS];
+  uint32_t cursor[WCN_BIN_SLOTS];   // entries of the block, then the next free place among them
+  uint32_t base[WCN_BIN_SLOTS];     // voxels of the blocks before this one
+  int32_t where[WCN_BIN_SLOTS];     // the block's slot in the table in memory
+  int32_t low[WCN_BIN_SLOTS];       // lowest row per voxel when keys repeat
+  int32_t part[3][16];
+};
+
+// Entry e of the bin: claims / finds its block in the LDS table, sets its bit, counts itself.
+// Returns the block's place in the LDS table, or -1 if the table is full.
+__device__ __forceinline__ int bin_insert(BinLds* s, unsigned long long key, uint32_t bit) {
+  uint32_t h = wcn_mix(key, WCN_BIN_SLOTS - 1);
+  for (int p = 0; p < WCN_BIN_SLOTS; ++p) {
+    unsigned long long seen = s->key[h];
     if (seen == WCN_EMPTY_KEY) {
-      seen = atomicCAS(&slots[h].key, WCN_EMPTY_KEY, key);
-      if (seen == WCN_EMPTY_KEY) seen = key;  // this thread claimed the slot
+      seen = atomicCAS(&s->key[h], WCN_EMPTY_KEY, key);
+      if (seen == WCN_EMPTY_KEY) seen = key;
     }
     if (seen == key) {
-      // the result of the atomic is not used, so it is issued without waiting for a reply;
-      // repeated keys show up later as fewer set bits than keys
-      uint32_t* half = reinterpret_cast<uint32_t*>(&slots[h].mask) + (bit_index >> 5);
-      atomicOr(half, bit);
-      placed = (int32_t)h;
-      break;
+      atomicOr(&s->mask[h], 1ull << bit);
+      atomicAdd(&s->cursor[h], 1u);
+      return (int)h;
     }
-    h = (h + 1) & cap_mask;
+    h = (h + 1) & (WCN_BIN_SLOTS - 1);
   }
-  if (placed < 0) atomicOr(&hdr->status, WCN_DEV_OVERFLOW);
-  slot_of[i] = placed;
+  return -1;
 }
 
-// base of every occupied slot = running sum of block populations.  A 1024-thread workgroup owns
-// BASE_CHUNKS x 1024 consecutive slots, scans them and takes its share of the running sum with a
-// single atomic (the atomics of all workgroups serialise on one word, so there should be few).
-constexpr int BASE_CHUNKS = 8;
-__global__ void __launch_bounds__(1024) table_base(WcnTableHeader* __restrict__ hdr,
-                                                   WcnSlot* __restrict__ slots, int64_t capacity) {
-  __shared__ int s_wave[BASE_CHUNKS][16];
-  __shared__ int s_occ[16];
-  __shared__ int s_group_base;
-  const int64_t j0 = (int64_t)blockIdx.x * (BASE_CHUNKS * 1024) + threadIdx.x;
-  const int lane = wcn_lane(), wave = threadIdx.x >> 6;
-  int cnt[BASE_CHUNKS], incl[BASE_CHUNKS], occ = 0;
+template <bool WANT_SLOT_OF>
+__global__ void __launch_bounds__(1024) table_bins(WcnTableHeader* __restrict__ hdr,
+                                                   WcnSlot* __restrict__ slots, uint32_t cap_mask,
+                                                   const int32_t* __restrict__ bin_start,
+                                                   const int4* __restrict__ bin_coords,
+                                                   const int32_t* __restrict__ bin_row,
+                                                   int4* __restrict__ order_coords,
+                                                   int32_t* __restrict__ order_row,
+                                                   int32_t* __restrict__ perm,
+                                                   int32_t* __restrict__ slot_of,
+                                                   int32_t* __restrict__ bin_stats) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char bin_smem[];
+  BinLds* s = reinterpret_cast<BinLds*>(bin_smem);
+  const int tid = threadIdx.x, lane = wcn_lane(), wave = tid >> 6;
+  const int lo = bin_start[blockIdx.x], hi = bin_start[blockIdx.x + 1];
+  if (tid == 0) {
+    bin_stats[2 * blockIdx.x] = 0;
+    bin_stats[2 * blockIdx.x + 1] = 0;
+  }
+  if (lo >= hi) return;
+  // A thread keeps its first E entries in registers from the first pass to the last (bins hold
+  // one to two thousand keys: one or two entries per thread); entries beyond that are read again.
+  constexpr int E = 4;
+  int4 c[E];
+  int32_t row[E];
+  int where[E];
 #pragma unroll
-  for (int t = 0; t < BASE_CHUNKS; ++t) {
-    const int64_t j = j0 + (int64_t)t * 1024;
-    cnt[t] = j < capacity ? __popcll(slots[j].mask) : 0;
+  for (int t = 0; t < E; ++t) {
+    const int e = lo + tid + t * 1024;
+    c[t] = bin_coords[e < hi ? e : lo];
+    row[t] = bin_row[e < hi ? e : lo];
+  }
+  const WcnLayout L = wcn_make_layout(hdr);
+  if (!L.ok) {
+    if (tid == 0) atomicOr(&hdr->status, WCN_DEV_RANGE);
+    for (int e = lo + tid; e < hi; e += 1024) {
+      if (WANT_SLOT_OF) slot_of[bin_row[e]] = -1;
+      order_row[e] = bin_row[e];
+      order_coords[e] = bin_coords[e];
+    }
+    return;
+  }
+  for (int h = tid; h < WCN_BIN_SLOTS; h += 1024) {
+    s->key[h] = WCN_EMPTY_KEY;
+    s->mask[h] = 0ull;
+    s->cursor[h] = 0u;
+    s->where[h] = -1;
+  }
+  __syncthreads();
+  // masks and entry counts
+  bool lost = false;
+#pragma unroll
+  for (int t = 0; t < E; ++t) {
+    where[t] = -1;
+    if (lo + tid + t * 1024 < hi) {
+      uint32_t r[4];
+      wcn_relative(L, c[t].x, c[t].y, c[t].z, c[t].w, r);  // always inside: the box was built from these keys
+      where[t] = bin_insert(s, wcn_block_key(L, r), wcn_block_bit(r));
+      lost |= where[t] < 0;
+    }
+  }
+  for (int e = lo + tid + E * 1024; e < hi; e += 1024) {
+    const int4 ce = bin_coords[e];
+    uint32_t r[4];
+    wcn_relative(L, ce.x, ce.y, ce.z, ce.w, r);
+    lost |= bin_insert(s, wcn_block_key(L, r), wcn_block_bit(r)) < 0;
+  }
+  if (lost) atomicOr(&hdr->status, WCN_DEV_OVERFLOW);  // more distinct blocks in this bin than its table holds
+  __syncthreads();
+  // prefix sums over the table's slots, PER consecutive ones per thread: entries and voxels
+  constexpr int PER = WCN_BIN_SLOTS / 1024;
+  uint32_t ne[PER], nv[PER], se = 0, sv = 0;
+#pragma unroll
+  for (int t = 0; t < PER; ++t) {
+    const int h = tid * PER + t;
+    ne[t] = s->cursor[h];
+    nv[t] = (uint32_t)__popcll(s->mask[h]);
+    se += ne[t];
+    sv += nv[t];
+  }
+  const int ie = wcn_wave_inclusive_sum((int)se), iv = wcn_wave_inclusive_sum((int)sv);
+  if (lane == 63) {
+    s->part[0][wave] = ie;
+    s->part[1][wave] = iv;
+  }
+  __syncthreads();
+  int be = 0, bv = 0, total_v = 0;
+  for (int w = 0; w < 16; ++w) {
+    if (w < wave) {
+      be += s->part[0][w];
+      bv += s->part[1][w];
+    }
+    total_v += s->part[1][w];
+  }
+  const bool repeats = total_v != hi - lo;          // some key of this bin came more than once
+  const bool low_in_lds = total_v <= WCN_BIN_SLOTS;  // room for one word per voxel
+  uint32_t re = (uint32_t)(be + ie) - se, rv = (uint32_t)(bv + iv) - sv;
+#pragma unroll
+  for (int t = 0; t < PER; ++t) {
+    const int h = tid * PER + t;
+    s->cursor[h] = re;
+    s->base[h] = rv;
+    re += ne[t];
+    rv += nv[t];
+  }
+  if (repeats) {
+    if (low_in_lds) {
+      for (int j = tid; j < total_v; j += 1024) s->low[j] = INT32_MAX;
+    } else {
+      for (int j = lo + tid; j < lo + total_v; j += 1024) perm[j] = INT32_MAX;
+      __threadfence();
+    }
+  }
+  __syncthreads();
+  // Every block claims a slot of the table in memory: one claimant per block in the whole grid,
+  // so the compare-and-swap only ever meets other blocks' keys.  Slot h of the LDS table goes to
+  // thread h mod 1024: the occupied ones are spread over the threads and their claims overlap.
+  int claimed = 0;
+#pragma unroll
+  for (int t = 0; t < PER; ++t) {
+    const int h = tid + t * 1024;
+    const unsigned long long key = s->key[h];
+    if (key != WCN_EMPTY_KEY) {
+      uint32_t g = wcn_mix(key, cap_mask);
+      int p = 0;
+      for (; p < WCN_MAX_PROBE; ++p) {
+        if (atomicCAS(&slots[g].key, WCN_EMPTY_KEY, key) == WCN_EMPTY_KEY) break;
+        g = (g + 1) & cap_mask;
+      }
+      if (p < WCN_MAX_PROBE) {
+        slots[g].mask = s->mask[h];
+        slots[g].base = lo + (int32_t)s->base[h];
+        if (WANT_SLOT_OF) s->where[h] = (int32_t)g;
+        ++claimed;
+      } else {
+        atomicOr(&hdr->status, WCN_DEV_OVERFLOW);
+      }
+    }
+  }
+  {
+    const int cw = wcn_wave_inclusive_sum(claimed);
+    if (lane == 63) s->part[2][wave] = cw;
+  }
+  // every key to its place in block order; the row of every voxel into perm
+  auto place = [&](const int4 ce, int32_t rw, int h, int e) {
+    if (h < 0) {  // its block did not fit (overflow is flagged): the entry stays where it is
+      order_coords[e] = ce;
+      order_row[e] = rw;
+      if (WANT_SLOT_OF) slot_of[rw] = -1;
+      return;
+    }
+    uint32_t r[4];
+    wcn_relative(L, ce.x, ce.y, ce.z, ce.w, r);
+    const int q = lo + (int)atomicAdd(&s->cursor[h], 1u);
+    order_coords[q] = ce;
+    order_row[q] = rw;
+    const int v = (int)s->base[h] + wcn_rank_below(s->mask[h], wcn_block_bit(r));
+    if (!repeats) perm[lo + v] = rw;
+    else if (low_in_lds) atomicMin(&s->low[v], rw);
+    else atomicMin(&perm[lo + v], rw);
+  };
+#pragma unroll
+  for (int t = 0; t < E; ++t) {
+    const int e = lo + tid + t * 1024;
+    if (e < hi) place(c[t], row[t], where[t], e);
+  }
+  for (int e = lo + tid + E * 1024; e < hi; e += 1024) {
+    const int4 ce = bin_coords[e];
+    uint32_t r[4];
+    wcn_relative(L, ce.x, ce.y, ce.z, ce.w, r);
+    const unsigned long long key = wcn_block_key(L, r);
+    uint32_t h = wcn_mix(key, WCN_BIN_SLOTS - 1);
+    int found = -1;
+    for (int p = 0; p < WCN_BIN_SLOTS && found < 0; ++p) {
+      if (s->key[h] == key) found = (int)h;
+      h = (h + 1) & (WCN_BIN_SLOTS - 1);
+    }
+    place(ce, bin_row[e], found, e);
+  }
+  __syncthreads();
+  if (WANT_SLOT_OF) {  // the claims have landed: the slot of every key
+#pragma unroll
+    for (int t = 0; t < E; ++t) {
+      const int e = lo + tid + t * 1024;
+      if (e < hi && where[t] >= 0) slot_of[row[t]] = s->where[where[t]];
+    }
+    for (int e = lo + tid + E * 1024; e < hi; e += 1024) {
+      const int4 ce = bin_coords[e];
+      uint32_t r[4];
+      wcn_relative(L, ce.x, ce.y, ce.z, ce.w, r);
+      const unsigned long long key = wcn_block_key(L, r);
+      uint32_t h = wcn_mix(key, WCN_BIN_SLOTS - 1);
+      for (int p = 0; p < WCN_BIN_SLOTS; ++p) {
+        if (s->key[h] == key) {
+          slot_of[bin_row[e]] = s->where[h];
+          break;
+        }
+        h = (h + 1) & (WCN_BIN_SLOTS - 1);
+      }
+    }
+  }
+  if (repeats && low_in_lds)
+    for (int j = tid; j < total_v; j += 1024) perm[lo + j] = s->low[j];
+  if (tid == 0) {
+    int blocks = 0;
+    for (int w = 0; w < 16; ++w) blocks += s->part[2][w];
+    bin_stats[2 * blockIdx.x] = total_v;
+    bin_stats[2 * blockIdx.x + 1] = blocks;
+  }
+}
+
+// Sums the bins' voxel and block counts into the header (for the host's status read; the
+// kernel-map builder adds them up itself).
+__global__ void __launch_bounds__(1024) table_sum_stats(WcnTableHeader* __restrict__ hdr) {
+  __shared__ int s_v[16], s_b[16];
+  const int32_t bins = hdr->bins;
+  const int32_t* bin_stats = reinterpret_cast<const int32_t*>(reinterpret_cast<const char*>(hdr) + hdr->stats_offset);
+  int v = 0, b = 0;
+  for (int i = threadIdx.x; i < bins; i += 1024) {
+    v += bin_stats[2 * i];
+    b += bin_stats[2 * i + 1];
   }
 #pragma unroll
-  for (int t = 0; t < BASE_CHUNKS; ++t) {
-    incl[t] = wcn_wave_inclusive_sum(cnt[t]);
-    occ += __popcll(__ballot(cnt[t] > 0));
-    if (lane == 63) s_wave[t][wave] = incl[t];
+  for (int s = 32; s > 0; s >>= 1) {
+    v += __shfl_xor(v, s, 64);
+    b += __shfl_xor(b, s, 64);
   }
-  if (lane == 0) s_occ[wave] = occ;
+  if (wcn_lane() == 0) {
+    s_v[threadIdx.x >> 6] = v;
+    s_b[threadIdx.x >> 6] = b;
+  }
   __syncthreads();
   if (threadIdx.x == 0) {
-    int total = 0, blocks = 0;
-    for (int t = 0; t < BASE_CHUNKS; ++t)
-      for (int w = 0; w < 16; ++w) {
-        const int v = s_wave[t][w];
-        s_wave[t][w] = total;  // exclusive prefix over (chunk, wave)
-        total += v;
-      }
-    for (int w = 0; w < 16; ++w) blocks += s_occ[w];
-    s_group_base = total ? atomicAdd(&hdr->total, total) : 0;
-    if (blocks) atomicAdd(&hdr->num_blocks, blocks);
+    v = b = 0;
+    for (int w = 0; w < 16; ++w) {
+      v += s_v[w];
+      b += s_b[w];
+    }
+    hdr->total = v;
+    hdr->num_blocks = b;
   }
-  __syncthreads();
-#pragma unroll
-  for (int t = 0; t < BASE_CHUNKS; ++t)
-    if (cnt[t] > 0) slots[j0 + (int64_t)t * 1024].base = s_group_base + s_wave[t][wave] + incl[t] - cnt[t];
-}
-
-__global__ void __launch_bounds__(256) table_perm(const int4* __restrict__ keys, int64_t n_keys,
-                                                  const WcnTableHeader* __restrict__ hdr,
-                                                  const WcnSlot* __restrict__ slots,
-                                                  const int32_t* __restrict__ slot_of,
-                                                  int32_t* __restrict__ perm) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n_keys) return;
-  const int32_t h = slot_of[i];
-  if (h < 0) return;
-  const WcnLayout L = wcn_make_layout(hdr);
-  const int4 c = keys[i];
-  uint32_t r[4];
-  wcn_relative(L, c.x, c.y, c.z, c.w, r);
-  const ulonglong2 km = *reinterpret_cast<const ulonglong2*>(&slots[h]);
-  const int32_t pos = slots[h].base + wcn_rank_below(km.y, wcn_block_bit(r));
-  if (pos < 0 || pos >= n_keys) return;
-  // without duplicate keys every position has exactly one writer
-  if (WCN_HAS_DUPLICATES(hdr)) atomicMin(&perm[pos], (int32_t)i); else perm[pos] = (int32_t)i;
 }
 
 __global__ void __launch_bounds__(256) table_query(const WcnTableHeader* __restrict__ hdr,
@@ -237,26 +542,41 @@ inline int grid_for(int64_t n, int block, int cap = 0x7fffffff) {
 
 }  // namespace
 
-// Enqueue the five build kernels.  Shared with the strided-coordinate path.
+// Enqueue the build kernels.  Shared with the strided-coordinate path, which also wants the slot of
+// every key (`want_slot_of`).
 int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView& v,
-                         hipStream_t s) {
+                         bool want_slot_of, hipStream_t s) {
   const uint32_t cap_mask = (uint32_t)(v.capacity - 1);
-  const int64_t clear_items = 2 * v.capacity > n_keys ? 2 * v.capacity : n_keys;
-  hipLaunchKernelGGL(table_clear, dim3(grid_for(clear_items, 256, 4096)), dim3(256), 0, s, v.hdr,
-                     v.slots, v.capacity, v.perm, n_keys);
-  if (n_keys > 0) {
-    hipLaunchKernelGGL(table_bbox, dim3(grid_for(n_keys, 1024 * 8, 128)), dim3(1024), 0, s,
-                       (const int4*)keys, n_keys, v.hdr);
-    hipLaunchKernelGGL(table_insert, dim3(grid_for(n_keys, 256)), dim3(256), 0, s,
-                       (const int4*)keys, n_keys, v.hdr, v.slots, cap_mask, v.slot_of);
-    hipLaunchKernelGGL(table_base, dim3(grid_for(v.capacity, 1024 * BASE_CHUNKS)), dim3(1024), 0, s, v.hdr,
-                       v.slots, v.capacity);
-    hipLaunchKernelGGL(table_perm, dim3(grid_for(n_keys, 256)), dim3(256), 0, s,
-                       (const int4*)keys, n_keys, v.hdr, v.slots, v.slot_of, v.perm);
+  const int4* k4 = (const int4*)keys;
+  hipLaunchKernelGGL(table_hist, dim3(v.parts), dim3(1024), 0, s, k4, n_keys, v.bins, v.hist,
+                     v.part_box, v.slots, v.capacity);
+  hipLaunchKernelGGL(table_colscan, dim3((v.bins + 3) / 4), dim3(256), 0, s, v.hist, v.bins,
+                     v.parts, v.bin_total);
+  hipLaunchKernelGGL(table_scatter, dim3(v.parts), dim3(1024), 0, s, k4, n_keys, v.bins, v.hist,
+                     v.bin_total, v.bin_start, v.part_box, v.hdr,
+                     (int64_t)((const char*)v.bin_stats - (const char*)v.hdr), (int4*)v.bin_coords,
+                     v.bin_row);
+  auto fn = want_slot_of ? table_bins<true> : table_bins<false>;
+  {  // the kernel's LDS exceeds the default limit: lift it once per device and instance
+    static std::mutex mu;
+    static bool allowed[2][64] = {};
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return WCN_ERR_LAUNCH;
+    std::lock_guard<std::mutex> hold(mu);
+    if (!allowed[want_slot_of][device]) {
+      if (hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)sizeof(BinLds)) != hipSuccess)
+        return WCN_ERR_LAUNCH;
+      allowed[want_slot_of][device] = true;
+    }
   }
+  hipLaunchKernelGGL(fn, dim3(v.bins), dim3(1024), sizeof(BinLds), s, v.hdr, v.slots, cap_mask,
+                     v.bin_start, (const int4*)v.bin_coords, v.bin_row, (int4*)v.order_coords,
+                     v.order_row, v.perm, v.slot_of, v.bin_stats);
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }
+
 
 // Host waits are polls (a blocking stream synchronisation wakes the host tens of microseconds
 // late) with an upper bound: WCN_WAIT_LIMIT_MS milliseconds (environment, default 60000), after
@@ -496,7 +816,7 @@ int wcn_table_build(const int32_t* keys, int64_t n_keys, void* table, int64_t ca
   if (n_keys >= (1ll << 31)) return WCN_ERR_INVALID_ARGUMENT;
   WcnTableView v;
   wcn_table_layout(table, n_keys, capacity, &v);
-  return wcn_table_build_impl(keys, n_keys, v, (hipStream_t)stream);
+  return wcn_table_build_impl(keys, n_keys, v, false, (hipStream_t)stream);
 }
 
 int wcn_table_query(const void* table, int64_t n_keys, int64_t capacity, const int32_t* queries,
@@ -517,6 +837,9 @@ int wcn_table_query(const void* table, int64_t n_keys, int64_t capacity, const i
 int wcn_table_read_status(const void* table, int32_t* host_num_blocks, void* stream) {
   if (!table) return WCN_ERR_INVALID_ARGUMENT;
   WcnTableHeader h;
+  hipLaunchKernelGGL(table_sum_stats, dim3(1), dim3(1024), 0, (hipStream_t)stream,
+                     reinterpret_cast<WcnTableHeader*>(const_cast<void*>(table)));
+  WCN_LAUNCH_CHECK();
   if (wcn_read_small(&h, table, sizeof(h), (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
   if (host_num_blocks) *host_num_blocks = h.num_blocks;
   return wcn_table_status_from_bits(h.status);
