@@ -149,6 +149,19 @@ int wcn_kmap_fill(const void* table, int64_t n_keys, int64_t capacity, const int
                   const void* workspace, int64_t pair_capacity, int32_t* in_maps,
                   int32_t* out_maps, void* stream);
 
+/* The map of a coordinate set onto itself (the stride-1 convolution: out_coords are the table's own
+ * keys, in the same rows): the same results as wcn_kmap_count / wcn_kmap_fill with out_coords =
+ * keys and stride 1, from a probe pass that walks the keys in the table's block order, where
+ * neighbours in the list are neighbours in space (the reference probes in row order,
+ * discrete_kernels.cu:264-334).  Kernel sizes 3x3x3 and 5x5x5 (wcn_kmap_self_supported says whether
+ * a size and key count are taken); the workspace is that of wcn_kmap_workspace_bytes(n_keys, K);
+ * wcn_kmap_read_result and wcn_kmap_group_start serve both kinds of call. */
+int wcn_kmap_self_supported(const int32_t host_kernel_size[3], int64_t n_keys);
+int wcn_kmap_count_self(const void* table, int64_t n_keys, int64_t capacity,
+                        const int32_t host_kernel_size[3], void* workspace, void* stream);
+int wcn_kmap_fill_self(int64_t n_keys, const int32_t host_kernel_size[3], const void* workspace,
+                       int64_t pair_capacity, int32_t* in_maps, int32_t* out_maps, void* stream);
+
 /* Device address, inside a kmap workspace, of the (K, ceil(num_out/64)+1) int32 table
  * group_start[k][g] = number of pairs of offset k whose output row is below 64*g (valid after
  * wcn_kmap_count).  The contraction accepts it to skip its own search. */

@@ -116,6 +116,48 @@ def test_kernel_map_bit_exact(oracle, name, gen, ksize, stride):
                           canonical_pairs(ref_in, ref_out_map, ref_off))
 
 
+BLOCK_CASES = [c for c in CASES if all(s == 1 for s in c[3]) and c[2] in ((3, 3, 3), (5, 5, 5))]
+
+
+@pytest.mark.parametrize("name,gen,ksize,stride", BLOCK_CASES, ids=[c[0] for c in BLOCK_CASES])
+def test_kernel_map_probed_block_by_block_bit_exact(oracle, monkeypatch, name, gen, ksize, stride):
+    """The other probe pass for a coordinate set mapped onto itself (WCN_KMAP_PROBE=blocks: hit masks
+    of whole 4x4x4 blocks from ANDs of shifted occupancy masks): the same map, bit for bit in native
+    order, with its group starts; also with repeated input rows (against the row-order probe: among
+    repeated keys the reference's winner is a race, here the lowest row) and with 27 pairs per voxel
+    (more than the emit pass assumes)."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    coords = gen()
+    variants = [(coords, True)]
+    if name == "cloud_k3":
+        rng = np.random.default_rng(5)
+        variants.append((np.concatenate([coords, coords[rng.integers(0, len(coords), 3000)]]), False))
+        cube = np.stack(np.meshgrid(*[np.arange(14)] * 3, indexing="ij"), axis=-1).reshape(-1, 3)
+        variants.append((synthetic.batch_indexed([cube.astype(np.int32) - 5]), True))
+    for c, unique in variants:
+        monkeypatch.setenv("WCN_KMAP_PROBE", "blocks")
+        same = _dev(c)
+        km = generate_kernel_map(same, same, stride, ksize)
+        if unique:
+            ref_in, ref_out_map, ref_off, ref_iden = oracle.kernel_map(c, c, ksize, stride)
+        else:
+            monkeypatch.setenv("WCN_KMAP_PROBE", "rows")
+            other = _dev(c)
+            by_rows = generate_kernel_map(other, other, stride, ksize)
+            ref_in, ref_out_map = by_rows.in_maps.cpu().numpy(), by_rows.out_maps.cpu().numpy()
+            ref_off, ref_iden = by_rows.offsets.numpy().astype(np.int64), by_rows.identity_map_index
+        assert km.identity_map_index == ref_iden
+        assert np.array_equal(km.offsets.numpy().astype(np.int64), ref_off)
+        assert np.array_equal(km.in_maps.cpu().numpy(), ref_in)
+        assert np.array_equal(km.out_maps.cpu().numpy(), ref_out_map)
+        groups, _, (K, M) = km._group_start
+        gs = groups.view(torch.int32).cpu().numpy().reshape(K, -1)
+        bounds = np.arange(0, 64 * (gs.shape[1] - 1), 64)
+        want = np.stack([np.searchsorted(ref_out_map[ref_off[k]:ref_off[k + 1]], bounds) for k in range(K)])
+        assert np.array_equal(gs[:, :-1], want)
+        assert np.array_equal(gs[:, -1], np.diff(ref_off))
+
+
 DILATED = [
     ("k3_d2", (3, 3, 3), (1, 1, 1), (2, 2, 2), None),
     ("k3_d123", (3, 3, 3), (1, 1, 1), (1, 2, 3), None),

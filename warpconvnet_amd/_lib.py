@@ -31,6 +31,9 @@ SIGNATURES = {
     "wcn_kmap_read_result": (ctypes.c_int, [_vp, _i64, _i32, _i64p, _vp]),
     "wcn_kmap_fill": (ctypes.c_int, [_vp, _i64, _i64, _vp, _i64, _i32p, _i32p, _vp, _i64, _vp, _vp,
                                      _vp]),
+    "wcn_kmap_self_supported": (ctypes.c_int, [_i32p, _i64]),
+    "wcn_kmap_count_self": (ctypes.c_int, [_vp, _i64, _i64, _i32p, _vp, _vp]),
+    "wcn_kmap_fill_self": (ctypes.c_int, [_i64, _i32p, _vp, _i64, _vp, _vp, _vp]),
     "wcn_kmap_group_start": (_vp, [_vp, _i64, _i32]),
     "wcn_kmap_last_table_flags": (_i32, []),
     "wcn_stride_unique_workspace_bytes": (_sz, [_i64, _i64]),

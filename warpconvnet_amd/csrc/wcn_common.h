@@ -50,10 +50,13 @@ struct WcnTableView {  // host-computed addresses inside a table workspace
   int32_t* perm;        // n_keys
   int32_t* slot_of;     // n_keys (slot of each key; written on request)
   // The keys in block order: every key once, the keys of one block next to each other, the blocks
-  // of one bin next to each other.  Queries walked in this order meet their neighbours' slots and
-  // `perm` entries in the caches.
-  int32_t* order_coords;  // (n_keys, 4)
+  // of one bin next to each other (bin b owns entries bin_start[b] .. bin_start[b + 1]).
+  int32_t* order_tag;     // n_keys: (index of the entry's block in its bin's block list) << 6 | voxel bit
   int32_t* order_row;     // n_keys: input row of each entry
+  // The blocks of bin b, in the order of its entries: block_list[bin_start[b] + j], j < blocks of
+  // the bin.  key, mask and base as in the table's slot; pad[0] = first entry of the block,
+  // counted from bin_start[b].
+  WcnSlot* block_list;    // n_keys places (a bin has at most as many blocks as keys)
   // build scratch
   int32_t* bin_coords;    // (n_keys, 4) keys grouped by bin
   int32_t* bin_row;       // n_keys
@@ -73,7 +76,7 @@ static inline size_t wcn_align256(size_t x) { return (x + 255) & ~(size_t)255; }
 // Keys are first grouped into bins of one to two thousand (a bin is a hash of the key's 16x16x16-voxel
 // cell, so the 4x4x4 blocks of a cell stay together); the bin count follows the slot count, so a
 // rebuild with more slots also re-deals the bins.
-#define WCN_BIN_SLOTS 4096      // distinct blocks a bin can hold (its table in LDS)
+#define WCN_BIN_SLOTS 2048      // distinct blocks a bin can hold (its table in LDS)
 #define WCN_PART_KEYS 4096      // keys per workgroup of the histogram and scatter passes
 static inline int32_t wcn_table_bins(int64_t capacity) {
   int64_t b = capacity / 2048;
@@ -101,10 +104,12 @@ static inline size_t wcn_table_layout(void* base, int64_t n_keys, int64_t capaci
   off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
   if (v) v->slot_of = (int32_t*)(p + off);
   off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
-  if (v) v->order_coords = (int32_t*)(p + off);
-  off += wcn_align256(sizeof(int32_t) * 4 * (size_t)n_keys);
+  if (v) v->order_tag = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
   if (v) v->order_row = (int32_t*)(p + off);
   off += wcn_align256(sizeof(int32_t) * (size_t)n_keys);
+  if (v) v->block_list = (WcnSlot*)(p + off);
+  off += wcn_align256(sizeof(WcnSlot) * (size_t)n_keys);
   if (v) v->bin_coords = (int32_t*)(p + off);
   off += wcn_align256(sizeof(int32_t) * 4 * (size_t)n_keys);
   if (v) v->bin_row = (int32_t*)(p + off);
@@ -178,14 +183,17 @@ __device__ __forceinline__ uint32_t wcn_block_bit(const uint32_t r[4]) {
   return ((r[1] & 3u) << 4) | ((r[2] & 3u) << 2) | (r[3] & 3u);
 }
 
-// 64-bit finaliser of MurmurHash3: spreads neighbouring block keys over the table.
+// Slot of a block key: the key's two halves folded into one word, then the 32-bit finaliser of
+// MurmurHash3 (neighbouring block keys spread over the table; a third of the instructions of a
+// 64-bit mix, and every probe of the kernel-map passes pays for it).
 __device__ __forceinline__ uint32_t wcn_mix(unsigned long long k, uint32_t cap_mask) {
-  k ^= k >> 33;
-  k *= 0xff51afd7ed558ccdull;
-  k ^= k >> 33;
-  k *= 0xc4ceb9fe1a85ec53ull;
-  k ^= k >> 33;
-  return (uint32_t)k & cap_mask;
+  uint32_t h = (uint32_t)k ^ ((uint32_t)(k >> 32) * 0x9E3779B1u);
+  h ^= h >> 16;
+  h *= 0x85ebca6bu;
+  h ^= h >> 13;
+  h *= 0xc2b2ae35u;
+  h ^= h >> 16;
+  return h & cap_mask;
 }
 
 // Finds the slot of a block key.  Returns its mask (0 if the block is absent) and base.  Both

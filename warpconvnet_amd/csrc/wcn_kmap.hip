@@ -177,7 +177,8 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
   unsigned long long key[8];
   uint32_t hh[8];
   bool need[8];
-  uint4 lo[8], hi[8];
+  uint4 lo[8];
+  int32_t hi[8];  // only the base is needed of a slot's second half: a 4-byte load
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const int dx = e >> 2, dy = (e >> 1) & 1, dz = e & 1;
@@ -190,11 +191,11 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     lo[e] = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0u, 0u);
-    hi[e] = make_uint4(0u, 0u, 0u, 0u);
+    hi[e] = 0;
     if (need[e]) {
       const uint4* raw = reinterpret_cast<const uint4*>(&slots[hh[e]]);
       lo[e] = raw[0];
-      hi[e] = raw[1];
+      hi[e] = slots[hh[e]].base;
     }
   }
 #pragma unroll
@@ -205,7 +206,7 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
       const unsigned long long k0 = ((unsigned long long)lo[e].y << 32) | lo[e].x;
       if (k0 == key[e]) {
         mask = ((unsigned long long)lo[e].w << 32) | lo[e].z;
-        base = (int32_t)hi[e].x;
+        base = hi[e];
       } else if (k0 != WCN_EMPTY_KEY) {  // collision on the first probe: walk on
         mask = wcn_lookup_block_from(slots, cap_mask, key[e], (hh[e] + 1) & cap_mask, 1, &base);
       }
@@ -501,6 +502,462 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
   }
 }
 
+// ---- maps of a coordinate set onto itself (stride 1), probed block by block ----------------------
+// The table build leaves, per bin, the list of its blocks and its keys in block order.  This probe
+// pass walks the blocks: the 64 voxels of a block are tested against a kernel offset with one
+// 64-bit AND of occupancy masks, and the neighbours' slots are fetched once per block instead of
+// once per voxel.  What it finds goes back to row order through two small per-row records: the
+// hit mask of the row (bit k = offset k has a pair) and the place where the found rows are parked.
+// The count and emit passes then run in row order, as the reference's pair order demands.
+struct SelfWorkspace {
+  int64_t* result;      // as KmapWorkspace (same places: the read-result call serves both)
+  int64_t* row_total;
+  int32_t* ticket;
+  int32_t* groups;      // (K+1, G+1): the finished group starts of every offset (written by the emit pass)
+  uint32_t* hm;         // (num_out, words) hit masks per row
+  int32_t* ptr;         // num_out: index into park of the row's first found row
+  int32_t* park;        // (num_out, K) at most: found rows, row by row of a tile, offsets ascending
+  int32_t* chunk;       // (K, C + 1): pairs per offset and chunk of SELF_CHUNK rows, then prefix sums
+  int64_t G, C;
+  int32_t words;
+};
+constexpr int SELF_CHUNK = 256;  // rows per workgroup of the count and emit passes
+
+inline size_t self_layout(void* base, int64_t num_out, int32_t K, SelfWorkspace* w) {
+  char* p = (char*)base;
+  size_t off = 0;
+  const int64_t G = (num_out + 63) / 64, C = (num_out + SELF_CHUNK - 1) / SELF_CHUNK;
+  const int32_t words = (K + 31) / 32;
+  if (w) w->result = (int64_t*)(p + off);
+  off += wcn_align256(sizeof(int64_t) * (size_t)(K + 3));
+  if (w) w->row_total = (int64_t*)(p + off);
+  off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
+  if (w) w->ticket = (int32_t*)(p + off);
+  off += 256;
+  if (w) w->groups = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)(K + 1) * (size_t)(G + 1));
+  if (w) w->hm = (uint32_t*)(p + off);
+  off += wcn_align256(sizeof(uint32_t) * (size_t)words * (size_t)num_out);
+  if (w) w->ptr = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)num_out);
+  if (w) w->park = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)K * (size_t)num_out);
+  if (w) w->chunk = (int32_t*)(p + off);
+  off += wcn_align256(sizeof(int32_t) * (size_t)K * (size_t)(C + 1));
+  if (w) {
+    w->G = G;
+    w->C = C;
+    w->words = words;
+  }
+  return off;
+}
+
+// Occupancy of a 4x4x4 block (bit x * 16 + y * 4 + z) as seen from d voxels further along one
+// axis, |d| <= 2: A is the block itself, B its neighbour block in the direction of d.
+__device__ __forceinline__ unsigned long long shift_z(unsigned long long A, unsigned long long B, int d) {
+  const int s = d > 0 ? d : -d;
+  const bool up = d > 0;
+  const uint32_t nib = up ? ((1u << (4 - s)) - 1u) : (0xFu & ~((1u << s) - 1u));  // z the block itself answers
+  const uint32_t m32 = 0x11111111u * nib;
+  const unsigned long long m = ((unsigned long long)m32 << 32) | m32;
+  const unsigned long long a = up ? A >> s : A << s;
+  const unsigned long long b = up ? B << (4 - s) : B >> (4 - s);
+  return d == 0 ? A : ((a & m) | (b & ~m));
+}
+template <int D>
+__device__ __forceinline__ unsigned long long shift_y(unsigned long long A, unsigned long long B) {
+  if (D == 0) return A;
+  constexpr int S = D > 0 ? D : -D;
+  constexpr unsigned long long M = D > 0 ? 0x0001000100010001ull * ((1u << (16 - 4 * S)) - 1u)
+                                         : 0x0001000100010001ull * (0xFFFFu & ~((1u << (4 * S)) - 1u));
+  return D > 0 ? (((A >> (4 * S)) & M) | ((B << (16 - 4 * S)) & ~M))
+               : (((A << (4 * S)) & M) | ((B >> (16 - 4 * S)) & ~M));
+}
+template <int D>
+__device__ __forceinline__ unsigned long long shift_x(unsigned long long A, unsigned long long B) {
+  if (D == 0) return A;
+  constexpr int S = D > 0 ? D : -D;
+  return D > 0 ? ((A >> (16 * S)) | (B << (64 - 16 * S))) : ((A << (16 * S)) | (B >> (64 - 16 * S)));
+}
+
+// One (dy, dx) pair of hit masks of a block for a fixed dz: Z[i][j] is the z-shifted occupancy of
+// the block column (bx + i - 1, by + j - 1).
+template <int R, int DY, int DX>
+__device__ __forceinline__ void self_hits_xy(const unsigned long long (&Z)[3][3], unsigned long long self,
+                                             int dzi, unsigned long long* __restrict__ out) {
+  constexpr int S = 2 * R + 1;
+  constexpr int J = DY > 0 ? 2 : (DY < 0 ? 0 : 1), I = DX > 0 ? 2 : (DX < 0 ? 0 : 1);
+  const unsigned long long y_here = shift_y<DY>(Z[1][1], Z[1][J]);
+  const unsigned long long y_next = DX == 0 ? 0ull : shift_y<DY>(Z[I][1], Z[I][J]);
+  out[((DX + R) * S + (DY + R)) * S + dzi] = self & shift_x<DX>(y_here, y_next);
+}
+template <int R, int DY>
+__device__ __forceinline__ void self_hits_y(const unsigned long long (&Z)[3][3], unsigned long long self,
+                                            int dzi, unsigned long long* __restrict__ out) {
+  self_hits_xy<R, DY, -1>(Z, self, dzi, out);
+  self_hits_xy<R, DY, 0>(Z, self, dzi, out);
+  self_hits_xy<R, DY, 1>(Z, self, dzi, out);
+  if (R == 2) {
+    self_hits_xy<R, DY, -2>(Z, self, dzi, out);
+    self_hits_xy<R, DY, 2>(Z, self, dzi, out);
+  }
+}
+
+// The probe pass, a workgroup per tile of SELF_TILE consecutive blocks of one bin's block list:
+//   1a. a lane per block: its line of the block list, and which of its 26 neighbour blocks matter
+//       (a neighbour is looked up only if the block has a voxel within R of the face, edge or
+//       corner it lies behind: 9 or 10 of 26 for a block of a surface);
+//   1b. a lane per lookup: the neighbour's slot from the table (mask and base into LDS);
+//   2.  a lane per (block, dz): the hit masks of all (2R+1)^2 offsets with that dz, 64 voxels at
+//       a time, from shifts and ANDs of the occupancy masks;
+//   3.  a lane per entry (key) of the tile: its bit of every hit mask makes the row's hit mask;
+//       the positions of the found rows go into an LDS list, and the rows are fetched from perm
+//       and parked behind one another with a lane per found row.
+constexpr int SELF_TILE = 32;
+constexpr int SELF_LIST = 1024;  // found rows fetched per turn of a workgroup
+template <int R>
+__global__ void __launch_bounds__(256) self_probe(const WcnTableHeader* __restrict__ hdr,
+                                                  const WcnSlot* __restrict__ slots, uint32_t cap_mask,
+                                                  const int32_t* __restrict__ perm,
+                                                  const int32_t* __restrict__ bin_start,
+                                                  const int32_t* __restrict__ bin_stats,
+                                                  const WcnSlot* __restrict__ block_list,
+                                                  const int32_t* __restrict__ order_tag,
+                                                  const int32_t* __restrict__ order_row,
+                                                  uint32_t* __restrict__ hm_out,
+                                                  int32_t* __restrict__ ptr_out,
+                                                  int32_t* __restrict__ park, int32_t* __restrict__ ticket) {
+  constexpr int S = 2 * R + 1, K = S * S * S, WORDS = (K + 31) / 32;
+  __shared__ unsigned long long s_nmask[SELF_TILE][27];
+  __shared__ int32_t s_nbase[SELF_TILE][27];
+  __shared__ unsigned long long s_hit[SELF_TILE][K];
+  __shared__ uint32_t s_coord[SELF_TILE][4];  // batch and block coordinates of every block of the tile
+  __shared__ int32_t s_first[SELF_TILE + 1];  // first entry of every block of the tile, and the end
+  __shared__ int32_t s_wave[4];
+  __shared__ int32_t s_list[SELF_LIST];
+  __shared__ uint16_t s_task[SELF_TILE * 26];  // (block of the tile) << 5 | neighbour: the lookups to make
+  __shared__ int32_t s_tasks;
+  const int tid = threadIdx.x, lane = wcn_lane(), wave = tid >> 6;
+  if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *ticket = 0;
+  const int bin = blockIdx.x;
+  const int lo = bin_start[bin], entries = bin_start[bin + 1] - lo, blocks = bin_stats[2 * bin + 1];
+  const WcnLayout L = wcn_make_layout(hdr);
+  if (!L.ok) return;
+  const uint32_t lim[3] = {L.span[1] >> 2, L.span[2] >> 2, L.span[3] >> 2};
+  for (int j0 = (int)blockIdx.y * SELF_TILE; j0 < blocks; j0 += (int)gridDim.y * SELF_TILE) {
+    const int nblk = blocks - j0 < SELF_TILE ? blocks - j0 : SELF_TILE;
+    // neighbours that are not looked up count as empty
+    for (int idx = tid; idx < SELF_TILE * 27; idx += 256) {
+      const int t = idx / 27, n = idx - t * 27;
+      if (n != 13) {
+        s_nmask[t][n] = 0ull;
+        s_nbase[t][n] = 0;
+      }
+    }
+    // 1a
+    if (wave == 0) {
+      uint32_t wanted = 0;
+      if (lane < nblk) {
+        const uint4* line = reinterpret_cast<const uint4*>(&block_list[lo + j0 + lane]);
+        const uint4 a = line[0], b = line[1];
+        const unsigned long long key = ((unsigned long long)a.y << 32) | a.x;
+        const unsigned long long self = ((unsigned long long)a.w << 32) | a.z;
+        s_nmask[lane][13] = self;
+        s_nbase[lane][13] = (int32_t)b.x;
+        s_first[lane] = (int32_t)b.y;
+        const uint32_t bz = (uint32_t)(key & ((1ull << L.shift[2]) - 1ull));
+        const uint32_t by = (uint32_t)((key >> L.shift[2]) & ((1ull << (L.shift[1] - L.shift[2])) - 1ull));
+        const uint32_t bx = (uint32_t)((key >> L.shift[1]) & ((1ull << (L.shift[0] - L.shift[1])) - 1ull));
+        s_coord[lane][0] = (uint32_t)(key >> L.shift[0]);
+        s_coord[lane][1] = bx;
+        s_coord[lane][2] = by;
+        s_coord[lane][3] = bz;
+        // voxels within R of the low / high end of every axis
+        constexpr unsigned long long XL = (1ull << (16 * R)) - 1ull, XH = ~0ull << (64 - 16 * R);
+        constexpr unsigned long long YL = 0x0001000100010001ull * ((1u << (4 * R)) - 1u);
+        constexpr unsigned long long YH = 0x0001000100010001ull * (0xFFFFu & (0xFFFFu << (16 - 4 * R)));
+        constexpr unsigned long long ZL = 0x1111111111111111ull * ((1u << R) - 1u);
+        constexpr unsigned long long ZH = 0x1111111111111111ull * (0xFu & (0xFu << (4 - R)));
+        const unsigned long long mx[3] = {self & XL, self, self & XH};
+        const bool inx[3] = {bx >= 1u, true, bx + 1u <= lim[0]};
+        const bool iny[3] = {by >= 1u, true, by + 1u <= lim[1]};
+        const bool inz[3] = {bz >= 1u, true, bz + 1u <= lim[2]};
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+          const unsigned long long my[3] = {mx[i] & YL, mx[i], mx[i] & YH};
+#pragma unroll
+          for (int j = 0; j < 3; ++j) {
+            const unsigned long long mz[3] = {my[j] & ZL, my[j], my[j] & ZH};
+#pragma unroll
+            for (int k = 0; k < 3; ++k) {
+              const int n = i * 9 + j * 3 + k;
+              if (n != 13 && mz[k] != 0ull && inx[i] && iny[j] && inz[k]) wanted |= 1u << n;
+            }
+          }
+        }
+      }
+      const int cnt = __popc(wanted);
+      const int incl = wcn_wave_inclusive_sum(cnt);
+      int at = incl - cnt;
+      while (wanted) {
+        const int n = __builtin_ctz(wanted);
+        wanted &= wanted - 1u;
+        s_task[at++] = (uint16_t)((lane << 5) | n);
+      }
+      if (lane == 63) s_tasks = incl;
+      if (lane == 0) s_first[nblk] = j0 + nblk < blocks ? block_list[lo + j0 + nblk].pad[0] : entries;
+    }
+    __syncthreads();
+    // the tile's first round of entries is requested now and used in step 3
+    const int e0 = s_first[0], ne = s_first[nblk] - e0;
+    int32_t tag_ahead = 0, row_ahead = -1;
+    if (tid < ne) {
+      tag_ahead = order_tag[lo + e0 + tid];
+      row_ahead = order_row[lo + e0 + tid];
+    }
+    // 1b
+    const int tasks = s_tasks;
+    for (int i = tid; i < tasks; i += 256) {
+      const int task = s_task[i], t = task >> 5, n = task & 31;
+      const int dx = n / 9 - 1, dy = (n / 3) % 3 - 1, dz = n % 3 - 1;
+      const unsigned long long nkey = ((unsigned long long)s_coord[t][0] << L.shift[0]) |
+                                      ((unsigned long long)(s_coord[t][1] + (uint32_t)dx) << L.shift[1]) |
+                                      ((unsigned long long)(s_coord[t][2] + (uint32_t)dy) << L.shift[2]) |
+                                      (unsigned long long)(s_coord[t][3] + (uint32_t)dz);
+      int32_t base = 0;
+      s_nmask[t][n] = wcn_lookup_block(slots, cap_mask, nkey, &base);
+      s_nbase[t][n] = base;
+    }
+    __syncthreads();
+    // 2
+    for (int idx = tid; idx < nblk * S; idx += 256) {
+      const int t = idx / S, dzi = idx - t * S, dz = dzi - R;
+      const int nz = dz > 0 ? 2 : (dz < 0 ? 0 : 1);
+      unsigned long long Z[3][3];
+#pragma unroll
+      for (int i = 0; i < 3; ++i)
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          Z[i][j] = shift_z(s_nmask[t][i * 9 + j * 3 + 1], s_nmask[t][i * 9 + j * 3 + nz], dz);
+      const unsigned long long self = s_nmask[t][13];
+      unsigned long long* out = &s_hit[t][0];
+      self_hits_y<R, -1>(Z, self, dzi, out);
+      self_hits_y<R, 0>(Z, self, dzi, out);
+      self_hits_y<R, 1>(Z, self, dzi, out);
+      if (R == 2) {
+        self_hits_y<R, -2>(Z, self, dzi, out);
+        self_hits_y<R, 2>(Z, self, dzi, out);
+      }
+    }
+    __syncthreads();
+    // 3
+    int run = 0;  // found rows parked so far (the same in every thread)
+    for (int i0 = 0; i0 < ne; i0 += 256) {
+      const int i = i0 + tid;
+      const bool live = i < ne;
+      int32_t tag = tag_ahead, m = row_ahead;
+      if (live && i0 > 0) {
+        tag = order_tag[lo + e0 + i];
+        m = order_row[lo + e0 + i];
+      }
+      const int t = (tag >> 6) - j0;
+      const uint32_t bit = (uint32_t)tag & 63u;
+      const bool known = live && t >= 0 && t < nblk;  // an entry whose block overflowed the table's build has no tag
+      uint32_t hm[WORDS];
+#pragma unroll
+      for (int w = 0; w < WORDS; ++w) hm[w] = 0;
+      if (known) {
+        const uint32_t* half = reinterpret_cast<const uint32_t*>(&s_hit[t][0]) + (bit >> 5);
+#pragma unroll
+        for (int k = 0; k < K; ++k) hm[k >> 5] |= ((half[2 * k] >> (bit & 31u)) & 1u) << (k & 31);
+      }
+      int cnt = 0;
+#pragma unroll
+      for (int w = 0; w < WORDS; ++w) cnt += __popc(hm[w]);
+      const int incl = wcn_wave_inclusive_sum(cnt);
+      if (lane == 63) s_wave[wave] = incl;
+      __syncthreads();
+      int before = run + incl - cnt, all = 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        if (w < wave) before += s_wave[w];
+        all += s_wave[w];
+      }
+      run += all;
+      const int64_t mine = (int64_t)(lo + e0) * K + before;  // the row's place in the tile's piece of park
+      if (live) {
+#pragma unroll
+        for (int w = 0; w < WORDS; ++w) hm_out[(int64_t)m * WORDS + w] = hm[w];
+        ptr_out[m] = (int32_t)mine;
+      }
+      // The positions in perm of this round's found rows go into an LDS list, in the order of
+      // their places in park; the rows are then fetched and parked with a lane per found row
+      // (independent loads, coalesced stores).  The list holds SELF_LIST positions at a time.
+      const int x = (int)(bit >> 4), y = (int)((bit >> 2) & 3u), z = (int)(bit & 3u);
+      const int64_t round_base = (int64_t)(lo + e0) * K + (run - all);
+      const int first = before - (run - all);  // this row's first place in the round's list
+      for (int win = 0; win < all; win += SELF_LIST) {
+        int done = 0;
+#pragma unroll
+        for (int w = 0; w < WORDS; ++w) {
+          uint32_t rest = hm[w];
+          while (rest) {
+            const int k = 32 * w + __builtin_ctz(rest);
+            rest &= rest - 1u;
+            const int at = first + done - win;
+            ++done;
+            if (at < 0 || at >= SELF_LIST) continue;
+            const int ax = x + k / (S * S) - R, ay = y + (k / S) % S - R, az = z + k % S - R;
+            const int n = ((ax >> 2) + 1) * 9 + ((ay >> 2) + 1) * 3 + (az >> 2) + 1;
+            const uint32_t nbit = (uint32_t)(((ax & 3) << 4) | ((ay & 3) << 2) | (az & 3));
+            s_list[at] = s_nbase[t][n] + wcn_rank_below(s_nmask[t][n], nbit);
+          }
+        }
+        __syncthreads();
+        const int have = all - win < SELF_LIST ? all - win : SELF_LIST;
+        for (int h0 = 0; h0 < have; h0 += 4 * 256) {
+          int32_t got[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int h = h0 + u * 256 + tid;
+            got[u] = h < have ? perm[s_list[h]] : 0;
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int h = h0 + u * 256 + tid;
+            if (h < have) park[round_base + win + h] = got[u];
+          }
+        }
+        __syncthreads();  // the list (and s_wave) are written again
+      }
+      if (all == 0) __syncthreads();
+    }
+    __syncthreads();  // the tile's tables are rewritten by the next tile
+  }
+}
+
+// Row order again: pairs per offset in every chunk of SELF_CHUNK rows.
+template <int K>
+__global__ void __launch_bounds__(SELF_CHUNK) self_count(const uint32_t* __restrict__ hm, int64_t num_out,
+                                                         int32_t* __restrict__ chunk_count, int64_t C) {
+  constexpr int WORDS = (K + 31) / 32, WAVES = SELF_CHUNK / 64;
+  __shared__ int s_cnt[WAVES][K];
+  const int tid = threadIdx.x, lane = wcn_lane(), wave = tid >> 6;
+  const int64_t m = (int64_t)blockIdx.x * SELF_CHUNK + tid;
+  uint32_t h[WORDS];
+#pragma unroll
+  for (int w = 0; w < WORDS; ++w) h[w] = m < num_out ? hm[m * WORDS + w] : 0u;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const int n = __popcll(__ballot((h[k >> 5] >> (k & 31)) & 1u));
+    if (lane == 0) s_cnt[wave][k] = n;
+  }
+  __syncthreads();
+  for (int k = tid; k < K; k += SELF_CHUNK) {
+    int n = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) n += s_cnt[w][k];
+    chunk_count[(int64_t)k * (C + 1) + blockIdx.x] = n;
+  }
+}
+
+// Row order, a lane per PAIR.  A wave's pairs are numbered offset by offset and, inside an offset,
+// by lane; pair number q finds its offset by binary search over the running counts, its rank
+// there, from rank and the offset's lane mask its row, and from the row's hit mask the place of the
+// found row among that row's parked rows.
+template <int K>
+__global__ void __launch_bounds__(SELF_CHUNK) self_emit(const uint32_t* __restrict__ hm,
+                                                        const int32_t* __restrict__ ptr,
+                                                        const int32_t* __restrict__ park,
+                                                        const int32_t* __restrict__ chunk_start,
+                                                        const int64_t* __restrict__ offsets,
+                                                        int64_t num_out, int64_t G, int64_t C,
+                                                        int64_t pair_capacity,
+                                                        int32_t* __restrict__ groups,
+                                                        int32_t* __restrict__ in_maps,
+                                                        int32_t* __restrict__ out_maps) {
+  constexpr int WORDS = (K + 31) / 32, WAVES = SELF_CHUNK / 64;
+  __shared__ unsigned long long s_hits[WAVES][K];
+  __shared__ int s_incl[WAVES][K];      // pairs of the wave in offsets 0..k
+  __shared__ int s_start[WAVES][K];     // pairs of offset k below the wave's first row
+  __shared__ uint32_t s_hm[WAVES][64][WORDS];
+  __shared__ int32_t s_ptr[WAVES][64];
+  // see kmap_emit; the group starts are written whatever the room for pairs (the caller keeps them)
+  if (offsets[K + 1] != 0) return;
+  const bool room = offsets[K] <= pair_capacity;
+  const int tid = threadIdx.x, lane = wcn_lane(), wave = tid >> 6;
+  const int64_t m = (int64_t)blockIdx.x * SELF_CHUNK + tid;
+  const int64_t group = m >> 6;
+  uint32_t h[WORDS];
+#pragma unroll
+  for (int w = 0; w < WORDS; ++w) {
+    h[w] = m < num_out ? hm[m * WORDS + w] : 0u;
+    s_hm[wave][lane][w] = h[w];
+  }
+  s_ptr[wave][lane] = m < num_out ? ptr[m] : 0;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const unsigned long long b = __ballot((h[k >> 5] >> (k & 31)) & 1u);
+    if (lane == 0) s_hits[wave][k] = b;
+  }
+  __syncthreads();
+  // per offset: pairs of the waves before this one (thread k of the workgroup)
+  for (int k = tid; k < K; k += SELF_CHUNK) {
+    int run = chunk_start[(int64_t)k * (C + 1) + blockIdx.x];
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      s_start[w][k] = run;
+      const int64_t g = (int64_t)blockIdx.x * WAVES + w;
+      if (g < G) groups[(int64_t)k * (G + 1) + g] = run;
+      run += __popcll(s_hits[w][k]);
+    }
+    if (blockIdx.x == gridDim.x - 1) groups[(int64_t)k * (G + 1) + G] = run;  // the offset's total
+  }
+  __syncthreads();
+  if (group >= G || !room) return;
+  // running counts over the offsets of this wave (lane j sums offsets j, j + 64)
+  {
+    int carry = 0;
+#pragma unroll
+    for (int k0 = 0; k0 < K; k0 += 64) {
+      const int k = k0 + lane;
+      const int n = k < K ? __popcll(s_hits[wave][k]) : 0;
+      const int incl = wcn_wave_inclusive_sum(n);
+      if (k < K) s_incl[wave][k] = carry + incl;
+      carry += __shfl(incl, 63, 64);
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int total = s_incl[wave][K - 1];
+  for (int q0 = 0; q0 < total; q0 += 64) {
+    const int q = q0 + lane;
+    if (q >= total) continue;
+    // first offset whose running count exceeds q
+    int lo = 0, hi = K - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (s_incl[wave][mid] <= q) lo = mid + 1; else hi = mid;
+    }
+    const int k = lo;
+    const unsigned long long hk = s_hits[wave][k];
+    const int rank = q - (s_incl[wave][k] - __popcll(hk));
+    const int t = kmap_nth_set_bit(hk, rank);  // the lane (row) of this pair
+    // the found row is the j-th parked row of row t, j = hits of that row in the offsets below k
+    int j = 0;
+#pragma unroll
+    for (int w = 0; w < WORDS; ++w) {
+      const uint32_t word = s_hm[wave][t][w];
+      const int kw = k - 32 * w;
+      j += kw >= 32 ? __popc(word) : (kw > 0 ? __popc(word & ((1u << kw) - 1u)) : 0);
+    }
+    const int64_t dst = offsets[k] + s_start[wave][k] + rank;
+    in_maps[dst] = park[s_ptr[wave][t] + j];
+    out_maps[dst] = (int32_t)(group * 64 + t);
+  }
+}
+
 bool make_geom(const int32_t ks[3], const int32_t st[3], const int32_t* dil, const int32_t* centre,
                KmapGeom* g) {
   if (!ks || !st) return false;
@@ -670,7 +1127,9 @@ extern "C" {
 
 size_t wcn_kmap_workspace_bytes(int64_t num_out, int32_t num_offsets) {
   if (num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS) return 0;
-  return kmap_layout(nullptr, num_out, num_offsets, nullptr);
+  const size_t a = kmap_layout(nullptr, num_out, num_offsets, nullptr);
+  const size_t b = self_layout(nullptr, num_out, num_offsets, nullptr);
+  return a > b ? a : b;
 }
 
 static int kmap_count_impl(const void* table, int64_t n_keys, int64_t capacity, const int32_t* out_coords,
@@ -729,6 +1188,81 @@ int wcn_kmap_count_dilated(const void* table, int64_t n_keys, int64_t capacity, 
   if (!host_dilation || !host_centre) return WCN_ERR_INVALID_ARGUMENT;
   return kmap_count_impl(table, n_keys, capacity, out_coords, num_out, host_kernel_size, host_stride,
                          host_dilation, host_centre, workspace, stream);
+}
+
+static bool self_size(const int32_t ks[3], int32_t* K) {
+  if (!ks) return false;
+  if (ks[0] == 3 && ks[1] == 3 && ks[2] == 3) { *K = 27; return true; }
+  if (ks[0] == 5 && ks[1] == 5 && ks[2] == 5) { *K = 125; return true; }
+  return false;
+}
+
+int wcn_kmap_self_supported(const int32_t host_kernel_size[3], int64_t n_keys) {
+  int32_t K = 0;
+  return self_size(host_kernel_size, &K) && n_keys > 0 && n_keys * (int64_t)K < (1ll << 31);
+}
+
+int wcn_kmap_count_self(const void* table, int64_t n_keys, int64_t capacity,
+                        const int32_t host_kernel_size[3], void* workspace, void* stream) {
+  int32_t K = 0;
+  if (!self_size(host_kernel_size, &K) || !table_args_ok(table, n_keys, capacity) || !workspace ||
+      n_keys <= 0 || n_keys * (int64_t)K >= (1ll << 31))
+    return WCN_ERR_INVALID_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  WcnTableView v;
+  wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
+  SelfWorkspace w;
+  self_layout(workspace, n_keys, K, &w);
+  const uint32_t cap_mask = (uint32_t)(capacity - 1);
+  // a bin of the usual size has about ten tiles; bins with more are walked in turns
+  const dim3 pgrid((unsigned)v.bins, 8), cgrid((unsigned)w.C);
+  if (K == 27) {
+    hipLaunchKernelGGL(self_probe<1>, pgrid, dim3(256), 0, s, v.hdr, v.slots, cap_mask, v.perm, v.bin_start,
+                       v.bin_stats, v.block_list, v.order_tag, v.order_row, w.hm, w.ptr, w.park, w.ticket);
+    hipLaunchKernelGGL(self_count<27>, cgrid, dim3(SELF_CHUNK), 0, s, w.hm, n_keys, w.chunk, w.C);
+  } else {
+    hipLaunchKernelGGL(self_probe<2>, pgrid, dim3(256), 0, s, v.hdr, v.slots, cap_mask, v.perm, v.bin_start,
+                       v.bin_stats, v.block_list, v.order_tag, v.order_row, w.hm, w.ptr, w.park, w.ticket);
+    hipLaunchKernelGGL(self_count<125>, cgrid, dim3(SELF_CHUNK), 0, s, w.hm, n_keys, w.chunk, w.C);
+  }
+  int64_t* box = nullptr;
+  int64_t sequence = 0;
+  if (wcn_mailbox_begin(&box, &sequence) != WCN_OK) {  // no mailbox: a copy command instead
+    box = nullptr;
+    sequence = 0;
+  }
+  g_pending_sequence = sequence;
+  g_pending_result = w.result;
+  const KmapFinish fin = {w.result, w.ticket, v.hdr, K, box, sequence};
+  hipLaunchKernelGGL(kmap_scan_rows, dim3(K), dim3(1024), 0, s, w.chunk, w.C, w.row_total, fin);
+  WCN_LAUNCH_CHECK();
+  if (box) {
+    if (wcn_mailbox_mark(s) != WCN_OK) return WCN_ERR_LAUNCH;
+  } else if (wcn_read_early_begin(w.result, sizeof(int64_t) * (size_t)(K + 3), s) != WCN_OK) {
+    return WCN_ERR_LAUNCH;
+  }
+  return WCN_OK;
+}
+
+int wcn_kmap_fill_self(int64_t n_keys, const int32_t host_kernel_size[3], const void* workspace,
+                       int64_t pair_capacity, int32_t* in_maps, int32_t* out_maps, void* stream) {
+  int32_t K = 0;
+  if (!self_size(host_kernel_size, &K) || !workspace || n_keys <= 0 || pair_capacity < 0 ||
+      n_keys * (int64_t)K >= (1ll << 31) || !in_maps || !out_maps)
+    return WCN_ERR_INVALID_ARGUMENT;
+  SelfWorkspace w;
+  self_layout(const_cast<void*>(workspace), n_keys, K, &w);
+  const int64_t* offsets = (const int64_t*)w.result;
+  const dim3 grid((unsigned)w.C), block(SELF_CHUNK);
+  if (K == 27) {
+    hipLaunchKernelGGL(self_emit<27>, grid, block, 0, (hipStream_t)stream, w.hm, w.ptr, w.park, w.chunk,
+                       offsets, n_keys, w.G, w.C, pair_capacity, w.groups, in_maps, out_maps);
+  } else {
+    hipLaunchKernelGGL(self_emit<125>, grid, block, 0, (hipStream_t)stream, w.hm, w.ptr, w.park, w.chunk,
+                       offsets, n_keys, w.G, w.C, pair_capacity, w.groups, in_maps, out_maps);
+  }
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
 }
 
 int32_t wcn_kmap_last_table_flags(void) { return g_last_table_flags; }

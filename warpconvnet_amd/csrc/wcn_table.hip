@@ -241,6 +241,7 @@ struct BinLds {
   uint32_t base[WCN_BIN_SLOTS];     // voxels of the blocks before this one
   int32_t where[WCN_BIN_SLOTS];     // the block's slot in the table in memory
   int32_t low[WCN_BIN_SLOTS];       // lowest row per voxel when keys repeat
+  int32_t index[WCN_BIN_SLOTS];     // the block's number in the bin's block list
   int32_t part[3][16];
 };
 
@@ -270,8 +271,9 @@ __global__ void __launch_bounds__(1024) table_bins(WcnTableHeader* __restrict__ 
                                                    const int32_t* __restrict__ bin_start,
                                                    const int4* __restrict__ bin_coords,
                                                    const int32_t* __restrict__ bin_row,
-                                                   int4* __restrict__ order_coords,
+                                                   int32_t* __restrict__ order_tag,
                                                    int32_t* __restrict__ order_row,
+                                                   WcnSlot* __restrict__ block_list,
                                                    int32_t* __restrict__ perm,
                                                    int32_t* __restrict__ slot_of,
                                                    int32_t* __restrict__ bin_stats) {
@@ -302,7 +304,7 @@ __global__ void __launch_bounds__(1024) table_bins(WcnTableHeader* __restrict__ 
     for (int e = lo + tid; e < hi; e += 1024) {
       if (WANT_SLOT_OF) slot_of[bin_row[e]] = -1;
       order_row[e] = bin_row[e];
-      order_coords[e] = bin_coords[e];
+      order_tag[e] = 0;
     }
     return;
   }
@@ -333,42 +335,79 @@ __global__ void __launch_bounds__(1024) table_bins(WcnTableHeader* __restrict__ 
   }
   if (lost) atomicOr(&hdr->status, WCN_DEV_OVERFLOW);  // more distinct blocks in this bin than its table holds
   __syncthreads();
-  // prefix sums over the table's slots, PER consecutive ones per thread: entries and voxels
+  // Prefix sums over the table's slots, entries and voxels.  Thread t owns slots t, t + 1024, ...
+  // and counts them as neighbours in the order of the sums (any fixed order will do, and this one
+  // reads LDS without bank conflicts and spreads the occupied slots over the threads).
   constexpr int PER = WCN_BIN_SLOTS / 1024;
-  uint32_t ne[PER], nv[PER], se = 0, sv = 0;
+  uint32_t ne[PER], nv[PER], se = 0, sv = 0, sb = 0;
+  unsigned long long bkey[PER], bmask[PER];
 #pragma unroll
   for (int t = 0; t < PER; ++t) {
-    const int h = tid * PER + t;
+    const int h = tid + t * 1024;
+    bkey[t] = s->key[h];
+    bmask[t] = s->mask[h];
     ne[t] = s->cursor[h];
-    nv[t] = (uint32_t)__popcll(s->mask[h]);
+    nv[t] = (uint32_t)__popcll(bmask[t]);
     se += ne[t];
     sv += nv[t];
+    sb += bkey[t] != WCN_EMPTY_KEY ? 1u : 0u;
   }
   const int ie = wcn_wave_inclusive_sum((int)se), iv = wcn_wave_inclusive_sum((int)sv);
+  const int ib = wcn_wave_inclusive_sum((int)sb);
   if (lane == 63) {
     s->part[0][wave] = ie;
     s->part[1][wave] = iv;
+    s->part[2][wave] = ib;
   }
   __syncthreads();
-  int be = 0, bv = 0, total_v = 0;
+  int be = 0, bv = 0, bb = 0, total_v = 0, total_b = 0;
   for (int w = 0; w < 16; ++w) {
     if (w < wave) {
       be += s->part[0][w];
       bv += s->part[1][w];
+      bb += s->part[2][w];
     }
     total_v += s->part[1][w];
+    total_b += s->part[2][w];
   }
   const bool repeats = total_v != hi - lo;          // some key of this bin came more than once
   const bool low_in_lds = total_v <= WCN_BIN_SLOTS;  // room for one word per voxel
   uint32_t re = (uint32_t)(be + ie) - se, rv = (uint32_t)(bv + iv) - sv;
+  int rb = bb + ib - (int)sb;
+  // Every block claims a slot of the table in memory: one claimant per block in the whole grid,
+  // so the compare-and-swap only ever meets other blocks' keys.
+  int claimed = 0;
 #pragma unroll
   for (int t = 0; t < PER; ++t) {
-    const int h = tid * PER + t;
+    const int h = tid + t * 1024;
     s->cursor[h] = re;
     s->base[h] = rv;
+    if (bkey[t] != WCN_EMPTY_KEY) {
+      uint32_t g = wcn_mix(bkey[t], cap_mask);
+      int p = 0;
+      for (; p < WCN_MAX_PROBE; ++p) {
+        if (atomicCAS(&slots[g].key, WCN_EMPTY_KEY, bkey[t]) == WCN_EMPTY_KEY) break;
+        g = (g + 1) & cap_mask;
+      }
+      if (p < WCN_MAX_PROBE) {
+        slots[g].mask = bmask[t];
+        slots[g].base = lo + (int32_t)rv;
+        if (WANT_SLOT_OF) s->where[h] = (int32_t)g;
+        ++claimed;
+      } else {
+        atomicOr(&hdr->status, WCN_DEV_OVERFLOW);
+      }
+      // the block's line of the bin's block list (two 16-byte stores)
+      uint4* line = reinterpret_cast<uint4*>(&block_list[lo + rb]);
+      line[0] = make_uint4((uint32_t)bkey[t], (uint32_t)(bkey[t] >> 32), (uint32_t)bmask[t], (uint32_t)(bmask[t] >> 32));
+      line[1] = make_uint4((uint32_t)(lo + (int32_t)rv), re, 0u, 0u);
+      s->index[h] = rb;
+      ++rb;
+    }
     re += ne[t];
     rv += nv[t];
   }
+  (void)claimed;
   if (repeats) {
     if (low_in_lds) {
       for (int j = tid; j < total_v; j += 1024) s->low[j] = INT32_MAX;
@@ -378,49 +417,21 @@ __global__ void __launch_bounds__(1024) table_bins(WcnTableHeader* __restrict__ 
     }
   }
   __syncthreads();
-  // Every block claims a slot of the table in memory: one claimant per block in the whole grid,
-  // so the compare-and-swap only ever meets other blocks' keys.  Slot h of the LDS table goes to
-  // thread h mod 1024: the occupied ones are spread over the threads and their claims overlap.
-  int claimed = 0;
-#pragma unroll
-  for (int t = 0; t < PER; ++t) {
-    const int h = tid + t * 1024;
-    const unsigned long long key = s->key[h];
-    if (key != WCN_EMPTY_KEY) {
-      uint32_t g = wcn_mix(key, cap_mask);
-      int p = 0;
-      for (; p < WCN_MAX_PROBE; ++p) {
-        if (atomicCAS(&slots[g].key, WCN_EMPTY_KEY, key) == WCN_EMPTY_KEY) break;
-        g = (g + 1) & cap_mask;
-      }
-      if (p < WCN_MAX_PROBE) {
-        slots[g].mask = s->mask[h];
-        slots[g].base = lo + (int32_t)s->base[h];
-        if (WANT_SLOT_OF) s->where[h] = (int32_t)g;
-        ++claimed;
-      } else {
-        atomicOr(&hdr->status, WCN_DEV_OVERFLOW);
-      }
-    }
-  }
-  {
-    const int cw = wcn_wave_inclusive_sum(claimed);
-    if (lane == 63) s->part[2][wave] = cw;
-  }
   // every key to its place in block order; the row of every voxel into perm
   auto place = [&](const int4 ce, int32_t rw, int h, int e) {
     if (h < 0) {  // its block did not fit (overflow is flagged): the entry stays where it is
-      order_coords[e] = ce;
+      order_tag[e] = 0;
       order_row[e] = rw;
       if (WANT_SLOT_OF) slot_of[rw] = -1;
       return;
     }
     uint32_t r[4];
     wcn_relative(L, ce.x, ce.y, ce.z, ce.w, r);
-    const int q = lo + (int)atomicAdd(&s->cursor[h], 1u);
-    order_coords[q] = ce;
-    order_row[q] = rw;
     const int v = (int)s->base[h] + wcn_rank_below(s->mask[h], wcn_block_bit(r));
+    // without repeated keys the entries of a block are its voxels: block order is perm's order
+    const int q = lo + (repeats ? (int)atomicAdd(&s->cursor[h], 1u) : v);
+    order_tag[q] = (s->index[h] << 6) | (int32_t)wcn_block_bit(r);
+    order_row[q] = rw;
     if (!repeats) perm[lo + v] = rw;
     else if (low_in_lds) atomicMin(&s->low[v], rw);
     else atomicMin(&perm[lo + v], rw);
@@ -468,10 +479,8 @@ __global__ void __launch_bounds__(1024) table_bins(WcnTableHeader* __restrict__ 
   if (repeats && low_in_lds)
     for (int j = tid; j < total_v; j += 1024) perm[lo + j] = s->low[j];
   if (tid == 0) {
-    int blocks = 0;
-    for (int w = 0; w < 16; ++w) blocks += s->part[2][w];
     bin_stats[2 * blockIdx.x] = total_v;
-    bin_stats[2 * blockIdx.x + 1] = blocks;
+    bin_stats[2 * blockIdx.x + 1] = total_b;
   }
 }
 
@@ -571,8 +580,8 @@ int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView
     }
   }
   hipLaunchKernelGGL(fn, dim3(v.bins), dim3(1024), sizeof(BinLds), s, v.hdr, v.slots, cap_mask,
-                     v.bin_start, (const int4*)v.bin_coords, v.bin_row, (int4*)v.order_coords,
-                     v.order_row, v.perm, v.slot_of, v.bin_stats);
+                     v.bin_start, (const int4*)v.bin_coords, v.bin_row, v.order_tag, v.order_row,
+                     v.block_list, v.perm, v.slot_of, v.bin_stats);
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }

@@ -12,6 +12,7 @@ where the reference waits five times and round-trips a dense (K, M) table throug
 (torch_discrete.py:80-157,301-337).
 """
 import ctypes
+import os
 from typing import Literal, Optional, Sequence, Tuple
 
 import numpy as np
@@ -80,9 +81,29 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     assumed = min(K * M, max(8 * M, 1 << 16))
     in_buf = torch.empty(assumed, dtype=torch.int32, device=device)
     out_buf = torch.empty(assumed, dtype=torch.int32, device=device)
+    # A coordinate set mapped onto itself can also be probed block by block (WCN_KMAP_PROBE=blocks:
+    # the 64 voxels of a block tested against an offset with one AND of occupancy masks, neighbour
+    # slots fetched once per block).  Same results; measured a little slower than the row-order
+    # probe on the benchmark's scenes, so it is not the default.
+    onto_itself = (os.environ.get("WCN_KMAP_PROBE") == "blocks"
+                   and dilation is None and all(int(v) == 1 for v in stride)
+                   and out4.data_ptr() == table._keys4.data_ptr() and M == table._keys4.shape[0]
+                   and bool(L.wcn_kmap_self_supported(ks, M)))
+
+    def fill(capacity, ins, outs):
+        if onto_itself:
+            check(L.wcn_kmap_fill_self(M, ks, ptr(ws), capacity, ptr(ins), ptr(outs), stream_ptr(device)),
+                  "wcn_kmap_fill_self")
+        else:
+            check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), capacity,
+                                  ptr(ins), ptr(outs), stream_ptr(device)), "wcn_kmap_fill")
+
     while True:
         raw, n_keys, slots = table._raw()
-        if dilation is None:
+        if onto_itself:
+            check(L.wcn_kmap_count_self(ptr(raw), n_keys, slots, ks, ptr(ws), stream_ptr(device)),
+                  "wcn_kmap_count_self")
+        elif dilation is None:
             check(L.wcn_kmap_count(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws),
                                    stream_ptr(device)), "wcn_kmap_count")
         else:
@@ -90,8 +111,7 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
                                            int3(_pad_kernel_args(dilation, 1)),
                                            int3(_pad_kernel_args(centres, 0)), ptr(ws),
                                            stream_ptr(device)), "wcn_kmap_count_dilated")
-        check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), assumed,
-                              ptr(in_buf), ptr(out_buf), stream_ptr(device)), "wcn_kmap_fill")
+        fill(assumed, in_buf, out_buf)
         # By-product the contraction reuses: the per-64-row group starts of every offset, (K, G + 1)
         # int32, final once the count call's kernels have run.  Only this table is kept with the
         # map (a copy of about K * M / 16 bytes; the workspace, whose probe results are K * M * 4
@@ -115,8 +135,7 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     else:
         in_maps = torch.empty(total, dtype=torch.int32, device=device)
         out_maps = torch.empty(total, dtype=torch.int32, device=device)
-        check(L.wcn_kmap_fill(ptr(raw), n_keys, slots, ptr(out4), M, ks, st, ptr(ws), total,
-                              ptr(in_maps), ptr(out_maps), stream_ptr(device)), "wcn_kmap_fill")
+        fill(total, in_maps, out_maps)
     offsets = offsets64.to(torch.int32)
     result = IntSearchResult(in_maps, out_maps, offsets, identity_map_index=identity_map_index)
     result._host_offsets = host_offsets  # the contraction passes them on as they are
