@@ -43,3 +43,32 @@ def kaiming_weight(K, c_in, c_out, seed=0, dtype=torch.float32):
 def normal_features(n, c, seed=0, dtype=torch.float32):
     g = torch.Generator().manual_seed(seed + 1)
     return torch.randn(n, c, generator=g).to(dtype)
+
+
+def oracle_kernel_map_by_item(oracle, in_coords, out_coords, kernel_size, stride=(1, 1, 1), threads=16):
+    """The C oracle's kernel map of batch-sorted coordinates, one batch item per host thread (a pair
+    never crosses items; the C code releases the interpreter lock), merged into one map in the
+    reference's order: offsets in k order, ascending output row inside an offset."""
+    from concurrent.futures import ThreadPoolExecutor
+    in_coords, out_coords = np.asarray(in_coords), np.asarray(out_coords)
+
+    def cuts(c):
+        assert (np.diff(c[:, 0]) >= 0).all(), "coordinates must be sorted by batch item"
+        return np.searchsorted(c[:, 0], np.arange(int(max(in_coords[:, 0].max(), out_coords[:, 0].max())) + 2))
+
+    ci, co = cuts(in_coords), cuts(out_coords)
+    parts = [(np.ascontiguousarray(in_coords[ci[b]:ci[b + 1]]), np.ascontiguousarray(out_coords[co[b]:co[b + 1]]))
+             for b in range(len(ci) - 1)]
+    with ThreadPoolExecutor(max_workers=max(1, min(threads, len(parts)))) as pool:
+        maps = list(pool.map(lambda p: oracle.kernel_map(p[0], p[1], kernel_size, stride), parts))
+    K = len(maps[0][2]) - 1
+    ins, outs, off = [], [], [0]
+    for k in range(K):
+        for b, (im, om, o, _) in enumerate(maps):
+            ins.append(im[o[k]:o[k + 1]] + ci[b])
+            outs.append(om[o[k]:o[k + 1]] + co[b])
+        off.append(off[-1] + sum(int(m[2][k + 1] - m[2][k]) for m in maps))
+    odd = all(int(k) % 2 == 1 for k in kernel_size)
+    iden = K // 2 if odd and len(in_coords) == len(out_coords) else None
+    return (np.concatenate(ins).astype(np.int32), np.concatenate(outs).astype(np.int32),
+            np.asarray(off, dtype=np.int64), iden)

@@ -15,6 +15,12 @@ from warpconvnet_amd.utils import synthetic
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 TOL = {torch.float32: 1e-5, torch.float16: 1e-2, torch.bfloat16: 1e-2}
+# Entry by entry, |a - b| / (|b| + 1e-6) over the entries above a thousandth of the largest (the form
+# the reference's native GEMM tests print, tests/csrc/test_cutlass_gemm.py:24-26).  16-bit results
+# are correctly rounded sums, so the tensor-wide bound holds per entry as well.  An fp32 sum of a few
+# hundred to a few thousand products carries an absolute error of some 1e-7 of the largest entry
+# (measured: 1.4e-7 to 9.7e-7), which is up to 1e-3 of an entry a thousand times smaller.
+ELEM_TOL = {torch.float32: 1e-3, torch.float16: 1e-2, torch.bfloat16: 1e-2}
 
 
 def _dev_i32(a):
@@ -86,6 +92,11 @@ def test_conv_stride1_matches_oracle(oracle, name, dtype, c_in, c_out, n, batch,
     got = out.feature_tensor.float().cpu().numpy()
     want, (im, om, off, iden) = _oracle_out(oracle, x, w, bc, bc, ksize, (1, 1, 1), bias)
     assert rel_err(got, want) <= TOL[dtype], name
+    # and entry by entry, in the form the reference's native GEMM tests print
+    # (tests/csrc/test_cutlass_gemm.py:24-26), over the entries above a thousandth of the largest
+    # (a 1x1x1 kernel is a torch matmul followed by a torch add, as in the reference,
+    # sparse_conv.py:1715-1721: two roundings, felt where product and bias cancel)
+    assert elementwise_rel_err(got, want) <= (5e-2 if K == 1 else ELEM_TOL[dtype]), name
     # the reference's own operation order (per-offset rounding) on the CPU, same tolerance
     ref = explicit_gemm_forward(x.float() if dtype != torch.float32 else x, w.float(),
                                 torch.as_tensor(im), torch.as_tensor(om), off, iden, len(bc))

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import kaiming_weight, rel_err
+from helpers import elementwise_rel_err, kaiming_weight, oracle_kernel_map_by_item, rel_err, sort_rows
 from warpconvnet_amd.utils import synthetic
 
 pytestmark = pytest.mark.gpu
@@ -99,6 +99,48 @@ def test_cfg5a_5x5x5_map_bound(scenes):
     w = kaiming_weight(125, 16, 16, seed=6, dtype=torch.float16).to(DEV)
     got = sparse_conv_forward(x, w, km, n)
     assert rel_err(got.float().cpu().numpy(), torch_explicit_fp32(x, w, km, n).cpu().numpy()) <= 1e-2
+
+
+def _assert_same_map(km, ref):
+    ref_in, ref_out, ref_off, ref_iden = ref
+    assert km.identity_map_index == ref_iden
+    assert np.array_equal(km.offsets.numpy().astype(np.int64), ref_off)
+    assert np.array_equal(km.in_maps.cpu().numpy(), ref_in)
+    assert np.array_equal(km.out_maps.cpu().numpy(), ref_out)
+
+
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (5, 5, 5)], ids=["cfg2_3x3x3", "cfg5a_5x5x5"])
+def test_full_size_map_equals_the_oracle_bit_for_bit(oracle, scenes, ksize):
+    """The 1,000,000-voxel maps of the benchmark configurations against the C oracle, in native
+    order (offsets in k order, ascending output row inside an offset: discrete_kernels.cu:183-213),
+    from both probe passes."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    host = scenes.cpu().numpy()
+    ref = oracle_kernel_map_by_item(oracle, host, host, ksize)
+    _assert_same_map(generate_kernel_map(scenes, scenes, (1, 1, 1), ksize), ref)
+    mp = pytest.MonkeyPatch()
+    try:
+        mp.setenv("WCN_KMAP_PROBE", "blocks")
+        again = scenes.view(-1, 4)  # another tensor object: a table of its own
+        _assert_same_map(generate_kernel_map(again, again, (1, 1, 1), ksize), ref)
+    finally:
+        mp.undo()
+
+
+def test_full_size_strided_coordinates_and_map_equal_the_oracle(oracle, scenes):
+    """cfg3: the strided coordinates of 4 x 250k voxels (as a set, and in this implementation's
+    documented order: ascending first source row) and the 2x2x2 stride-2 map onto them."""
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    host = scenes.cpu().numpy()
+    coarse, offs = stride_coords(scenes, (2, 2, 2))
+    ref_coarse, _, ref_offs = oracle.stride_coords(host, (2, 2, 2), 4)
+    got = coarse.cpu().numpy()
+    assert np.array_equal(sort_rows(got), sort_rows(ref_coarse))
+    assert np.array_equal(got, ref_coarse)
+    assert np.array_equal(offs.numpy().astype(np.int64), ref_offs)
+    ref = oracle_kernel_map_by_item(oracle, host, ref_coarse, (2, 2, 2), (2, 2, 2))
+    _assert_same_map(generate_kernel_map(scenes, coarse, (2, 2, 2), (2, 2, 2)), ref)
 
 
 def test_cfg5b_wide_channels_small_map():

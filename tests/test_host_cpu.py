@@ -212,7 +212,11 @@ def test_reference_import_path_resolves_to_the_same_modules():
     import warpconvnet  # noqa: F401
     for rel in ("nn.modules.sparse_conv", "nn.functional.sparse_conv", "geometry.types.voxels",
                 "geometry.coords.search.torch_discrete", "geometry.coords.ops.stride"):
-        assert importlib.import_module("warpconvnet." + rel) is importlib.import_module("warpconvnet_amd." + rel)
+        m = importlib.import_module("warpconvnet." + rel)
+        assert m is importlib.import_module("warpconvnet_amd." + rel)
+        # the alias leaves the module's own spec in place (relative imports inside it go by it)
+        assert m.__spec__.name == m.__name__ == "warpconvnet_amd." + rel
+        assert m.__spec__.parent == m.__package__
     from warpconvnet.nn.modules.sparse_conv import SparseConv3d
     from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d as ours
     assert SparseConv3d is ours

@@ -31,10 +31,18 @@ class _Alias(importlib.abc.MetaPathFinder, importlib.abc.Loader):
         return importlib.util.spec_from_loader(fullname, self, is_package=True)
 
     def create_module(self, spec):
-        return importlib.import_module(_TARGET + spec.name[len(__name__):])
+        real = importlib.import_module(_TARGET + spec.name[len(__name__):])
+        # the import machinery is about to stamp the alias's spec onto the module it is handed;
+        # the real module keeps its own (relative imports and reloads go by __spec__.parent)
+        self._own_spec[id(real)] = real.__spec__
+        return real
 
     def exec_module(self, module):  # the real module is already initialised
-        pass
+        own = self._own_spec.pop(id(module), None)
+        if own is not None:
+            module.__spec__ = own
+
+    _own_spec = {}
 
 
 sys.meta_path.insert(0, _Alias())

@@ -145,6 +145,39 @@ def _loads_in_flight_touched(name, lines):
     return bad
 
 
+def _written_out_loads(lines):
+    """(number of loads written out in inline assembly, whether a branch behind the last of them
+    leads back to or before the first): what a kernel with a ring of such loads must show."""
+    code = [l.split(";")[0].strip() for l in lines]
+    in_asm, loads, labels = False, [], {}
+    for i, raw in enumerate(lines):
+        if "#ASMSTART" in raw:
+            in_asm = True
+        elif "#ASMEND" in raw:
+            in_asm = False
+        else:
+            if in_asm and re.match(r"global_load_dword(x2|x4)?\s+\S+,", code[i]):
+                loads.append(i)
+            m = re.match(r"(\.LBB\d+_\d+):", code[i])
+            if m:
+                labels[m.group(1)] = i
+    if not loads:
+        return 0, False
+    back = False
+    for i, st in enumerate(code):
+        m = re.match(r"s_c?branch\w*\s+(\.LBB\d+_\d+)", st)
+        if m and i > loads[0] and labels.get(m.group(1), n_inf) <= loads[0]:
+            back = True
+    return len(loads), back
+
+
+n_inf = 1 << 60
+# Kernels that are known to keep loads in flight across their loop (by name): a listing in which
+# the checker recognises none of them, or no loop around them, means the checker no longer reads
+# the compiler's output (another spelling of the markers, labels or mnemonics), not that all is well.
+RING_KERNELS = ("conv_fwd_pack",)
+
+
 def _check_loads_not_copied(src, asm_text):
     """The destination of a written-out load must not be read, moved or overwritten before a vmcnt
     wait that covers the load: a copy the compiler inserts between the load and its wait (at a
@@ -157,6 +190,12 @@ def _check_loads_not_copied(src, asm_text):
     for n, (begin, name) in enumerate(starts):
         end = starts[n + 1][0] if n + 1 < len(starts) else len(lines)
         bad += _loads_in_flight_touched(name, lines[begin:end])
+        if any(k in name for k in RING_KERNELS):
+            count, loops = _written_out_loads(lines[begin:end])
+            if count == 0 or not loops:
+                raise RuntimeError(f"{os.path.basename(src)}: {name}: {count} written-out loads recognised, "
+                                   f"loop around them {'found' if loops else 'not found'}: the listing is not "
+                                   "what this check was written for, so it cannot vouch for the kernel")
     if bad:
         raise RuntimeError(f"{os.path.basename(src)}: the compiler touches registers that loads are still in flight "
                            "into:\n  " + "\n  ".join(bad[:10]))
