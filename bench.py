@@ -289,6 +289,41 @@ def secondary_configs(dev, steps, warmup):
         "num_points": npts, "num_voxels": mvox, "call_ms": t_vox, "points_per_s": npts / (t_vox * 1e-3),
         "algorithmic_GBps": vox_bytes / (t_vox * 1e-3) / 1e9, "same_result_with_torch_ops_ms": t_vox_torch}
     del pts, pfeat, vox
+    # the reference's own standard fixture (tests/nn/test_sparse_conv.py:35-47): three clouds of
+    # randint(1e5, 1e6) points in [0, 100)^3 made unique, 16 channels; cold map + contraction of
+    # the two convolutions its tests run (3x3x3 stride 2 16 -> 13 fp32, 3x3x3 stride 1 16 -> 16 fp16)
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    torch.manual_seed(0)
+    Ns = torch.randint(100000, 1000000, (3,))
+    fix = Voxels([(torch.rand((int(N), 3)) / 0.01).int() for N in Ns],
+                 [torch.rand((int(N), 16)) for N in Ns], device=dev).unique()
+    fc = fix.batch_indexed_coordinates.contiguous()
+    nf = fc.shape[0]
+    w13 = weights(27, 16, 13, torch.float32, 9)
+    w16 = weights(27, 16, 16, torch.float16, 10)
+    xf32, xf16 = fix.feature_tensor.float().contiguous(), fix.feature_tensor.half().contiguous()
+
+    def fixture_s2():
+        cold = fc.view(-1, 4)
+        coarse, _ = stride_coords(cold, (2, 2, 2))
+        return coarse, generate_kernel_map(cold, coarse, (2, 2, 2), (3, 3, 3))
+
+    def fixture_s1():
+        cold = fc.view(-1, 4)
+        return generate_kernel_map(cold, cold, (1, 1, 1), (3, 3, 3))
+
+    t_map2, (fcoarse, fkm2) = timed(fixture_s2)
+    t_conv2, _ = timed(lambda: sparse_conv_forward(xf32, w13, fkm2, len(fcoarse)))
+    t_map1, fkm1 = timed(fixture_s1)
+    t_conv1, _ = timed(lambda: sparse_conv_forward(xf16, w16, fkm1, nf))
+    out["reference fixture (tests/nn/test_sparse_conv.py:35-47): 3 clouds in [0,100)^3, 16 channels"] = {
+        "num_voxels": nf, "occupancy_of_cells": nf / 3e6,
+        "3x3x3 s2 16->13 fp32": {"num_out": len(fcoarse), "num_pairs": int(fkm2.offsets[-1]),
+                                 "pairs_per_out_voxel": int(fkm2.offsets[-1]) / len(fcoarse),
+                                 "coords_and_kernel_map_build_ms": t_map2, "contraction_call_ms": t_conv2},
+        "3x3x3 s1 16->16 fp16": {"num_pairs": int(fkm1.offsets[-1]), "pairs_per_voxel": int(fkm1.offsets[-1]) / nf,
+                                 "kernel_map_build_ms": t_map1, "contraction_call_ms": t_conv1}}
+    del fix, fkm1, fkm2
     out["configs[2]: 2x2x2 s2 96->128 + transposed 128->96 bf16, 1M fine voxels"] = {
         "num_voxels": n, "num_coarse": m, "num_pairs": int(km.offsets[-1]),
         "coords_and_kernel_map_build_ms": t_map, "down_contraction_call_ms": t_down,
