@@ -31,20 +31,22 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
 # --calibrate-copy).  The summary names the kernel it was taken from; a line for another kernel
 # than the one this run launches is reported as stale (traffic: null).
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "conv_fwd_cfg2_hbm_traffic.txt")
-CONV_KERNEL = "conv_fwd_pack<f16, 512, 11, 4, 2, true, false, false>"  # what wcn_sparse_conv_fwd launches for 64 -> 64 fp16
+MAP_TRAFFIC_FILE = os.path.join(ROOT, "profiles", "kernel_map_cfg2_hbm_traffic.txt")
 
 
-def measured_traffic():
-    """(bytes per launch or None, note) from the line `TRAFFIC_JSON: {...}` of the summary."""
+def measured_traffic(path, kernel):
+    """(bytes per launch or None, note) from the line `TRAFFIC_JSON: {...}` of a counter summary;
+    `kernel` is what this run launched (the library says), and a summary taken from another kernel
+    is reported as stale."""
     try:
-        with open(TRAFFIC_FILE) as f:
+        with open(path) as f:
             for line in f:
                 if line.startswith("TRAFFIC_JSON:"):
                     rec = json.loads(line[len("TRAFFIC_JSON:"):])
-                    if rec.get("kernel") != CONV_KERNEL or os.environ.get("WCN_CONV_KERNEL"):
-                        return None, f"stale: {os.path.basename(TRAFFIC_FILE)} holds {rec.get('kernel')}"
+                    if rec.get("kernel") != kernel:
+                        return None, f"stale: {os.path.basename(path)} holds {rec.get('kernel')}, this run launched {kernel}"
                     total = (rec["fetch_kib"] * rec["fetch_factor"] + rec["write_kib"] * rec["write_factor"]) * 1024
-                    return float(total), f"{os.path.basename(TRAFFIC_FILE)} (tree {rec.get('tree', '?')})"
+                    return float(total), f"{os.path.basename(path)} (tree {rec.get('tree', '?')})"
     except (OSError, ValueError, KeyError):
         pass
     return None, "no counter summary found"
@@ -430,6 +432,11 @@ def main():
                          "the headline value stays the forward path)")
     ap.add_argument("--all-configs", action="store_true",
                     help="also time the other single-layer configurations (config.other_configs)")
+    ap.add_argument("--gather-floor", action="store_true",
+                    help="also time a kernel that only gathers the map's rows (roofline.gather_floor)")
+    ap.add_argument("--sorted-voxels", action="store_true",
+                    help="also time the same step on the voxels sorted along a Morton curve, and the sort "
+                         "(config.morton_sorted)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -556,6 +563,7 @@ def main():
                   f"{mids[i].elapsed_time(ends[i]):.3f} ms, kernel "
                   f"{kernel_events[i][0].elapsed_time(kernel_events[i][1]):.3f} ms", file=sys.stderr)
 
+    conv_kernel = L.wcn_conv_last_kernel().decode()  # this thread's last contraction: the timed one
     num_pairs = int(km.offsets[-1])
     c_in, c_out, K, s = 64, 64, 27, 2
     conv_bytes = s * (n * c_in + n * c_out + K * c_in * c_out) + 8 * num_pairs
@@ -563,7 +571,9 @@ def main():
     cap = 2 * n
     map_bytes = 24 * n + 8 * cap + 16 * n + 8 * K * n + 8 * num_pairs
     achieved = conv_bytes / (conv_kernel_ms * 1e-3) / 1e9
-    traffic_bytes, traffic_note = measured_traffic()
+    traffic_bytes, traffic_note = measured_traffic(TRAFFIC_FILE, conv_kernel)
+    map_kernels = ("kmap_pass_fixed<3, 3, 3>" if os.environ.get("WCN_KMAP_PROBE") != "blocks" else "self_probe<1>")
+    map_traffic_bytes, map_traffic_note = measured_traffic(MAP_TRAFFIC_FILE, map_kernels)
 
     result = {
         "metric": METRIC,
@@ -599,7 +609,7 @@ def main():
             "contraction_frac_of_mfma_peak": conv_flops / (conv_kernel_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
         },
         "roofline": {
-            "kernel": CONV_KERNEL if os.environ.get("WCN_CONV_KERNEL") != "ring" else "conv_fwd_ring<f16, 6, false, 0>",
+            "kernel": conv_kernel,
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
@@ -609,8 +619,79 @@ def main():
             "traffic_source": traffic_note,
             "algorithmic_bytes": conv_bytes,
             "measured_peaks": measured_peaks(dev),
+            # the second half of the metric as a roofline line of its own: all kernels of the map
+            # build together (table: hist, colscan, scatter, bins; map: probe, scan, emit) against
+            # the bytes the survey's formula prices for it
+            "map_build": {
+                "kernel": "table_hist + table_colscan + table_scatter + table_bins + " + map_kernels
+                          + " + kmap_scan_rows + " + ("kmap_emit_flat" if "kmap_pass" in map_kernels else "self_count + self_emit"),
+                "probe_kernel": map_kernels,
+                "bound": "hbm",
+                "achieved": map_bytes / (map_ms * 1e-3) / 1e9,
+                "peak": HBM_PEAK_GBS,
+                "unit": "GB/s",
+                "frac": map_bytes / (map_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "ms": map_ms,
+                "traffic": map_traffic_bytes,
+                "traffic_source": map_traffic_note,
+                "algorithmic_bytes": map_bytes,
+            },
         },
     }
+
+    if args.gather_floor:
+        sink = torch.zeros(64, dtype=torch.int32, device=dev)
+        from warpconvnet_amd._lib import check, ptr
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(30)]
+        for a, b in ev:
+            a.record()
+            check(L.wcn_probe_gather_rows(ptr(feats_d), n, 128, ptr(km.in_maps), num_pairs, ptr(sink),
+                                          stream_ptr(dev)), "wcn_probe_gather_rows")
+            b.record()
+        torch.cuda.synchronize()
+        floor_ms = float(np.median([a.elapsed_time(b) for a, b in ev[10:]]))
+        result["roofline"]["gather_floor"] = {
+            "kernel": "gather_rows_probe<8>", "ms": floor_ms,
+            "gathered_GBps": num_pairs * 128 / (floor_ms * 1e-3) / 1e9,
+            "note": ("a kernel that only fetches features[in_maps[p]] for every pair (128-byte rows, 16 rows per "
+                     "wave and request, four requests in flight): no contraction that gathers every pair's row "
+                     "from beyond the L2 runs faster than this plus the output's write")}
+
+    if args.sorted_voxels:
+        from warpconvnet_amd.geometry.coords.ops.serialization import encode
+        a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        offsets_i = torch.as_tensor(np.asarray(offsets, dtype=np.int64))
+        sort_ms = []
+        for _ in range(5):
+            a0.record()
+            res = encode(coords_d[:, 1:].contiguous(), batch_offsets=offsets_i, return_perm=True)
+            order = res.perm
+            sorted_coords = coords_d[order.long()].contiguous()
+            sorted_feats = feats_d[order.long()].contiguous()
+            a1.record()
+            torch.cuda.synchronize()
+            sort_ms.append(a0.elapsed_time(a1))
+        maps, kernels = [], []
+        for _ in range(30):
+            cold = sorted_coords.view(-1, 4)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            k0.record(); k1.record()
+            e0.record()
+            km_s = generate_kernel_map(cold, cold, (1, 1, 1), (3, 3, 3))
+            e1.record()
+            L.wcn_conv_set_timing_events(ctypes.c_void_p(k0.cuda_event), ctypes.c_void_p(k1.cuda_event))
+            sparse_conv_forward(sorted_feats, weight_d, km_s, n)
+            torch.cuda.synchronize()
+            maps.append(e0.elapsed_time(e1))
+            kernels.append(k0.elapsed_time(k1))
+        result["config"]["morton_sorted"] = {
+            "sort_ms": float(np.median(sort_ms)),
+            "sort_note": "Morton codes + torch sorts + the permuted copies of coordinates (16 MB) and features (128 MB)",
+            "kernel_map_build_ms": float(np.median(maps[10:])),
+            "contraction_kernel_ms": float(np.median(kernels[10:])),
+            "unsorted_kernel_map_build_ms": map_ms, "unsorted_contraction_kernel_ms": conv_kernel_ms}
 
     if args.backward:
         from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_backward
@@ -650,6 +731,12 @@ def main():
         got = out.float().cpu()
         err = float((got - ref_out.float()).abs().max() / ref_out.float().abs().max())
         result["config"]["max_rel_err_vs_cpu_baseline"] = err
+        # entry by entry, the form the reference's native GEMM tests print (tests/csrc/test_cutlass_gemm.py:24-26),
+        # over the entries above a thousandth of the largest
+        ref64 = ref_out.double()
+        keep = ref64.abs() > 1e-3 * ref64.abs().max()
+        result["config"]["elementwise_rel_err_vs_cpu_baseline"] = float(
+            ((got.double() - ref64).abs()[keep] / (ref64.abs()[keep] + 1e-6)).max())
     print(json.dumps(result))
 
 

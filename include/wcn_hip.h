@@ -447,12 +447,27 @@ int wcn_segment_reduce_bwd(const void* grad_out, int64_t num_segments, int32_t c
                            const int64_t* segment_offsets, const int64_t* segment_of_row, int64_t num_in,
                            int32_t mode, const int64_t* argmax_or_null, void* grad_in, void* stream);
 
+/* Name of the contraction kernel the last wcn_sparse_conv_fwd / _dgrad call of this host thread
+ * enqueued, template arguments included, as a profiler prints it ("" before the first call).  A
+ * measurement aid with no counterpart in the reference: the benchmark reports the kernel that ran. */
+const char* wcn_conv_last_kernel(void);
+
 /* Measurement hook (no counterpart in the reference, which times whole calls with CUDA events:
  * warpconvnet/utils/timer.py:41-60).  The two hipEvent_t handles are recorded on the call's
  * stream immediately before and after the contraction kernel of the NEXT wcn_sparse_conv_fwd
  * call made by this host thread, so that hipEventElapsedTime gives that kernel's duration
  * alone; the hook then disarms itself.  Pass NULLs to disarm. */
 int wcn_conv_set_timing_events(void* start_event, void* stop_event);
+
+/* ---------------------------------------------------------------------------------------------
+ * Measurement probe (no counterpart in the reference; not on the product path).  Gathers the rows
+ * features[in_maps[p]] (row_bytes = 32, 64 or 128 each; in_maps entries must lie in [0, num_rows))
+ * for all num_pairs pairs, 16 rows per wave and request as the contraction does, and does nothing
+ * with them: its run time is what the memory system needs for the gather alone.  `sink` is one
+ * device word the kernel may write.  Used by `bench.py --gather-floor`.
+ * ------------------------------------------------------------------------------------------- */
+int wcn_probe_gather_rows(const void* features, int64_t num_rows, int32_t row_bytes,
+                          const int32_t* in_maps, int64_t num_pairs, void* sink, void* stream);
 
 #ifdef __cplusplus
 }

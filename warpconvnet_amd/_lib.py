@@ -40,6 +40,7 @@ SIGNATURES = {
     "wcn_stride_unique": (ctypes.c_int, [_vp, _i64, _i32p, _vp, _i64, _vp, _vp, _vp]),
     "wcn_stride_unique_read_count": (ctypes.c_int, [_vp, _i64, _i64, _i64p, _vp]),
     "wcn_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i32, _i64, _i32]),
+    "wcn_conv_last_kernel": (ctypes.c_char_p, []),
     "wcn_conv_set_timing_events": (ctypes.c_int, [_vp, _vp]),
     "wcn_sparse_conv_fwd": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                            _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
@@ -64,6 +65,7 @@ SIGNATURES = {
     "wcn_conv_wgrad_workspace_bytes": (_sz, [_i32, _i32, _i32, _i64, _i64]),
     "wcn_sparse_conv_wgrad": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _i32, _i32, _vp, _vp, _i64p,
                                              _i32, _i32, _vp, _i32, _vp, _sz, _vp]),
+    "wcn_probe_gather_rows": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _vp, _vp]),
     "wcn_voxel_rows": (ctypes.c_int, [_vp, _i64, _i64p, _vp, _i32, ctypes.c_double, _vp, _vp]),
     "wcn_unique_rows_workspace_bytes": (_sz, [_i64]),
     "wcn_unique_rows_csr": (ctypes.c_int, [_vp, _i64, _i32, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _i64p, _vp]),

@@ -35,6 +35,9 @@
 #include <string>
 #include <type_traits>
 
+#include <stdarg.h>
+#include <stdio.h>
+
 #include "wcn_common.h"
 #include "wcn_conv_args.h"
 #include "wcn_mma.h"
@@ -1158,6 +1161,8 @@ int launch_conv(const ConvArgs& a, hipStream_t s) {
       hipLaunchKernelGGL((conv_fwd_ring<T, NC, false, 2>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
     else
       hipLaunchKernelGGL((conv_fwd_ring<T, NC, false, 3>), rgrid, dim3(RING_THREADS), RingCfg<NC>::LDS_BYTES, s, a);
+    wcn_conv_note_kernel("conv_fwd_ring<%s, %d, %s, %d>", wcn_type_text<T>(), NC, a.split ? "true" : "false",
+                         a.split ? 0 : narrow);
     if (a.split) {
       const int64_t items = a.num_out * (a.c_out_pad / 4);
       hipLaunchKernelGGL(conv_split_reduce<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
@@ -1166,6 +1171,7 @@ int launch_conv(const ConvArgs& a, hipStream_t s) {
     }
   } else {
     hipLaunchKernelGGL(conv_fwd<T>, grid, dim3(THREADS), 0, s, a);
+    wcn_conv_note_kernel("conv_fwd<%s>", wcn_type_text<T>());
   }
   if (g_time_stop) (void)hipEventRecord(g_time_stop, s);
   g_time_start = g_time_stop = nullptr;
@@ -1224,7 +1230,19 @@ int wcn_rows_build(const int32_t* in_maps, const int32_t* out_maps, int num_offs
   return WCN_OK;
 }
 
+namespace {
+thread_local char g_last_kernel[160] = "";
+}
+void wcn_conv_note_kernel(const char* format, ...) {
+  va_list ap;
+  va_start(ap, format);
+  vsnprintf(g_last_kernel, sizeof(g_last_kernel), format, ap);
+  va_end(ap);
+}
+
 extern "C" {
+
+const char* wcn_conv_last_kernel(void) { return g_last_kernel; }
 
 int wcn_conv_set_timing_events(void* start_event, void* stop_event) {
   g_time_start = (hipEvent_t)start_event;

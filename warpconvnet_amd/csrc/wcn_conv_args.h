@@ -3,6 +3,8 @@
 #define WCN_CONV_ARGS_H_
 #include "wcn_common.h"
 
+#include <type_traits>
+
 struct ConvArgs {
   const void* X;
   const void* Wt;
@@ -38,3 +40,12 @@ bool wcn_conv_dense_takes(const ConvArgs& a, int dtype);
 int wcn_conv_dense_launch(const ConvArgs& a, int dtype, hipStream_t stream);
 
 #endif  // WCN_CONV_ARGS_H_
+
+// The contraction kernel a launcher has just enqueued, as the profiler would print its name
+// ("conv_fwd_pack<f16, 512, 11, 4, 2, true, false, false>"): kept per host thread for
+// wcn_conv_last_kernel (a measurement aid: reports name what ran, not what was expected to run).
+void wcn_conv_note_kernel(const char* format, ...);
+template <typename T>
+inline const char* wcn_type_text() {
+  return sizeof(T) == 4 ? "float" : (std::is_same<T, _Float16>::value ? "f16" : "bf16");
+}

@@ -290,6 +290,7 @@ int launch_dense(const ConvArgs& a, hipStream_t s) {
   if (tiles <= 0 || tiles > INT32_MAX) return WCN_ERR_INVALID_ARGUMENT;
   const unsigned grid = (unsigned)std::min<int64_t>(tiles, dense_cus());
   hipLaunchKernelGGL((conv_fwd_dense<T, NCB, WAVES, RB>), dim3(grid), dim3(WAVES * 64), lds, s, a, (int)tiles);
+  wcn_conv_note_kernel("conv_fwd_dense<%s, %d, %d, %d>", wcn_type_text<T>(), NCB, WAVES, RB);
   return hipGetLastError() == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
 }
 

@@ -658,6 +658,8 @@ int launch_instance(const ConvArgs& a, hipStream_t s) {
   const unsigned grid = (unsigned)std::min<int64_t>(vtiles, (int64_t)cus[device] * per_cu);
   hipLaunchKernelGGL((conv_fwd_pack<T, R, NW, NB, NL, FULL, K2, WIDE>), dim3(grid), dim3((NW + 1) * 64), lds, s, a,
                      (int)vtiles, ny);
+  wcn_conv_note_kernel("conv_fwd_pack<%s, %d, %d, %d, %d, %s, %s, %s>", wcn_type_text<T>(), R, NW, NB, NL,
+                       FULL ? "true" : "false", K2 ? "true" : "false", WIDE ? "true" : "false");
   return hipGetLastError() == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
 }
 
