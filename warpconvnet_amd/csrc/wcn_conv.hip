@@ -1121,6 +1121,13 @@ int launch_conv(const ConvArgs& a, hipStream_t s) {
     g_time_start = g_time_stop = nullptr;
     return st;
   }
+  if (only == 0 && wcn_conv_group_takes(a, dtype)) {
+    if (g_time_start) (void)hipEventRecord(g_time_start, s);
+    const int st = wcn_conv_group_launch(a, dtype, s);
+    if (g_time_stop) (void)hipEventRecord(g_time_stop, s);
+    g_time_start = g_time_stop = nullptr;
+    return st;
+  }
   if (!ring_only && wcn_conv_pack_takes(a, dtype)) {
     if (g_time_start) (void)hipEventRecord(g_time_start, s);
     const int st = wcn_conv_pack_launch(a, dtype, s);

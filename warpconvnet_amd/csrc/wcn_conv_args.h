@@ -41,6 +41,10 @@ int wcn_conv_dense_launch(const ConvArgs& a, int dtype, hipStream_t stream);
 
 #endif  // WCN_CONV_ARGS_H_
 
+// The contraction for narrow layers (wcn_conv_group.hip): a wave per group of 64 output rows.
+bool wcn_conv_group_takes(const ConvArgs& a, int dtype);
+int wcn_conv_group_launch(const ConvArgs& a, int dtype, hipStream_t stream);
+
 // The contraction kernel a launcher has just enqueued, as the profiler would print its name
 // ("conv_fwd_pack<f16, 512, 11, 4, 2, true, false, false>"): kept per host thread for
 // wcn_conv_last_kernel (a measurement aid: reports name what ran, not what was expected to run).
