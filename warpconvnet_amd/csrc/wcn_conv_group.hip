@@ -32,7 +32,6 @@ using namespace wcn_mma;
 
 namespace {
 
-constexpr int GROUP_WAVES = 12;  // groups in work per workgroup (three waves per SIMD)
 constexpr int GROUP_AHEAD = 8;     // blocks of 16 pairs whose gathered rows are on their way
 constexpr int GROUP_ENTRIES = 16;  // blocks whose pair-list entries are on their way or held
 
@@ -69,12 +68,12 @@ struct GroupOp<__bf16, true> {
   }
 };
 
-template <typename T, int NCB, bool HALF_K, int NCH>  // NCB: 16-channel blocks of output; NCH: 64s of offsets
-__global__ void __launch_bounds__(GROUP_WAVES * 64) conv_fwd_group(ConvArgs a) {
+// NCB: 16-channel blocks of output; NCH: 64s of kernel offsets; WAVES: groups in work per workgroup
+template <typename T, int NCB, bool HALF_K, int NCH, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64) conv_fwd_group(ConvArgs a) {
   typedef GroupOp<T, HALF_K> Op;
   typedef typename Op::V V;
   constexpr int PER = Op::PER_LANE;
-  constexpr int NG = NCB * 4;     // 16-byte granules per row of sums
   constexpr int ROWF = NCB * 16;  // floats per row of sums
   constexpr int ACC_FLOATS = 65 * ROWF;  // row 64: sums of pairs that do not exist
   extern __shared__ __attribute__((aligned(16))) unsigned char group_smem[];
@@ -94,25 +93,25 @@ __global__ void __launch_bounds__(GROUP_WAVES * 64) conv_fwd_group(ConvArgs a) {
   // weight operands: lane (pr, kg) of block cb holds W[k]^T[cb * 16 + pr][kg * PER ..]
   {
     const T* __restrict__ Wt = (const T*)a.Wt;
-    for (int i = threadIdx.x; i < K * NCB * 64; i += GROUP_WAVES * 64) {
+    for (int i = threadIdx.x; i < K * NCB * 64; i += WAVES * 64) {
       const int l = i & 63, cb = (i >> 6) % NCB, k = (i >> 6) / NCB;
       s_w[i] = *reinterpret_cast<const V*>(Wt + ((int64_t)(k * a.c_out_pad + cb * 16 + (l & 15)) * a.c_in_pad + (l >> 4) * PER));
     }
   }
   __syncthreads();  // the only barrier: from here on a wave works alone
 
-  // granule gi of row r of the sums: stored at a position permuted by the row, so that the 16 rows
-  // one instruction touches spread over the banks (rows are 64 or 128 bytes)
-  auto granule = [&](int r, int gi) -> f32x4* {
-    return reinterpret_cast<f32x4*>(acc + r * ROWF + (((gi ^ (NCB == 2 ? r : (r >> 1))) & (NG - 1)) << 2));
-  };
+  // granule gi (4 channels) of row r of the sums: the sums are kept granule by granule, 65 rows of
+  // 16 bytes each, so that the 16 rows one instruction touches spread over the banks and an
+  // address is one shift-and-add away from the row number
+  auto granule = [&](int r, int gi) -> f32x4* { return reinterpret_cast<f32x4*>(acc) + gi * 65 + r; };
   // 8 (4) channels of input row idx.  No lane is switched off and nothing is replaced by zeros
   // afterwards (a select fed by a load is turned into a branch around the load, and the straight
   // line is gone): a pair that does not exist reads row 0 and adds its product to the spare row of
   // sums, and a lane whose channels lie beyond c_in reads the row's first channels, which meet the
   // zero padding of the weight operand.
   auto x_operand = [&](int32_t idx) -> V {
-    return *reinterpret_cast<const V*>(reinterpret_cast<const unsigned char*>(X) + (uint32_t)idx * row_bytes + lane_bytes);
+    const uint32_t at = __umul24((uint32_t)idx, row_bytes) + lane_bytes;  // rows number below 2^24
+    return *reinterpret_cast<const V*>(reinterpret_cast<const unsigned char*>(X) + at);
   };
   auto add_block = [&](int k, V xv, int r) {  // r: the pair's row in the group, 64 if it does not exist
     f32x4* at[NCB];
@@ -134,7 +133,7 @@ __global__ void __launch_bounds__(GROUP_WAVES * 64) conv_fwd_group(ConvArgs a) {
   for (int e = 0; e < 8; ++e)
     bias_v[e] = (a.bias && cpart * 8 + e < a.c_out) ? to_float(((const T*)a.bias)[cpart * 8 + e]) : 0.f;
   const bool with_identity = a.identity >= 0 && a.identity < K;
-  const int64_t total_waves = (int64_t)gridDim.x * GROUP_WAVES;
+  const int64_t total_waves = (int64_t)gridDim.x * WAVES;
   const int32_t* __restrict__ in_maps = a.in_maps;
   const int32_t* __restrict__ out_maps = a.out_maps;
 
@@ -149,7 +148,7 @@ __global__ void __launch_bounds__(GROUP_WAVES * 64) conv_fwd_group(ConvArgs a) {
     list_at[c] = mine[c] ? (int)a.offsets[k] : 0;
     bounds_at[c] = mine[c] ? k * (int)(a.G + 1) : 0;
   }
-  const int64_t g_first = (int64_t)blockIdx.x * GROUP_WAVES + wave;
+  const int64_t g_first = (int64_t)blockIdx.x * WAVES + wave;
   int next_lo[NCH], next_hi[NCH];  // the bounds of the group after this one, requested a group ahead
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
@@ -176,28 +175,37 @@ __global__ void __launch_bounds__(GROUP_WAVES * 64) conv_fwd_group(ConvArgs a) {
       next_lo[c] = a.group_start[bounds_at[c] + gn];
       next_hi[c] = a.group_start[bounds_at[c] + gn + 1];
     }
-    // block t of the list: its offset, the first of its pairs in the lists and how many pairs of
-    // its run it and the blocks after it hold (all three the same in every lane; past the end of
-    // the list: offset 0, no pairs)
-    auto block_at = [&](int t, int& k, int& first, int& left) {
-      int kk = 0;
+    // What block t of the list is: its offset, the first of its pairs in the lists, and how many
+    // pairs of its run it and the blocks after it hold.  Worked out for 64 blocks at a time, a lane
+    // per block (a search of the running block counts), and read from that lane when the block's
+    // entries are requested; past the end of the list: offset 0, no pairs.
+    int page_k = 0, page_first = 0, page_left = 0;
+    auto turn_page = [&](int page) {
+      const int t = page * 64 + lane;
+      int c = 0, at = 0;  // the first offset whose count of blocks exceeds t
+      if (NCH == 2) c = __builtin_amdgcn_readlane(ends[0], 63) <= t ? 1 : 0;
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) kk += __popcll(__ballot(ends[c] <= t));
-      const bool live = t < blocks;
-      kk = live ? kk : 0;
-      int e = 0, lo = 0, cnt = 0;
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        if (NCH == 1 || (kk >> 6) == c) {
-          e = __builtin_amdgcn_readlane(ends[c], kk & 63);
-          lo = __builtin_amdgcn_readlane(run_lo[c], kk & 63);
-          cnt = __builtin_amdgcn_readlane(run_cnt[c], kk & 63);
+      for (int step = 32; step >= 1; step >>= 1) {
+        int e = __shfl(ends[0], at + step - 1, 64);
+        if (NCH == 2) {
+          const int e1 = __shfl(ends[NCH - 1], at + step - 1, 64);
+          e = c ? e1 : e;
         }
+        if (e <= t) at += step;
+      }
+      int e = __shfl(ends[0], at, 64), lo = __shfl(run_lo[0], at, 64), cnt = __shfl(run_cnt[0], at, 64);
+      if (NCH == 2) {
+        const int e1 = __shfl(ends[NCH - 1], at, 64), lo1 = __shfl(run_lo[NCH - 1], at, 64),
+                  cnt1 = __shfl(run_cnt[NCH - 1], at, 64);
+        e = c ? e1 : e;
+        lo = c ? lo1 : lo;
+        cnt = c ? cnt1 : cnt;
       }
       const int b = t - (e - ((cnt + 15) >> 4));  // which block of its run
-      k = kk;
-      first = live ? lo + b * 16 : 0;
-      left = live ? cnt - b * 16 : 0;
+      const bool live = t < blocks;
+      page_k = live ? c * 64 + at : 0;
+      page_first = live ? lo + b * 16 : 0;
+      page_left = live ? cnt - b * 16 : 0;
     };
 
     // the sums start as the identity offset's product (every row reads its own input row; the
@@ -223,13 +231,14 @@ __global__ void __launch_bounds__(GROUP_WAVES * 64) conv_fwd_group(ConvArgs a) {
     int32_t e_in[GROUP_ENTRIES], e_row[GROUP_ENTRIES];
     int b_k[GROUP_ENTRIES], b_left[GROUP_ENTRIES];
     V xv[GROUP_AHEAD];
-    auto request_entries = [&](int slot, int t) {
-      int first;
-      block_at(t, b_k[slot], first, b_left[slot]);
+    auto request_entries = [&](int slot, int on_page) {
+      b_k[slot] = __builtin_amdgcn_readlane(page_k, on_page);
+      b_left[slot] = __builtin_amdgcn_readlane(page_left, on_page);
+      const int first = __builtin_amdgcn_readlane(page_first, on_page);
       const int last = b_left[slot] > 0 ? b_left[slot] - 1 : 0;
-      const int i = first + (pr < last ? pr : last);
-      e_in[slot] = in_maps[i];
-      e_row[slot] = out_maps[i];
+      const uint32_t at = (uint32_t)(first + (pr < last ? pr : last)) * 4u;  // fewer than 2^30 pairs
+      e_in[slot] = *reinterpret_cast<const int32_t*>(reinterpret_cast<const unsigned char*>(in_maps) + at);
+      e_row[slot] = *reinterpret_cast<const int32_t*>(reinterpret_cast<const unsigned char*>(out_maps) + at);
     };
     auto request_rows = [&](int slot, int xslot) {
       const uint32_t row = (uint32_t)(e_row[slot] - (int32_t)m0);
@@ -237,20 +246,36 @@ __global__ void __launch_bounds__(GROUP_WAVES * 64) conv_fwd_group(ConvArgs a) {
       xv[xslot] = x_operand(ok ? e_in[slot] : 0);
       e_row[slot] = ok ? (int)row : 64;
     };
+    // (the requests of the first blocks come in the order the loop issues them, so that one count
+    // of requests issued since holds for a wait on either way into the loop)
+    turn_page(0);
 #pragma unroll
-    for (int u = 0; u < GROUP_ENTRIES; ++u) request_entries(u, u);
-#pragma unroll
-    for (int u = 0; u < GROUP_AHEAD; ++u) request_rows(u, u);
-    __builtin_amdgcn_sched_barrier(0);
+    for (int u = 0; u < GROUP_ENTRIES; ++u) {
+      if (u >= GROUP_AHEAD) request_rows(u - GROUP_AHEAD, u - GROUP_AHEAD);
+      request_entries(u, u);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    static_assert(GROUP_ENTRIES == 16 && GROUP_AHEAD == 8, "the turn below is written out for a ring of 16 and 8");
     for (int t0 = 0; t0 < blocks; t0 += GROUP_ENTRIES) {
-#pragma unroll
-      for (int u = 0; u < GROUP_ENTRIES; ++u) {
-        if (t0 + u >= blocks) break;
-        add_block(b_k[u], xv[u % GROUP_AHEAD], e_row[u]);
-        request_rows((u + GROUP_AHEAD) % GROUP_ENTRIES, u % GROUP_AHEAD);
-        request_entries(u, t0 + u + GROUP_ENTRIES);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      const int ask = t0 + GROUP_ENTRIES;  // the first block whose entries this turn requests
+      if ((ask & 63) == 0) turn_page(ask >> 6);
+      const int todo = blocks - t0, on_page = ask & 63;
+      // one block: multiply it, request the rows of the block 8 further on (whose entries have
+      // arrived) and the entries of the block 16 further on (into the slot just multiplied).
+      // Written out rather than left to the unroller: the turn ends at the list's last block from
+      // any of its 16 places, and the register of every slot has to be fixed at compile time.
+#define WCN_GROUP_STEP(u)                                                      \
+  if ((u) >= todo) goto turn_done;                                             \
+  add_block(b_k[(u)], xv[(u) % GROUP_AHEAD], e_row[(u)]);                      \
+  request_rows(((u) + GROUP_AHEAD) % GROUP_ENTRIES, (u) % GROUP_AHEAD);        \
+  request_entries((u), on_page + (u));                                         \
+  __builtin_amdgcn_sched_barrier(0);
+      WCN_GROUP_STEP(0) WCN_GROUP_STEP(1) WCN_GROUP_STEP(2) WCN_GROUP_STEP(3)
+      WCN_GROUP_STEP(4) WCN_GROUP_STEP(5) WCN_GROUP_STEP(6) WCN_GROUP_STEP(7)
+      WCN_GROUP_STEP(8) WCN_GROUP_STEP(9) WCN_GROUP_STEP(10) WCN_GROUP_STEP(11)
+      WCN_GROUP_STEP(12) WCN_GROUP_STEP(13) WCN_GROUP_STEP(14) WCN_GROUP_STEP(15)
+#undef WCN_GROUP_STEP
+    turn_done:;
     }
 
     // bias, one rounding, 16-byte stores: lane (row = lane >> 2 (+16 per turn), 8 channels = lane & 3)
@@ -297,15 +322,17 @@ inline int group_cus() {
 }
 
 template <typename T, int NCB, bool HALF_K>
-size_t group_lds(int K) {
+size_t group_lds(int K, int waves) {
   typedef typename GroupOp<T, HALF_K>::V V;
-  return (size_t)K * NCB * 64 * sizeof(V) + (size_t)GROUP_WAVES * 65 * NCB * 16 * sizeof(float);
+  return (size_t)K * NCB * 64 * sizeof(V) + (size_t)waves * 65 * NCB * 16 * sizeof(float);
 }
 
-template <typename T, int NCB, bool HALF_K, int NCH>
-int launch_group_chunks(const ConvArgs& a, hipStream_t s) {
-  const size_t lds = group_lds<T, NCB, HALF_K>(a.K);
-  const void* fn = (const void*)conv_fwd_group<T, NCB, HALF_K, NCH>;
+constexpr size_t GROUP_LDS_MAX = 160 * 1024;
+
+template <typename T, int NCB, bool HALF_K, int NCH, int WAVES>
+int launch_group_waves(const ConvArgs& a, hipStream_t s) {
+  const size_t lds = group_lds<T, NCB, HALF_K>(a.K, WAVES);
+  const void* fn = (const void*)conv_fwd_group<T, NCB, HALF_K, NCH, WAVES>;
   {  // more than 64 KiB of dynamic LDS has to be allowed per device and kernel
     static std::mutex mu;
     static size_t allowed[64] = {};
@@ -313,16 +340,26 @@ int launch_group_chunks(const ConvArgs& a, hipStream_t s) {
     if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return WCN_ERR_LAUNCH;
     std::lock_guard<std::mutex> hold(mu);
     if (allowed[device] < lds) {
-      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)GROUP_LDS_MAX) != hipSuccess)
         return WCN_ERR_LAUNCH;
-      allowed[device] = 160 * 1024;
+      allowed[device] = GROUP_LDS_MAX;
     }
   }
-  const int64_t wgs = (a.G + GROUP_WAVES - 1) / GROUP_WAVES;
+  const int64_t wgs = (a.G + WAVES - 1) / WAVES;
   const unsigned grid = (unsigned)std::min<int64_t>(wgs, group_cus());
-  hipLaunchKernelGGL((conv_fwd_group<T, NCB, HALF_K, NCH>), dim3(grid), dim3(GROUP_WAVES * 64), lds, s, a);
-  wcn_conv_note_kernel("conv_fwd_group<%s, %d, %s, %d>", wcn_type_text<T>(), NCB, HALF_K ? "true" : "false", NCH);
+  hipLaunchKernelGGL((conv_fwd_group<T, NCB, HALF_K, NCH, WAVES>), dim3(grid), dim3(WAVES * 64), lds, s, a);
+  wcn_conv_note_kernel("conv_fwd_group<%s, %d, %s, %d, %d>", wcn_type_text<T>(), NCB, HALF_K ? "true" : "false", NCH, WAVES);
   return hipGetLastError() == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
+}
+
+// Sixteen waves per workgroup (four per SIMD) where 16 channels of output keep a wave within 128
+// registers and the sums of sixteen groups fit LDS beside the weights; twelve otherwise.
+template <typename T, int NCB, bool HALF_K, int NCH>
+int launch_group_chunks(const ConvArgs& a, hipStream_t s) {
+  if constexpr (NCB == 1 && (HALF_K || NCH == 1)) {
+    if (group_lds<T, NCB, HALF_K>(a.K, 16) <= GROUP_LDS_MAX) return launch_group_waves<T, NCB, HALF_K, NCH, 16>(a, s);
+  }
+  return launch_group_waves<T, NCB, HALF_K, NCH, 12>(a, s);
 }
 
 template <typename T, int NCB, bool HALF_K>
@@ -341,9 +378,9 @@ int launch_group(const ConvArgs& a, hipStream_t s) {
 template <typename T>
 bool group_fits(const ConvArgs& a) {
   const bool half_k = a.c_in <= 16;
-  const size_t lds = a.c_out <= 16 ? (half_k ? group_lds<T, 1, true>(a.K) : group_lds<T, 1, false>(a.K))
-                                   : (half_k ? group_lds<T, 2, true>(a.K) : group_lds<T, 2, false>(a.K));
-  return lds <= 160 * 1024;
+  const size_t lds = a.c_out <= 16 ? (half_k ? group_lds<T, 1, true>(a.K, 12) : group_lds<T, 1, false>(a.K, 12))
+                                   : (half_k ? group_lds<T, 2, true>(a.K, 12) : group_lds<T, 2, false>(a.K, 12));
+  return lds <= GROUP_LDS_MAX;
 }
 
 }  // namespace
@@ -357,7 +394,9 @@ bool wcn_conv_group_takes(const ConvArgs& a, int dtype) {
   if (!a.vec_in || a.split || !a.group_start || a.G <= 0 || a.num_pairs <= 0) return false;
   if (a.c_in > 32 || a.c_out > 32 || (a.c_in <= 16 && a.c_in % 4 != 0)) return false;
   if ((uint64_t)a.num_in * (uint64_t)a.c_in * 2u >= (1ull << 32)) return false;
-  if (a.K > 128 || (int64_t)a.K * (a.G + 1) >= (1ll << 31) || a.num_pairs >= (1ll << 31)) return false;
+  if (a.K > 128 || (int64_t)a.K * (a.G + 1) >= (1ll << 31) || a.num_pairs >= (1ll << 30) ||
+      a.num_in > (1ll << 24))
+    return false;
   return dtype == WCN_DTYPE_F16 ? group_fits<_Float16>(a) : group_fits<__bf16>(a);
 }
 
