@@ -352,11 +352,13 @@ int launch_group_waves(const ConvArgs& a, hipStream_t s) {
   return hipGetLastError() == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
 }
 
-// Sixteen waves per workgroup (four per SIMD) where 16 channels of output keep a wave within 128
-// registers and the sums of sixteen groups fit LDS beside the weights; twelve otherwise.
+// Sixteen waves per workgroup (four per SIMD) where the sums of sixteen groups fit LDS beside the
+// weights, twelve otherwise (3x3x3 with 32 channels on both sides: 54 KB of weights and 8 KB of
+// sums per wave).  The one instance that does not stay within 128 registers has weights that fit
+// LDS for no kernel of more than 64 offsets and is not built.
 template <typename T, int NCB, bool HALF_K, int NCH>
 int launch_group_chunks(const ConvArgs& a, hipStream_t s) {
-  if constexpr (NCB == 1 && (HALF_K || NCH == 1)) {
+  if constexpr (!(NCB == 2 && !HALF_K && NCH == 2)) {
     if (group_lds<T, NCB, HALF_K>(a.K, 16) <= GROUP_LDS_MAX) return launch_group_waves<T, NCB, HALF_K, NCH, 16>(a, s);
   }
   return launch_group_waves<T, NCB, HALF_K, NCH, 12>(a, s);
