@@ -216,6 +216,24 @@ def test_pair_lists_are_reordered_once_and_kept_on_the_map(oracle):
         assert ins.tolist()[:2] == [7, 3] and outs.tolist()[:2] == [0, 2]
         assert ins.tolist()[4] == 1 and outs.tolist()[4] == 1
 
+    # through the operator interface such lists are refused: the reference's scatter would add up
+    # all three pairs of (offset 0, row 2), the device contraction takes one pair per offset and row
+    from warpconvnet_amd.geometry.coords.search.search_results import IntSearchResult
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    repeated = IntSearchResult(in_l, out_l, torch.tensor([0, 4, 6], dtype=torch.int32))
+    feats = torch.randn(10, 16, device=DEV)
+    weights = torch.randn(2, 16, 16, device=DEV)
+    with pytest.raises(ValueError, match="repeat an"):
+        sparse_conv_forward(feats, weights, repeated, 3)
+    # the same lists without the repeats pass, out of order as they are
+    clean = IntSearchResult(in_l[[2, 4, 0]], out_l[[2, 4, 0]], torch.tensor([0, 2, 3], dtype=torch.int32))
+    got = sparse_conv_forward(feats, weights, clean, 3)
+    want = torch.zeros(3, 16, device=DEV)
+    want[0] += feats[7] @ weights[0]
+    want[1] += feats[1] @ weights[0]
+    want[2] += feats[9] @ weights[1]
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
+
 
 def test_transposed_adjoint_identity():
     """<conv(x), y> == <x, conv_T(y)> when the transposed weights are W[k]^T on the same map."""

@@ -1106,9 +1106,10 @@ template <typename T>
 int launch_conv(const ConvArgs& a, hipStream_t s) {
   constexpr int dtype = std::is_same<T, float>::value ? WCN_DTYPE_F32
                         : std::is_same<T, _Float16>::value ? WCN_DTYPE_F16 : WCN_DTYPE_BF16;
-  // Wide rows on both sides go to the output-stationary kernel of wcn_conv_dense.hip, rows of up to
-  // four k-slices to the pair-packed kernel.  WCN_CONV_KERNEL=ring in the environment keeps
-  // everything on the kernels below, WCN_CONV_KERNEL=pack skips the first of the two (for comparisons).
+  // Wide rows on both sides go to the output-stationary kernel of wcn_conv_dense.hip, 16-bit rows of
+  // at most 32 channels on both sides to the kernel of wcn_conv_group.hip, rows of up to four
+  // k-slices to the pair-packed kernel.  WCN_CONV_KERNEL=ring in the environment keeps everything on
+  // the kernels below, WCN_CONV_KERNEL=pack skips the first two of the three (for comparisons).
   static const int only = [] {
     const char* e = getenv("WCN_CONV_KERNEL");
     return !e ? 0 : std::string(e) == "ring" ? 1 : std::string(e) == "pack" ? 2 : 0;

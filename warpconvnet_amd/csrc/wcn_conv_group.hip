@@ -11,15 +11,15 @@
 // once per workgroup.  After that load there is no barrier and no atomic in the kernel:
 //
 //   * the pairs of offset k whose output row lies in the group are one run of the pair lists
-//     (bounds from group_start); the runs of 32 offsets are requested together, a lane per pair;
-//   * a run is multiplied in blocks of 16 pairs: the gathered rows are the B operand (lane = (pair,
-//     8 or 4 channels)), W[k]^T the A operand, so that a lane ends up with 4 consecutive output
-//     channels of one pair and adds them to that pair's row of sums with one 16-byte LDS read and
-//     write; pairs that do not exist add zeros to a spare row, and every offset issues its loads
-//     whether it has pairs or not: the code of a chunk of 32 offsets is one straight line, in
-//     which the compiler's own waits for the gathered rows (requested GROUP_AHEAD offsets ahead)
-//     are exact;
-//   * runs of more than 16 pairs (dense data) get their further blocks in a second, plain pass;
+//     (bounds from group_start); a run is cut into blocks of 16 pairs, and the blocks of all offsets
+//     of a group form one list that the wave walks from end to end;
+//   * a block is multiplied transposed: the gathered rows are the B operand (lane = (pair, 8 or 4
+//     channels)), W[k]^T the A operand, so that a lane ends up with 4 consecutive output channels of
+//     one pair and hands that pair's row of sums to the MFMA as its C operand: one 16-byte LDS read
+//     and write per 16 channels.  Pairs that do not exist read row 0 and add into a spare row;
+//   * requests run a fixed distance ahead of the multiplications (the rows 8 blocks, the pair-list
+//     entries 16), in a ring whose 16 steps are written out: plain loads, and the compiler's own
+//     waits for them come out exact because the start-up issues its requests in the loop's order;
 //   * the additions of a row happen in a fixed order: results are bitwise reproducible.
 #include <algorithm>
 #include <mutex>

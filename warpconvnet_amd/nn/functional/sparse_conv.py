@@ -13,6 +13,7 @@ the map with in and out exchanged; `wcn_sparse_conv_wgrad`: per-offset X^T dY ov
 reference: sparse_conv.py:314-355).
 """
 import ctypes
+import warnings
 import enum
 import os
 from typing import List, Optional, Tuple, Union
@@ -100,6 +101,25 @@ def _pairs_sorted(km: IntSearchResult, by: str, num_rows: int):
                                   host_offsets, K, num_rows, ptr(g_sorted), ptr(a_sorted),
                                   ptr(groups), ptr(ws), ws.numel(), stream_ptr(device)),
           "wcn_pairs_sort_by_out")
+    # The re-ordering keeps one pair per (offset, ascending-side row).  Kernel maps of duplicate-free
+    # coordinate sets have no more than that.  Lists with more (hand-made ones, or a map over
+    # coordinates that repeat rows) lose pairs here that the reference's atomic scatter adds up
+    # (sparse_conv.py:495-544): for the forward product they are refused instead of contracted
+    # wrongly; for the input gradient one contribution per row is what the reference's explicit path
+    # keeps as well (`grad_in[in_map] += ...` without accumulation, sparse_conv.py:350), so that
+    # case only warns.  One read of K counts per map object, skipped where the map builder vouches
+    # for the lists.
+    vouched = getattr(km, "_keys_unique", False) and getattr(km, "_same_set", False)
+    if num_pairs > 0 and not vouched:
+        kept_pairs = int(groups.view(K, (num_rows + 63) // 64 + 1)[:, -1].sum())
+        if kept_pairs != num_pairs:
+            what = (f"kernel map holds {num_pairs - kept_pairs} pairs that repeat an (offset, "
+                    f"{'output' if by == 'out' else 'input'} row) of another pair; the device contraction "
+                    "takes one pair per offset and row (coordinates with repeated rows? make them unique first)")
+            if by == "out":
+                raise ValueError(what)
+            warnings.warn(what + "; the input gradient keeps the pair with the lowest row", RuntimeWarning,
+                          stacklevel=3)
     kept = (g_sorted, a_sorted, groups, num_rows)
     if by == "out":
         km._by_out = kept
@@ -113,7 +133,12 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
                         num_out_coords: int, bias: Optional[Tensor] = None,
                         compute_dtype: Optional[torch.dtype] = None) -> Tensor:
     """out = bias + sum_k scatter(X[in_k] @ W[k]) on the GPU (replaces the per-offset loops of
-    sparse_conv.py:281-311 / :358-415 / :495-544 and the native GEMMs they call)."""
+    sparse_conv.py:281-311 / :358-415 / :495-544 and the native GEMMs they call).
+
+    A map whose out_maps does not ascend inside every offset (a hand-made one, the exchanged map
+    of a transposed convolution) is re-ordered once; that step takes at most one pair per (offset,
+    output row), which every kernel map of duplicate-free coordinates satisfies, and raises
+    ValueError for lists that hold more (the reference would add all of them up)."""
     require_device(in_features, "in_features")
     if in_features.ndim != 2 or weight.ndim != 3 or weight.shape[1] != in_features.shape[1]:
         raise ValueError(f"shape mismatch: features {tuple(in_features.shape)}, "
@@ -174,7 +199,14 @@ def sparse_conv_backward(grad_output: Tensor, in_features: Tensor, weight: Tenso
     sparse_conv.py:314-355 / :418-492 / :547-627 and the native GEMMs they call):
     dX[in_k] += dY[out_k] @ W[k]^T ;  dW[k] = X[in_k]^T @ dY[out_k], fp32 accumulation, one
     rounding.  Returns (grad_in_features or None, grad_weight or None) in the dtypes of
-    in_features and weight."""
+    in_features and weight.
+
+    The input gradient walks the map by input row; a map whose in_maps does not ascend inside
+    every offset is re-ordered once for that, keeping one pair per (offset, input row).  Where the
+    lists hold more (coordinates with repeated rows) the pair with the lowest row is kept and a
+    RuntimeWarning says how many were left out: the reference's explicit path keeps one such
+    contribution as well (an index assignment without accumulation, sparse_conv.py:350), its
+    atomic paths add them up."""
     require_device(grad_output, "grad_output")
     require_device(in_features, "in_features")
     dtype = compute_dtype or in_features.dtype
