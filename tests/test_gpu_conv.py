@@ -104,6 +104,48 @@ def test_conv_stride1_matches_oracle(oracle, name, dtype, c_in, c_out, n, batch,
     assert rel_err(got, ref) <= TOL[dtype], name
 
 
+NARROW_CASES = [
+    # name, dtype, c_in, c_out, kernel, voxels (0: a full 14^3 cube, runs of up to 64 pairs), extent
+    ("bf16_32_32", torch.bfloat16, 32, 32, (3, 3, 3), 9000, 26),          # twelve waves: 54 KB of weights
+    ("f16_24_32", torch.float16, 24, 32, (3, 3, 3), 5000, 22),            # the last quarter of the k-step is padding
+    ("bf16_8_16", torch.bfloat16, 8, 16, (3, 3, 3), 5000, 22),            # 16-channel k-step, one block of output channels
+    ("f16_12_20", torch.float16, 12, 20, (3, 3, 3), 5000, 22),            # output rows that are not whole 16-byte vectors
+    ("f16_16_16_k5", torch.float16, 16, 16, (5, 5, 5), 4000, 24),         # more than 64 offsets, 16-channel k-step
+    ("f16_32_16_k357", torch.float16, 32, 16, (3, 5, 7), 4000, 24),       # 105 offsets of 32 channels: 105 KB of weights
+    ("bf16_16_16_k2", torch.bfloat16, 16, 16, (2, 2, 2), 5000, 22),       # no identity offset
+    ("f16_16_32_cube", torch.float16, 16, 32, (3, 3, 3), 0, 14),          # every run full: four blocks per offset and group
+    ("bf16_32_32_sparse", torch.bfloat16, 32, 32, (3, 3, 3), 3000, 60),   # nearly every run empty
+]
+
+
+@pytest.mark.parametrize("name,dtype,c_in,c_out,ksize,n,extent", NARROW_CASES, ids=[c[0] for c in NARROW_CASES])
+def test_narrow_layers_take_the_group_kernel_and_match_the_oracle(oracle, name, dtype, c_in, c_out, ksize, n, extent):
+    """16-bit rows of at most 32 channels on both sides: a wave per group of 64 output rows, all weight
+    tiles in LDS (conv_fwd_group).  Every instance of the kernel, against the fp64 oracle."""
+    from warpconvnet_amd._lib import lib
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    if n == 0:
+        xs, ys, zs = np.meshgrid(np.arange(extent), np.arange(extent), np.arange(extent), indexing="ij")
+        cube = np.stack([xs, ys, zs], axis=-1).reshape(-1, 3).astype(np.int32)
+        items = [cube[np.random.default_rng(1).permutation(len(cube))]]
+    else:
+        items = [synthetic.random_cloud(70 + b, n, extent)[:, 1:] for b in range(2)]
+    bc = synthetic.batch_indexed(items)
+    K = int(np.prod(ksize))
+    x = normal_features(len(bc), c_in, seed=21, dtype=dtype)
+    w = kaiming_weight(K, c_in, c_out, seed=22, dtype=dtype)
+    bias = (torch.randn(c_out, generator=torch.Generator().manual_seed(23)) * 0.1).to(dtype)
+    out = spatially_sparse_conv(_voxels(items, x), w.to(DEV), ksize, bias=bias.to(DEV))
+    assert lib().wcn_conv_last_kernel().decode().startswith("conv_fwd_group<"), lib().wcn_conv_last_kernel()
+    got = out.feature_tensor.float().cpu().numpy()
+    want, _ = _oracle_out(oracle, x, w, bc, bc, ksize, (1, 1, 1), bias)
+    assert rel_err(got, want) <= TOL[dtype], name
+    assert elementwise_rel_err(got, want) <= ELEM_TOL[dtype], name
+    # the same call again: the additions of a row happen in a fixed order
+    again = spatially_sparse_conv(_voxels(items, x), w.to(DEV), ksize, bias=bias.to(DEV))
+    assert torch.equal(out.feature_tensor, again.feature_tensor)
+
+
 def test_conv_dense_cube_equals_conv3d():
     """Textbook anchor: on a fully occupied cube with zero padding the sparse convolution is
     torch.nn.functional.conv3d (cross-correlation), W[k] <-> weight[:, :, i, j, kk].T with
