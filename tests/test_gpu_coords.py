@@ -207,6 +207,23 @@ def test_ordered_stride_coords():
         assert bool((torch.diff(seg) >= 0).all())
 
 
+def test_batch_offsets_of_an_ascending_column_by_search():
+    """The search for the bounds of an ascending batch column gives what counting gives, with batch
+    items that have no rows in the middle, and falls back to counting beyond its limit of items."""
+    from warpconvnet_amd.geometry.coords.ops import batch_index as bi
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    col = torch.tensor([0, 0, 1, 1, 1, 4, 4, 7], dtype=torch.int32, device=DEV)
+    counted = bi.offsets_from_batch_index(col)
+    assert counted.tolist() == [0, 2, 5, 5, 5, 7, 7, 7, 8]
+    assert bi.offsets_from_batch_index(col, ascending=True).tolist() == counted.tolist()
+    many = torch.arange(0, 3000, dtype=torch.int32, device=DEV).repeat_interleave(2)  # more items than searched for
+    assert bi.offsets_from_batch_index(many, ascending=True).tolist() == bi.offsets_from_batch_index(many).tolist()
+    in_coords = synthetic.random_cloud(34, 20000, 40, batch_size=4)
+    a, a_off = stride_coords(_dev(in_coords), (2, 2, 2))
+    b, b_off = stride_coords(_dev(in_coords), (2, 2, 2), batch_sorted=True)
+    assert torch.equal(a, b) and a_off.tolist() == b_off.tolist()
+
+
 def test_kernel_map_invariants_full_size():
     """Size-independent properties at the benchmark's size (4 x 250k voxels, 3x3x3):
     identity row, offset symmetry, duplicate-free rows."""

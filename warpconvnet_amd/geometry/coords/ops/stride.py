@@ -14,7 +14,7 @@ from ..search.torch_hashmap import _four_columns
 
 @torch.no_grad()
 def stride_coords(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
-                  order="random") -> Tuple[Tensor, Tensor]:
+                  order="random", batch_sorted: bool = False) -> Tuple[Tensor, Tensor]:
     """Unique rows of floor(coords / [1, *stride]) and their batch offsets.
 
     One call into the HIP library (floor division, table build over the coarse rows, selection of
@@ -23,18 +23,20 @@ def stride_coords(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
     yields a batch-sorted output (the reference sorts by batch afterwards, stride.py:44-48, with an
     order inside a batch that depends on a thread race; as sets the results are identical).
     Any other `order` sorts the coarse voxels of every batch item along that curve.
+    `batch_sorted=True` (not in the reference) vouches that the input's batch column does not
+    descend, which makes the batch offsets of the output one device search and one read.
     """
     num_spatial_dims = batch_indexed_coords.shape[1] - 1
     assert len(stride) == num_spatial_dims, \
         (f"Stride must match the number of spatial dimensions. Got {len(stride)} spatial "
          f"dimensions for but coordinates with {num_spatial_dims} spatial dimensions.")
     if all(s == 1 for s in stride):
-        return batch_indexed_coords, offsets_from_batch_index(batch_indexed_coords[:, 0])
+        return batch_indexed_coords, offsets_from_batch_index(batch_indexed_coords[:, 0], ascending=batch_sorted)
     out, count = unique_floor_div_rows(batch_indexed_coords, stride)
     unique_coords = out[:count, : num_spatial_dims + 1]
     if num_spatial_dims != 3:
         unique_coords = unique_coords.contiguous()
-    out_offsets = offsets_from_batch_index(unique_coords[:, 0])
+    out_offsets = offsets_from_batch_index(unique_coords[:, 0], ascending=batch_sorted)
     if str(getattr(order, "name", order)).lower() not in ("random", "point_ordering.random"):
         # The coarse voxels of every batch item along a space-filling curve.  (The reference hands
         # the four-column rows to `encode`, whose code function accepts three columns and raises,

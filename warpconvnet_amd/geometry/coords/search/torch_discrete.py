@@ -230,7 +230,7 @@ def generate_kernel_map(
     same_set = (batch_indexed_in_coords.data_ptr() == batch_indexed_out_coords.data_ptr()
                 and batch_indexed_in_coords.shape == batch_indexed_out_coords.shape
                 and batch_indexed_in_coords.stride() == batch_indexed_out_coords.stride())
-    result._same_set = bool(same_set)  # with _keys_unique: no row repeats on either side of a pair
+    result._from_builder = True  # pairs come from one lookup per (offset, output row)
     result._symmetric = bool(same_set and is_odd and all(s == 1 for s in stride)
                              and centres is None and getattr(result, "_keys_unique", False))
     if skip_symmetric_kernel_map and is_odd:

@@ -107,9 +107,9 @@ def _pairs_sorted(km: IntSearchResult, by: str, num_rows: int):
     # (sparse_conv.py:495-544): for the forward product they are refused instead of contracted
     # wrongly; for the input gradient one contribution per row is what the reference's explicit path
     # keeps as well (`grad_in[in_map] += ...` without accumulation, sparse_conv.py:350), so that
-    # case only warns.  One read of K counts per map object, skipped where the map builder vouches
-    # for the lists.
-    vouched = getattr(km, "_keys_unique", False) and getattr(km, "_same_set", False)
+    # case only warns.  One read of K counts (a wait for the stream) per map object, skipped for
+    # the maps the builder made over a coordinate table that reported no repeated key.
+    vouched = getattr(km, "_keys_unique", False) and getattr(km, "_from_builder", False)
     if num_pairs > 0 and not vouched:
         kept_pairs = int(groups.view(K, (num_rows + 63) // 64 + 1)[:, -1].sum())
         if kept_pairs != num_pairs:
@@ -337,7 +337,7 @@ def generate_output_coords_and_kernel_map(
         out_coords, out_offsets = expand_coords(in_coords, kernel_size=kernel_size,
                                                 kernel_dilation=kernel_dilation)
     elif any(s != 1 for s in stride):
-        out_coords, out_offsets = stride_coords(in_coords, stride)
+        out_coords, out_offsets = stride_coords(in_coords, stride, batch_sorted=True)
         if generative:  # the strided voxels are expanded in addition
             out_coords, out_offsets = expand_coords(out_coords, kernel_size=kernel_size,
                                                     kernel_dilation=kernel_dilation)
@@ -378,6 +378,8 @@ def generate_output_coords_and_kernel_map(
                                      offsets=forward_map.offsets)
         kernel_map._in_ascend = forward_map._out_ascend
         kernel_map._in_group_start = forward_map._group_start
+        kernel_map._keys_unique = getattr(forward_map, "_keys_unique", False)
+        kernel_map._from_builder = getattr(forward_map, "_from_builder", False)
     else:
         kernel_map = generate_kernel_map(in_coords, out_coords, stride, kernel_size,
                                          kernel_dilation, method=method,

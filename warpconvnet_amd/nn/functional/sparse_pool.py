@@ -105,7 +105,7 @@ def sparse_reduce(voxels: Voxels, kernel_size: Union[int, Tuple[int, ...]],
     out_tensor_stride = tuple(o * s for o, s in zip(stride, in_tensor_stride))
 
     in_coords = voxels.batch_indexed_coordinates
-    out_coords, out_offsets = stride_coords(in_coords, stride, order=order)
+    out_coords, out_offsets = stride_coords(in_coords, stride, order=order, batch_sorted=True)
     from .sparse_conv import STRIDED_CONV_MODE
     key = IntSearchCacheKey(kernel_size=kernel_size, kernel_dilation=ntuple(1, ndim=ndim),
                             transposed=False, generative=False,
