@@ -338,10 +338,12 @@ class _UNet:
     stages (32, 64, 128, 256: 2x2x2 stride-2 convolution + two residual blocks of two 3x3x3
     convolutions) and four up stages (transposed 2x2x2 stride-2 convolution, skip concatenation,
     two residual blocks, 1x1 shortcut where the channel count changes).  Batch norm is folded into
-    the convolutions' weight and bias; ReLU and the residual adds are torch elementwise ops."""
+    the convolutions' weight and bias; ReLU and the residual adds ride in the convolutions'
+    epilogues (`fused=False`: as torch elementwise ops after every convolution)."""
 
-    def __init__(self, dev, dtype, seed=0):
+    def __init__(self, dev, dtype, seed=0, fused=True):
         from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d
+        self.fused = fused
         torch.manual_seed(seed)
         mk = lambda *a, **k: SparseConv3d(*a, bias=True, **k).to(dev).to(dtype)  # noqa: E731
         enc = (32, 64, 128, 256)
@@ -364,24 +366,31 @@ class _UNet:
     def _relu(x):
         return x.replace(batched_features=torch.relu(x.feature_tensor))
 
+    def _conv_relu(self, conv, x, out=None, residual=None):
+        if self.fused:
+            return conv(x, out, residual=residual, relu=True)
+        y = conv(x, out)
+        if residual is not None:
+            y = y.replace(batched_features=y.feature_tensor + residual.feature_tensor)
+        return self._relu(y)
+
     def _block(self, x, blk):
         a, b, shortcut = blk
-        y = b(self._relu(a(x)))
         skip = x if shortcut is None else shortcut(x)
-        return self._relu(y.replace(batched_features=y.feature_tensor + skip.feature_tensor))
+        return self._conv_relu(b, self._conv_relu(a, x), residual=skip)
 
     @torch.no_grad()
     def __call__(self, x):
-        levels = [self._relu(self.stem(x))]
+        levels = [self._conv_relu(self.stem, x)]
         for down, blocks in zip(self.down, self.enc_blocks):
-            y = self._relu(down(levels[-1]))
+            y = self._conv_relu(down, levels[-1])
             for blk in blocks:
                 y = self._block(y, blk)
             levels.append(y)
         y = levels.pop()
         for up, blocks in zip(self.up, self.dec_blocks):
             skip = levels.pop()
-            y = self._relu(up(y, skip))
+            y = self._conv_relu(up, y, skip)
             y = y.replace(batched_features=torch.cat([y.feature_tensor, skip.feature_tensor], dim=1))
             for blk in blocks:
                 y = self._block(y, blk)

@@ -218,6 +218,24 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
                         const int32_t* group_start_or_null, void* out, int64_t num_out,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* wcn_sparse_conv_fwd with the elementwise work that follows a convolution in a residual network
+ * done in the kernel's epilogue, on the fp32 sums before the one rounding:
+ *
+ *   out[m, :] = act(bias + sum ... + residual[m, :]),   act = max(., 0) if relu != 0
+ *
+ * residual_or_null: (num_out, c_out) rows of the feature dtype, not the output buffer itself.
+ * Replaces the separate elementwise kernels of the reference's modules around a convolution: the
+ * addition of a block's shortcut and nn/modules/activations.py:36-52 (ReLU over the features),
+ * which read and write the whole output again.  Everything else as wcn_sparse_conv_fwd. */
+int wcn_sparse_conv_fwd_fused(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                              const void* weight, int32_t weight_dtype, int32_t num_offsets,
+                              int32_t c_out, const void* bias_or_null, const int32_t* in_maps,
+                              const int32_t* out_maps, const int64_t* host_offsets,
+                              int32_t identity_offset, int32_t out_maps_ascend,
+                              const int32_t* group_start_or_null, const void* residual_or_null,
+                              int32_t relu, void* out, int64_t num_out, void* workspace,
+                              size_t workspace_bytes, void* stream);
+
 /* wcn_sparse_conv_fwd for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
  * Same arguments and results as wcn_sparse_conv_fwd, minus the workspace: the scratch memory is a

@@ -146,6 +146,49 @@ def test_narrow_layers_take_the_group_kernel_and_match_the_oracle(oracle, name, 
     assert torch.equal(out.feature_tensor, again.feature_tensor)
 
 
+FUSED_CASES = [
+    # name, dtype, c_in, c_out, voxels, extent, kernel whose launcher takes it
+    ("group", torch.bfloat16, 32, 32, 6000, 24, "conv_fwd_group"),
+    ("pack", torch.float16, 64, 64, 6000, 24, "conv_fwd_pack"),
+    ("pack_f32", torch.float32, 32, 24, 4000, 22, "conv_fwd_pack"),
+    ("dense", torch.bfloat16, 128, 128, 30000, 64, "conv_fwd_dense"),
+    ("ring_split", torch.float16, 256, 256, 1500, 16, "conv_fwd_ring"),
+    ("odd_widths", torch.float32, 7, 13, 3000, 20, "conv_fwd"),  # whichever kernel takes the padded rows
+]
+
+
+@pytest.mark.parametrize("name,dtype,c_in,c_out,n,extent,kernel", FUSED_CASES, ids=[c[0] for c in FUSED_CASES])
+def test_residual_and_relu_in_the_epilogue(oracle, name, dtype, c_in, c_out, n, extent, kernel):
+    """act(conv + bias + residual) with the two extras inside the contraction (every kernel's epilogue)
+    against the fp64 oracle, and against the same call followed by the two torch operations."""
+    from warpconvnet_amd._lib import lib
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    items = [synthetic.random_cloud(80, n, extent)[:, 1:]]
+    bc = synthetic.batch_indexed(items)
+    x = normal_features(len(bc), c_in, seed=31, dtype=dtype)
+    w = kaiming_weight(27, c_in, c_out, seed=32, dtype=dtype)
+    bias = (torch.randn(c_out, generator=torch.Generator().manual_seed(33)) * 0.1).to(dtype)
+    res = normal_features(len(bc), c_out, seed=34, dtype=dtype)
+    vox = _voxels(items, x)
+    want, _ = _oracle_out(oracle, x, w, bc, bc, (3, 3, 3), (1, 1, 1), bias)
+    for residual, relu in ((res, True), (res, False), (None, True)):
+        out = spatially_sparse_conv(vox, w.to(DEV), 3, bias=bias.to(DEV),
+                                    residual=None if residual is None else residual.to(DEV), relu=relu)
+        assert lib().wcn_conv_last_kernel().decode().startswith(kernel), lib().wcn_conv_last_kernel()
+        ref = want + (0 if residual is None else residual.double().numpy())
+        ref = np.maximum(ref, 0.0) if relu else ref
+        got = out.feature_tensor.float().cpu().numpy()
+        assert rel_err(got, ref) <= TOL[dtype], (name, relu)
+        if relu:
+            assert (got >= 0).all()
+    # with gradients asked for, the extras are torch operations behind the same interface
+    xg = x.to(DEV).requires_grad_(True)
+    out = spatially_sparse_conv(_voxels(items, xg), w.to(DEV), 3, bias=bias.to(DEV), residual=res.to(DEV), relu=True)
+    out.feature_tensor.sum().backward()
+    assert xg.grad is not None and rel_err(out.feature_tensor.float().detach().cpu().numpy(),
+                                           np.maximum(want + res.double().numpy(), 0.0)) <= 2 * TOL[dtype]
+
+
 def test_conv_dense_cube_equals_conv3d():
     """Textbook anchor: on a fully occupied cube with zero padding the sparse convolution is
     torch.nn.functional.conv3d (cross-correlation), W[k] <-> weight[:, :, i, j, kk].T with

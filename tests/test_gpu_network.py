@@ -134,9 +134,9 @@ def _wrap_every_conv(net, check):
     for m in _conv_modules(net):
         plain = m.forward
 
-        def checked(x, *rest, _m=m, _plain=plain):
-            y = _plain(x, *rest)
-            check(_m, x, y)
+        def checked(x, *rest, _m=m, _plain=plain, **extras):
+            y = _plain(x, *rest, **extras)
+            check(_m, x, y, extras)
             return y
 
         m.forward = checked
@@ -168,7 +168,7 @@ def test_baseline_unet_every_layer_matches_oracle(oracle):
     net = _baseline_net(dtype)
     errors, maps = [], []
 
-    def check(m, x, y):
+    def check(m, x, y, extras):
         if int(np.prod(m.kernel_size)) == 1:
             return
         in_bc = x.batch_indexed_coordinates.cpu().numpy()
@@ -185,17 +185,39 @@ def test_baseline_unet_every_layer_matches_oracle(oracle):
         w = m.weight.detach().to(dtype).double().cpu().numpy()
         want = oracle.explicit_conv_f64(x.feature_tensor.double().cpu().numpy(), w, im, om, off, iden, len(out_bc))
         want = want + m.bias.detach().to(dtype).double().cpu().numpy()
+        # the block's shortcut and the ReLU ride in the convolution's epilogue
+        if extras.get("residual") is not None:
+            want = want + extras["residual"].feature_tensor.double().cpu().numpy()
+            fused.append("residual")
+        if extras.get("relu"):
+            want = np.maximum(want, 0.0)
+            fused.append("relu")
         errors.append(rel_err(y.feature_tensor.double().cpu().numpy(), want))
 
+    fused = []
     _wrap_every_conv(net, check)
     x = _voxels_of([synthetic.indoor_scene(60 + b, 15_000, 0.05) for b in range(4)], 3, dtype, seed=12)
     y = net(x)
     assert len(errors) == 41  # sparse convolutions; the four 1x1 shortcuts are dense products
     assert max(errors) <= 1e-2, errors
+    assert fused.count("relu") == 41 and fused.count("residual") == 16  # every block's second convolution
     assert len(set(maps)) == 13  # 3^3 maps at five resolutions, four strided, four transposed
     assert y.feature_tensor.shape == (len(x), 32) and y.feature_tensor.dtype == dtype
     assert torch.equal(y.coordinate_tensor, x.coordinate_tensor)
     assert bool(torch.isfinite(y.feature_tensor).all())
+
+
+def test_fused_epilogues_give_the_network_of_separate_elementwise_kernels():
+    """The same network with ReLU and the blocks' shortcuts as torch operations after every
+    convolution (one more rounding each): the outputs agree to bf16 accuracy over the depth of
+    the network."""
+    from bench import _UNet
+    dtype = torch.bfloat16
+    x = _voxels_of([synthetic.indoor_scene(70 + b, 12_000, 0.05) for b in range(2)], 3, dtype, seed=13)
+    fused = _UNet(torch.device(DEV), dtype, seed=5, fused=True)(x).feature_tensor.float()
+    plain = _UNet(torch.device(DEV), dtype, seed=5, fused=False)(x).feature_tensor.float()
+    assert float((fused - plain).abs().max()) <= 3e-2 * float(plain.abs().max())
+    assert bool((fused >= 0).all())
 
 
 def test_baseline_unet_full_size_every_layer_matches_plain_torch():
@@ -207,7 +229,7 @@ def test_baseline_unet_full_size_every_layer_matches_plain_torch():
     net = _baseline_net(dtype)
     errors, seen = [], {}
 
-    def check(m, x, y):
+    def check(m, x, y, extras):
         if int(np.prod(m.kernel_size)) == 1:
             return
         n_in, n_out = len(x), len(y)
@@ -231,6 +253,10 @@ def test_baseline_unet_full_size_every_layer_matches_plain_torch():
                 assert torch.equal(torch.sort(km.out_maps).values, torch.arange(n_out, dtype=torch.int32, device=DEV))
         w = m.weight.detach().to(dtype)
         want = torch_explicit_fp32(x.feature_tensor, w, km, n_out) + m.bias.detach().to(dtype).float()
+        if extras.get("residual") is not None:
+            want = want + extras["residual"].feature_tensor.float()
+        if extras.get("relu"):
+            want = torch.relu(want)
         scale = float(want.abs().max())
         errors.append(float((y.feature_tensor.float() - want).abs().max()) / max(scale, 1e-30))
 

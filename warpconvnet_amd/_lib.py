@@ -44,6 +44,8 @@ SIGNATURES = {
     "wcn_conv_set_timing_events": (ctypes.c_int, [_vp, _vp]),
     "wcn_sparse_conv_fwd": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                            _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
+    "wcn_sparse_conv_fwd_fused": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
+                                                 _vp, _i64p, _i32, _i32, _vp, _vp, _i32, _vp, _i64, _vp, _sz, _vp]),
     "wcn_sparse_conv_fwd_static": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                                   _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp]),
     "wcn_pairs_sort_workspace_bytes": (_sz, [_i64, _i32, _i64]),

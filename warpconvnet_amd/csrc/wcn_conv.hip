@@ -385,7 +385,10 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int lr = wrow + rb * 16 + kgrp * 4 + r;
-          stage[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC] = from_float<T>(acc[rb][nb][r] + bv);
+          float v = acc[rb][nb][r] + bv;
+          if ((a.residual || a.relu) && m0 + lr < a.num_out && n0 + col < a.c_out)
+            v = finish_sum<T>(v, a.residual, a.relu, m0 + lr, a.c_out, n0 + col);
+          stage[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC] = from_float<T>(v);
         }
       }
     __syncthreads();
@@ -406,7 +409,8 @@ __global__ void __launch_bounds__(THREADS, 2) conv_fwd(ConvArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int64_t orow = m0 + wrow + rb * 16 + kgrp * 4 + r;
-          if (orow < a.num_out) out[orow * a.c_out + col] = from_float<T>(acc[rb][nb][r] + bv);
+          if (orow < a.num_out)
+            out[orow * a.c_out + col] = from_float<T>(finish_sum<T>(acc[rb][nb][r] + bv, a.residual, a.relu, orow, a.c_out, col));
         }
       }
   }
@@ -718,7 +722,12 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
         const int col = nb * 16 + kgrp * 4;
         T v[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = from_float<T>(acc[rb][nb][r] + bias_v[nb][r]);
+        for (int r = 0; r < 4; ++r) {
+          float f = acc[rb][nb][r] + bias_v[nb][r];
+          if ((a.residual || a.relu) && m0 + lr < a.num_out && n0 + col + r < a.c_out)
+            f = finish_sum<T>(f, a.residual, a.relu, m0 + lr, a.c_out, n0 + col + r);
+          v[r] = from_float<T>(f);
+        }
         if (staged) {
           *reinterpret_cast<uint2*>(&stage[lr * CK + lds_part(lr, col / VEC) * VEC + col % VEC]) =
               *reinterpret_cast<const uint2*>(v);
@@ -862,7 +871,8 @@ __global__ void __launch_bounds__(RING_THREADS, 4) conv_fwd_ring(ConvArgs a) {
 template <typename T>
 __global__ void __launch_bounds__(256) conv_split_reduce(const float* __restrict__ partial, int slices,
                                                          int64_t num_out, int c_out, int c_out_pad,
-                                                         const T* __restrict__ bias, T* __restrict__ out) {
+                                                         const T* __restrict__ bias, T* __restrict__ out,
+                                                         const void* residual, int relu) {
   const int quads = c_out_pad / 4;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= num_out * quads) return;
@@ -875,7 +885,8 @@ __global__ void __launch_bounds__(256) conv_split_reduce(const float* __restrict
 #pragma unroll
   for (int r = 0; r < 4; ++r)
     if (col + r < c_out)
-      out[m * c_out + col + r] = from_float<T>(sum[r] + (bias ? to_float(bias[col + r]) : 0.f));
+      out[m * c_out + col + r] = from_float<T>(finish_sum<T>(sum[r] + (bias ? to_float(bias[col + r]) : 0.f),
+                                                             residual, relu, m, c_out, col + r));
 }
 
 // group_start[k][g] = number of pairs of offset k with out_maps < 64 * g (binary search; needs
@@ -1175,7 +1186,7 @@ int launch_conv(const ConvArgs& a, hipStream_t s) {
       const int64_t items = a.num_out * (a.c_out_pad / 4);
       hipLaunchKernelGGL(conv_split_reduce<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s,
                          (const float*)a.partial, (int)slices, a.num_out, a.c_out, a.c_out_pad,
-                         (const T*)a.bias, (T*)a.out);
+                         (const T*)a.bias, (T*)a.out, a.residual, a.relu);
     }
   } else {
     hipLaunchKernelGGL(conv_fwd<T>, grid, dim3(THREADS), 0, s, a);
@@ -1346,7 +1357,8 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
                     const int64_t* host_offsets, int32_t identity_offset, int32_t out_maps_ascend,
                     const int32_t* group_start_or_null, void* out, int64_t num_out,
                     void* workspace, size_t workspace_bytes, int weight_as_stored,
-                    int flip_offsets, bool no_copy_commands, void* stream) {
+                    int flip_offsets, bool no_copy_commands, void* stream,
+                    const void* residual_or_null = nullptr, int relu = 0) {
   if (dtype < 0 || dtype > 2 || (weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32))
     return WCN_ERR_INVALID_ARGUMENT;
   if (num_in < 0 || num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || c_in < 1 ||
@@ -1384,6 +1396,8 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   a.Wt = w.Wt;
   a.zeros = w.zeros;
   a.bias = bias_or_null;
+  a.residual = residual_or_null;
+  a.relu = relu ? 1 : 0;
   a.out = out;
   a.num_in = num_in;
   a.num_out = num_out;
@@ -1532,6 +1546,21 @@ int wcn_sparse_conv_fwd(const void* features, int64_t num_in, int32_t c_in, int3
   return conv_run(features, num_in, c_in, dtype, weight, weight_dtype, num_offsets, c_out,
                   bias_or_null, in_maps, out_maps, host_offsets, identity_offset, out_maps_ascend,
                   group_start_or_null, out, num_out, workspace, workspace_bytes, 0, 0, false, stream);
+}
+
+int wcn_sparse_conv_fwd_fused(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                              const void* weight, int32_t weight_dtype, int32_t num_offsets,
+                              int32_t c_out, const void* bias_or_null, const int32_t* in_maps,
+                              const int32_t* out_maps, const int64_t* host_offsets,
+                              int32_t identity_offset, int32_t out_maps_ascend,
+                              const int32_t* group_start_or_null, const void* residual_or_null,
+                              int32_t relu, void* out, int64_t num_out, void* workspace,
+                              size_t workspace_bytes, void* stream) {
+  if (residual_or_null && residual_or_null == out) return WCN_ERR_INVALID_ARGUMENT;  // rows are read and written by different threads
+  return conv_run(features, num_in, c_in, dtype, weight, weight_dtype, num_offsets, c_out,
+                  bias_or_null, in_maps, out_maps, host_offsets, identity_offset, out_maps_ascend,
+                  group_start_or_null, out, num_out, workspace, workspace_bytes, 0, 0, false, stream,
+                  residual_or_null, relu);
 }
 
 int wcn_sparse_conv_dgrad(const void* grad_out, int64_t num_out, int32_t c_out, int32_t dtype,

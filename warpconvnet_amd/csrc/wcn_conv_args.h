@@ -26,6 +26,11 @@ struct ConvArgs {
   // partial[slice][row][c_out_pad] and conv_split_reduce adds them in slice order.
   int32_t split;
   float* partial;
+  // What the epilogue does besides bias and rounding (wcn_sparse_conv_fwd_fused): add a row of
+  // `residual` (num_out x c_out, the element type of the features) and / or clamp at zero, both
+  // on the fp32 sums before the one rounding.
+  const void* residual;
+  int32_t relu;
 };
 
 

@@ -245,7 +245,8 @@ __global__ void __launch_bounds__(DENSE_WAVES * 64) conv_fwd_dense(ConvArgs a, i
         if (row < tile_rows) {
           T t[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) t[e] = from_float<T>(acc[rb][cb][e] + b[e]);
+          for (int e = 0; e < 4; ++e)
+            t[e] = from_float<T>(finish_sum<T>(acc[rb][cb][e] + b[e], a.residual, a.relu, m0 + row, a.c_out, col + e));
           *reinterpret_cast<uint2*>(out + (m0 + row) * a.c_out + col) = *reinterpret_cast<const uint2*>(t);
         }
       }

@@ -291,6 +291,11 @@ __global__ void __launch_bounds__(WAVES * 64) conv_fwd_group(ConvArgs a) {
         const int col = cpart * 8;
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += bias_v[e];
+        if (a.residual || a.relu) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (col + e < a.c_out) v[e] = finish_sum<T>(v[e], a.residual, a.relu, m, a.c_out, col + e);
+        }
         T* dst = out + m * a.c_out + col;
         if (a.vec_out && col + 8 <= a.c_out) {
           T t[8];

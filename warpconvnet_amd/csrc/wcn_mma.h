@@ -17,6 +17,14 @@ template <typename T>
 __device__ __forceinline__ T from_float(float v) {
   return (T)v;
 }
+// The fused part of a contraction's epilogue, on the fp32 sum (bias already added) of output row
+// `row`, channel `col`: plus the residual's entry, then clamped at zero (a NaN stays a NaN).
+template <typename T>
+__device__ __forceinline__ float finish_sum(float v, const void* residual, int relu, int64_t row, int c_out, int col) {
+  if (residual) v += to_float(static_cast<const T*>(residual)[row * c_out + col]);
+  if (relu) v = v < 0.f ? 0.f : v;
+  return v;
+}
 
 // MFMA operand handling per element type.  16x16x32 (f16/bf16): lane l holds row (l & 15),
 // k = 8 * (l >> 4) .. +7 of A and column (l & 15), same k of B; 16x16x4 (f32): lane l holds

@@ -131,14 +131,19 @@ def _pairs_sorted(km: IntSearchResult, by: str, num_rows: int):
 @torch.no_grad()
 def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSearchResult,
                         num_out_coords: int, bias: Optional[Tensor] = None,
-                        compute_dtype: Optional[torch.dtype] = None) -> Tensor:
+                        compute_dtype: Optional[torch.dtype] = None,
+                        residual: Optional[Tensor] = None, relu: bool = False) -> Tensor:
     """out = bias + sum_k scatter(X[in_k] @ W[k]) on the GPU (replaces the per-offset loops of
     sparse_conv.py:281-311 / :358-415 / :495-544 and the native GEMMs they call).
 
     A map whose out_maps does not ascend inside every offset (a hand-made one, the exchanged map
     of a transposed convolution) is re-ordered once; that step takes at most one pair per (offset,
     output row), which every kernel map of duplicate-free coordinates satisfies, and raises
-    ValueError for lists that hold more (the reference would add all of them up)."""
+    ValueError for lists that hold more (the reference would add all of them up).
+
+    `residual` ((num_out_coords, c_out), added to the sums) and `relu` (clamp at zero) are done in
+    the kernel's epilogue before the one rounding (wcn_sparse_conv_fwd_fused): what a residual
+    block does with two more elementwise kernels after the convolution.  Not in the reference."""
     require_device(in_features, "in_features")
     if in_features.ndim != 2 or weight.ndim != 3 or weight.shape[1] != in_features.shape[1]:
         raise ValueError(f"shape mismatch: features {tuple(in_features.shape)}, "
@@ -183,6 +188,20 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
                                         num_pairs, ascend)
     ws = workspace(nbytes, device)
     iden = -1 if km.identity_map_index is None else int(km.identity_map_index)
+    if residual is not None or relu:
+        r = None
+        if residual is not None:
+            if tuple(residual.shape) != (num_out_coords, c_out):
+                raise ValueError(f"residual has shape {tuple(residual.shape)}, the output {(num_out_coords, c_out)}")
+            require_device(residual, "residual")
+            r = residual.detach().to(x.dtype).contiguous()
+        check(L.wcn_sparse_conv_fwd_fused(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(w),
+                                          DTYPE_CODE[w.dtype], K, c_out, ptr(b), ptr(in_maps),
+                                          ptr(out_maps), host_offsets, iden, ascend, group_start,
+                                          ptr(r), 1 if relu else 0, ptr(out), num_out_coords,
+                                          ptr(ws), ws.numel(), stream_ptr(device)),
+              "wcn_sparse_conv_fwd_fused")
+        return out if out.dtype == in_features.dtype else out.to(in_features.dtype)
     check(L.wcn_sparse_conv_fwd(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(w),
                                 DTYPE_CODE[w.dtype], K, c_out, ptr(b), ptr(in_maps),
                                 ptr(out_maps), host_offsets, iden, ascend, group_start,
@@ -414,9 +433,16 @@ def spatially_sparse_conv(
     compute_dtype: Optional[torch.dtype] = None,
     implicit_matmul_fwd_block_size: Optional[int] = 16,
     implicit_matmul_bwd_block_size: Optional[int] = 16,
+    residual: Optional[Union[Tensor, Voxels]] = None,
+    relu: bool = False,
 ) -> Voxels:
     """Sparse convolution of a Voxels tensor with weight (K, C_in, C_out)
-    (reference: sparse_conv.py:1662-1805)."""
+    (reference: sparse_conv.py:1662-1805).
+
+    `residual` (features of the output's shape, or a Voxels tensor holding them) and `relu` are not
+    in the reference: out = act(conv(x) + bias + residual).  Without gradients they are carried out
+    in the contraction's epilogue, on the fp32 sums before the one rounding; with gradients (and
+    for 1x1x1 kernels) they are the torch operations a caller would write after the call."""
     if not isinstance(input_sparse_tensor, Voxels):
         raise TypeError("Native spatially_sparse_conv expects input_sparse_tensor of type Voxels, "
                         f"got {type(input_sparse_tensor)}")
@@ -430,11 +456,19 @@ def spatially_sparse_conv(
     _kernel_dilation = ntuple(kernel_dilation, ndim=ndim)
     _stride = ntuple(stride, ndim=ndim)
 
+    if isinstance(residual, Voxels):
+        residual = residual.feature_tensor
+
+    def after(out_features):  # the unfused form of the two extras
+        if residual is not None:
+            out_features = out_features + residual.to(out_features.dtype)
+        return torch.relu(out_features) if relu else out_features
+
     if int(np.prod(_kernel_size)) == 1 and int(np.prod(_stride)) == 1:
         out_features = input_sparse_tensor.feature_tensor @ weight[0]
         if bias is not None:
             out_features = out_features + bias.to(out_features.dtype)
-        return input_sparse_tensor.replace(batched_features=out_features)
+        return input_sparse_tensor.replace(batched_features=after(out_features))
 
     in_tensor_stride = input_sparse_tensor.tensor_stride
     if in_tensor_stride is None:
@@ -481,15 +515,23 @@ def spatially_sparse_conv(
             implicit_matmul_bwd_block_size)
         if bias is not None:
             out_features = out_features + bias.to(out_features.dtype)
+        out_features = after(out_features)
     elif num_out_coords == 0 or features.shape[0] == 0:
         out_features = torch.zeros((num_out_coords, weight.shape[-1]), dtype=features.dtype,
                                    device=features.device)
         if bias is not None:
             out_features = out_features + bias.to(features.dtype)
+        out_features = after(out_features)
     else:
-        # inference: the bias add is fused into the contraction's epilogue
+        # inference: bias, residual and clamp are fused into the contraction's epilogue
+        needs_residual_grad = residual is not None and torch.is_grad_enabled() and residual.requires_grad
+        fused = not needs_residual_grad
         out_features = sparse_conv_forward(features, weight, kernel_map, num_out_coords, bias=bias,
-                                           compute_dtype=effective_compute_dtype)
+                                           compute_dtype=effective_compute_dtype,
+                                           residual=residual if fused else None,
+                                           relu=relu and fused)
+        if not fused:
+            out_features = after(out_features)
 
     # The output's coordinate object.  Where the output rows are an existing tensor's (stride 1,
     # or a given output tensor) that tensor's coordinate object is reused, and a newly made one is

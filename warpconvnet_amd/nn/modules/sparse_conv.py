@@ -86,7 +86,10 @@ class SpatiallySparseConv(nn.Module):
         return s
 
     def forward(self, input_sparse_tensor: Voxels,
-                output_spatially_sparse_tensor: Optional[Voxels] = None) -> Voxels:
+                output_spatially_sparse_tensor: Optional[Voxels] = None, *,
+                residual=None, relu: bool = False) -> Voxels:
+        """`residual` and `relu` (keyword only, not in the reference): act(conv(x) + residual), done
+        in the convolution's epilogue where no gradient is asked for."""
         return spatially_sparse_conv(
             input_sparse_tensor, weight=self.weight, kernel_size=self.kernel_size,
             stride=self.stride, kernel_dilation=self.dilation, bias=self.bias,
@@ -95,7 +98,8 @@ class SpatiallySparseConv(nn.Module):
             transposed=self.transposed, fwd_algo=self.fwd_algo, bwd_algo=self.bwd_algo,
             stride_mode=self.stride_mode, order=self.order, compute_dtype=self.compute_dtype,
             implicit_matmul_fwd_block_size=self.implicit_matmul_fwd_block_size,
-            implicit_matmul_bwd_block_size=self.implicit_matmul_bwd_block_size)
+            implicit_matmul_bwd_block_size=self.implicit_matmul_bwd_block_size,
+            residual=residual, relu=relu)
 
 
 class SparseConv2d(SpatiallySparseConv):
