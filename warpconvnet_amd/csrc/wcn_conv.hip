@@ -1441,6 +1441,7 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   const size_t es = elem_size(dtype);
   a.vec_in = (((size_t)c_in * es) % 16 == 0 && ((uintptr_t)features % 16) == 0) ? 1 : 0;
   a.vec_out = (((size_t)c_out * es) % 16 == 0 && ((uintptr_t)out % 16) == 0) ? 1 : 0;
+  a.vec_res = (a.residual && ((size_t)c_out * es) % 16 == 0 && ((uintptr_t)a.residual % 16) == 0) ? 1 : 0;
   a.flat_in = (c_in % ck_of(dtype) == 0 && (uint64_t)num_in * c_in * es < (1ull << 32)) ? 1 : 0;
   a.partial = w.partial;
   a.split = (a.vec_in && w.partial != nullptr) ? 1 : 0;

@@ -31,6 +31,7 @@ struct ConvArgs {
   // on the fp32 sums before the one rounding.
   const void* residual;
   int32_t relu;
+  int32_t vec_res;  // rows of `residual` are 16-byte aligned and a whole number of 16-byte vectors
 };
 
 

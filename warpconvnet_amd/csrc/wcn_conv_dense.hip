@@ -244,9 +244,14 @@ __global__ void __launch_bounds__(DENSE_WAVES * 64) conv_fwd_dense(ConvArgs a, i
         const int row = wave * WROWS_OUT + rb * 16 + c;
         if (row < tile_rows) {
           T t[4];
+          float r[4] = {0.f, 0.f, 0.f, 0.f};  // rows are whole 16-byte vectors here: 128 or 256 channels
+          if (a.residual) load_floats<T, 4>(static_cast<const T*>(a.residual) + (m0 + row) * a.c_out + col, r);
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            t[e] = from_float<T>(finish_sum<T>(acc[rb][cb][e] + b[e], a.residual, a.relu, m0 + row, a.c_out, col + e));
+          for (int e = 0; e < 4; ++e) {
+            float f = acc[rb][cb][e] + b[e] + r[e];
+            if (a.relu) f = f < 0.f ? 0.f : f;
+            t[e] = from_float<T>(f);
+          }
           *reinterpret_cast<uint2*>(out + (m0 + row) * a.c_out + col) = *reinterpret_cast<const uint2*>(t);
         }
       }
@@ -321,6 +326,7 @@ int launch_dense_typed(const ConvArgs& a, hipStream_t s) {
 // and runs on one CU from the first offset to the last).
 bool wcn_conv_dense_takes(const ConvArgs& a, int dtype) {
   if (dtype == WCN_DTYPE_F32 || !a.vec_in || !a.vec_out || !a.group_start) return false;
+  if (a.residual && !a.vec_res) return false;  // the epilogue reads the residual in 8-byte pieces
   if (a.c_in != a.c_in_pad || a.c_in % 64 != 0 || a.c_in < 128) return false;
   if (a.c_out != a.c_out_pad || (a.c_out != 128 && a.c_out != 256)) return false;
   if (a.K < 1 || a.K > 64 || a.num_in >= (1ll << 31) || a.num_out >= (1ll << 31)) return false;

@@ -209,7 +209,9 @@ __global__ void __launch_bounds__(WAVES * 64) conv_fwd_group(ConvArgs a) {
     };
 
     // the sums start as the identity offset's product (every row reads its own input row; the
-    // map's pairs of that offset are ignored), or as zeros
+    // map's pairs of that offset are ignored), or as zeros, plus the row of the residual if one
+    // is given (requested here, where the group's first requests are on their way anyway, and not
+    // in the epilogue, where the wave would wait for it with nothing else to do)
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
       const int64_t m = m0 + rb * 16 + pr;
@@ -218,9 +220,22 @@ __global__ void __launch_bounds__(WAVES * 64) conv_fwd_group(ConvArgs a) {
       if (with_identity) xv = x_operand(here ? (int32_t)m : 0);
 #pragma unroll
       for (int cb = 0; cb < NCB; ++cb) {
+        float start[4] = {0.f, 0.f, 0.f, 0.f};
+        const int col = cb * 16 + kg * 4;
+        if (a.residual && m < a.num_out && col < a.c_out) {
+          const T* rs = static_cast<const T*>(a.residual) + m * a.c_out + col;
+          if (a.vec_res) {  // whole 16-byte vectors per row: c_out is a multiple of 8
+            load_floats<T, 4>(rs, start);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (col + e < a.c_out) start[e] = to_float(rs[e]);
+          }
+        }
         f32x4 d = (f32x4){0.f, 0.f, 0.f, 0.f};
         if (with_identity) d = Op::mma(s_w[(a.identity * NCB + cb) * 64 + lane], xv, d);
-        *granule(rb * 16 + pr, cb * 4 + kg) = here ? d : (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (!here) d = (f32x4){0.f, 0.f, 0.f, 0.f};
+        *granule(rb * 16 + pr, cb * 4 + kg) = d + (f32x4){start[0], start[1], start[2], start[3]};
       }
     }
 
@@ -291,10 +306,9 @@ __global__ void __launch_bounds__(WAVES * 64) conv_fwd_group(ConvArgs a) {
         const int col = cpart * 8;
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += bias_v[e];
-        if (a.residual || a.relu) {
+        if (a.relu) {  // (the residual went into the sums at the group's start)
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (col + e < a.c_out) v[e] = finish_sum<T>(v[e], a.residual, a.relu, m, a.c_out, col + e);
+          for (int e = 0; e < 8; ++e) v[e] = v[e] < 0.f ? 0.f : v[e];
         }
         T* dst = out + m * a.c_out + col;
         if (a.vec_out && col + 8 <= a.c_out) {

@@ -598,10 +598,24 @@ __global__ void __launch_bounds__((NW + 1) * 64) conv_fwd_pack(ConvArgs a, int n
             float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] += bias_v[e];
-            if (a.residual || a.relu) {
+            if (a.residual) {
+              const T* rs = static_cast<const T*>(a.residual) + (m0 + row) * a.c_out + col;
+              if (a.vec_res && col + 8 <= a.c_out) {
+                constexpr int PER = 16 / sizeof(T);  // entries per 16-byte load
+                float r[8];
 #pragma unroll
-              for (int e = 0; e < 8; ++e)
-                if (col + e < a.c_out) v[e] = finish_sum<T>(v[e], a.residual, a.relu, m0 + row, a.c_out, col + e);
+                for (int h = 0; h < 8 / PER; ++h) load_floats<T, PER>(rs + h * PER, *reinterpret_cast<float (*)[PER]>(r + h * PER));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += r[e];
+              } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                  if (col + e < a.c_out) v[e] += to_float(rs[e]);
+              }
+            }
+            if (a.relu) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[e] = v[e] < 0.f ? 0.f : v[e];
             }
             T* dst = out + (m0 + row) * a.c_out + col;
             if (a.vec_out && col + 8 <= a.c_out) {

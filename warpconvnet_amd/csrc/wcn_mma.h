@@ -17,6 +17,18 @@ template <typename T>
 __device__ __forceinline__ T from_float(float v) {
   return (T)v;
 }
+// N consecutive entries of a residual row as floats (N * sizeof(T) = 8 or 16 bytes: one load).
+template <typename T, int N>
+__device__ __forceinline__ void load_floats(const T* p, float (&v)[N]) {
+  static_assert(N * sizeof(T) == 8 || N * sizeof(T) == 16, "one 8- or 16-byte load");
+  T t[N];
+  if (N * sizeof(T) == 16)
+    *reinterpret_cast<u32x4*>(t) = *reinterpret_cast<const u32x4*>(p);
+  else
+    *reinterpret_cast<uint2*>(t) = *reinterpret_cast<const uint2*>(p);
+#pragma unroll
+  for (int e = 0; e < N; ++e) v[e] = to_float(t[e]);
+}
 // The fused part of a contraction's epilogue, on the fp32 sum (bias already added) of output row
 // `row`, channel `col`: plus the residual's entry, then clamped at zero (a NaN stays a NaN).
 template <typename T>
