@@ -339,13 +339,20 @@ class _UNet:
     convolutions) and four up stages (transposed 2x2x2 stride-2 convolution, skip concatenation,
     two residual blocks, 1x1 shortcut where the channel count changes).  Batch norm is folded into
     the convolutions' weight and bias; ReLU and the residual adds ride in the convolutions'
-    epilogues (`fused=False`: as torch elementwise ops after every convolution)."""
+    epilogues (`fused=False`: as torch elementwise ops after every convolution).  The weights do
+    not change between passes, so the layers keep the kernels' tiles of their weight
+    (`keep_tiles=False`: made again by one more kernel in every call)."""
 
-    def __init__(self, dev, dtype, seed=0, fused=True):
+    def __init__(self, dev, dtype, seed=0, fused=True, keep_tiles=True):
         from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d
         self.fused = fused
         torch.manual_seed(seed)
-        mk = lambda *a, **k: SparseConv3d(*a, bias=True, **k).to(dev).to(dtype)  # noqa: E731
+
+        def mk(*a, **k):
+            conv = SparseConv3d(*a, bias=True, **k).to(dev).to(dtype)
+            conv.keep_prepared_weight = keep_tiles
+            return conv
+
         enc = (32, 64, 128, 256)
         self.stem = mk(3, 32, 3)
         self.down, self.enc_blocks = [], []
@@ -406,25 +413,29 @@ def unet_config(dev, steps, warmup):
     coords = torch.as_tensor(np.concatenate(items), dtype=torch.int32, device=dev)
     n = coords.shape[0]
     feats = torch.randn(n, 3, generator=torch.Generator().manual_seed(11)).to(torch.bfloat16).to(dev)
+    def timed(net):
+        def run():
+            return net(Voxels(coords, feats, offsets=torch.as_tensor(np.asarray(offsets))))
+
+        for _ in range(warmup):
+            out = run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            out = run()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps, out
+
     net = _UNet(dev, torch.bfloat16)
-
-    def run():
-        return net(Voxels(coords, feats, offsets=torch.as_tensor(np.asarray(offsets))))
-
-    for _ in range(warmup):
-        out = run()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        out = run()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms, out = timed(net)
+    ms_every_call, out_every_call = timed(_UNet(dev, torch.bfloat16, keep_tiles=False))
     assert out.feature_tensor.shape == (n, 32) and bool(torch.isfinite(out.feature_tensor).all())
+    assert torch.equal(out.feature_tensor, out_every_call.feature_tensor)
     convs = [net.stem] + net.down + net.up + [m for stage in net.enc_blocks + net.dec_blocks
                                              for blk in stage for m in blk if m is not None]
     sparse = sum(1 for m in convs if int(np.prod(m.kernel_size)) > 1)
     return {"num_voxels": n, "sparse_convolutions": sparse, "pointwise_convolutions": len(convs) - sparse,
-            "ms_per_pass": ms,
+            "ms_per_pass": ms, "ms_per_pass_weight_tiles_made_in_every_call": ms_every_call,
             "voxels_per_s": n / (ms * 1e-3)}
 
 

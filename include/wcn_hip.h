@@ -236,6 +236,35 @@ int wcn_sparse_conv_fwd_fused(const void* features, int64_t num_in, int32_t c_in
                               int32_t relu, void* out, int64_t num_out, void* workspace,
                               size_t workspace_bytes, void* stream);
 
+/* The forward contraction with the weight's tiles made ahead of the call, for weights that stay
+ * the same over many calls (inference, the layers of a network between two optimiser steps).
+ * wcn_sparse_conv_fwd turns W (K, c_in, c_out) into zero-padded transposed tiles in the kernels'
+ * dtype at the start of every call (one more kernel per call: 4 us of a 30 us layer);
+ * wcn_conv_prepare_weight does that once into `prepared` (wcn_conv_prepared_weight_bytes bytes of
+ * device memory the caller keeps; to be made again whenever W changes), and
+ * wcn_sparse_conv_fwd_prepared enqueues the contraction alone.  It takes maps as the map builder
+ * leaves them: out_maps ascending inside every offset, `group_start` (wcn_kmap_group_start) and
+ * `device_offsets` = the (K + 1) offsets as int64 in device memory (the first K + 1 words of the
+ * map builder's workspace; equal to host_offsets).  residual_or_null / relu as in
+ * wcn_sparse_conv_fwd_fused; results identical to that entry's bit for bit.  Replaces the same
+ * reference path as wcn_sparse_conv_fwd (sparse_conv.py:495-544 + the native GEMMs it calls, which
+ * read the caller's weight as it is and need no such step). */
+size_t wcn_conv_prepared_weight_bytes(int32_t num_offsets, int32_t c_in, int32_t c_out, int32_t dtype);
+
+int wcn_conv_prepare_weight(const void* weight, int32_t weight_dtype, int32_t num_offsets, int32_t c_in,
+                            int32_t c_out, int32_t dtype, void* prepared, size_t prepared_bytes,
+                            void* stream);
+
+int wcn_sparse_conv_fwd_prepared(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                                 const void* prepared_weight, size_t prepared_bytes,
+                                 int32_t num_offsets, int32_t c_out, const void* bias_or_null,
+                                 const int32_t* in_maps, const int32_t* out_maps,
+                                 const int64_t* host_offsets, const int64_t* device_offsets,
+                                 int32_t identity_offset, const int32_t* group_start,
+                                 const void* residual_or_null, int32_t relu, void* out,
+                                 int64_t num_out, void* workspace, size_t workspace_bytes,
+                                 void* stream);
+
 /* wcn_sparse_conv_fwd for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
  * Same arguments and results as wcn_sparse_conv_fwd, minus the workspace: the scratch memory is a

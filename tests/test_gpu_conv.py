@@ -189,6 +189,55 @@ def test_residual_and_relu_in_the_epilogue(oracle, name, dtype, c_in, c_out, n, 
                                            np.maximum(want + res.double().numpy(), 0.0)) <= 2 * TOL[dtype]
 
 
+@pytest.mark.parametrize("name,dtype,c_in,c_out,n,extent,kernel", FUSED_CASES, ids=[c[0] for c in FUSED_CASES])
+def test_prepared_weight_tiles_give_the_same_bits(name, dtype, c_in, c_out, n, extent, kernel):
+    """keep_prepared_weight: the tiles of the weight made once and kept on the tensor
+    (wcn_conv_prepare_weight + wcn_sparse_conv_fwd_prepared) against the call that makes them every
+    time, bit for bit, through every kernel; the tiles follow a change of the weight."""
+    from warpconvnet_amd._lib import lib
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    items = [synthetic.random_cloud(81, n, extent)[:, 1:]]
+    bc = synthetic.batch_indexed(items)
+    x = normal_features(len(bc), c_in, seed=41, dtype=dtype)
+    w = kaiming_weight(27, c_in, c_out, seed=42, dtype=dtype).to(DEV)
+    bias = (torch.randn(c_out, generator=torch.Generator().manual_seed(43)) * 0.1).to(dtype).to(DEV)
+    res = normal_features(len(bc), c_out, seed=44, dtype=dtype).to(DEV)
+    vox = _voxels(items, x)
+    for residual, relu in ((None, False), (res, True)):
+        plain = spatially_sparse_conv(vox, w, 3, bias=bias, residual=residual, relu=relu).feature_tensor
+        for _ in range(2):  # the second call finds the tiles
+            kept = spatially_sparse_conv(vox, w, 3, bias=bias, residual=residual, relu=relu,
+                                         keep_prepared_weight=True).feature_tensor
+            assert lib().wcn_conv_last_kernel().decode().startswith(kernel), lib().wcn_conv_last_kernel()
+            assert torch.equal(plain, kept), (name, relu)
+    tiles = w._wcn_prepared[1]
+    w.mul_(0.5)  # the version counter moves: new tiles
+    plain = spatially_sparse_conv(vox, w, 3, bias=bias).feature_tensor
+    kept = spatially_sparse_conv(vox, w, 3, bias=bias, keep_prepared_weight=True).feature_tensor
+    assert w._wcn_prepared[1] is not tiles and torch.equal(plain, kept)
+
+
+def test_prepared_weight_tiles_over_an_exchanged_map_and_fp32_master_weights():
+    """The transposed convolution's map (lists re-ordered by the library, offsets copied to the device
+    on first use) and a float32 weight under bfloat16 features, both with kept tiles."""
+    from warpconvnet_amd.nn.modules.sparse_conv import SparseConv3d
+    items = [synthetic.random_cloud(24 + b, 5000, 30)[:, 1:] for b in range(2)]
+    x = normal_features(sum(len(i) for i in items), 32, seed=9, dtype=torch.bfloat16)
+    fine = _voxels(items, x)
+    down = SparseConv3d(32, 64, 2, stride=2, bias=False).to(DEV)  # float32 parameters
+    up = SparseConv3d(64, 32, 2, stride=2, bias=True, transposed=True).to(DEV)
+    with torch.no_grad():
+        coarse = down(fine)
+        back = up(coarse, fine)
+        down.keep_prepared_weight = up.keep_prepared_weight = True
+        for _ in range(2):
+            coarse_kept = down(fine)
+            back_kept = up(coarse_kept, fine)
+            assert torch.equal(coarse.feature_tensor, coarse_kept.feature_tensor)
+            assert torch.equal(back.feature_tensor, back_kept.feature_tensor)
+    assert hasattr(down.weight, "_wcn_prepared") and hasattr(up.weight, "_wcn_prepared")
+
+
 def test_conv_dense_cube_equals_conv3d():
     """Textbook anchor: on a fully occupied cube with zero padding the sparse convolution is
     torch.nn.functional.conv3d (cross-correlation), W[k] <-> weight[:, :, i, j, kk].T with

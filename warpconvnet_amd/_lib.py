@@ -46,6 +46,11 @@ SIGNATURES = {
                                            _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp, _sz, _vp]),
     "wcn_sparse_conv_fwd_fused": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                                  _vp, _i64p, _i32, _i32, _vp, _vp, _i32, _vp, _i64, _vp, _sz, _vp]),
+    "wcn_conv_prepared_weight_bytes": (_sz, [_i32, _i32, _i32, _i32]),
+    "wcn_conv_prepare_weight": (ctypes.c_int, [_vp, _i32, _i32, _i32, _i32, _i32, _vp, _sz, _vp]),
+    "wcn_sparse_conv_fwd_prepared": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _sz, _i32, _i32, _vp, _vp,
+                                                    _vp, _i64p, _vp, _i32, _vp, _vp, _i32, _vp, _i64,
+                                                    _vp, _sz, _vp]),
     "wcn_sparse_conv_fwd_static": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                                   _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp]),
     "wcn_pairs_sort_workspace_bytes": (_sz, [_i64, _i32, _i64]),
@@ -109,7 +114,15 @@ def check(status: int, where: str) -> None:
         raise WcnError(status, where)
 
 
+# The current stream's handle without the Stream object torch.cuda.current_stream builds around it
+# (a few microseconds, several times per layer of a network).
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device) -> ctypes.c_void_p:
+    if _raw_stream is not None and isinstance(device, torch.device) and device.type == "cuda":
+        index = device.index if device.index is not None else torch.cuda.current_device()
+        return ctypes.c_void_p(_raw_stream(index))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 

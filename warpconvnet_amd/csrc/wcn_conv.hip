@@ -73,7 +73,7 @@ __global__ void __launch_bounds__(256) conv_prep_weight(const WT* __restrict__ W
                                                         T* __restrict__ Wt, uint32_t* __restrict__ zeros,
                                                         int64_t* __restrict__ offsets_dst,
                                                         int n_offsets, OffsetsByValue ov) {
-  if (blockIdx.x == 0) {
+  if (blockIdx.x == 0 && zeros) {
     zeros[threadIdx.x] = 0u;  // 256 threads x 4 bytes
     // the map's offsets, handed over in the kernel arguments (saves a copy command per call)
     if ((int)threadIdx.x < n_offsets) offsets_dst[threadIdx.x] = ov.v[threadIdx.x];
@@ -1347,6 +1347,30 @@ size_t wcn_conv_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_
                      out_maps_ascend ? -1 : num_pairs, nullptr);
 }
 
+// 1 KiB of zeros that no kernel writes (the source of loads that have nothing to fetch), for calls
+// that bring prepared weight tiles and so run no preparation kernel that could write such a block
+// into the workspace.  Host code uses the address hipGetSymbolAddress reports for the current
+// device, never the array's name.
+static __device__ __align__(256) uint32_t zero_page[256];
+
+namespace {
+std::mutex g_zero_page_mutex;
+void* g_zero_page_ptr[64] = {};
+
+int static_zero_page(void** ptr) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return WCN_ERR_LAUNCH;
+  std::lock_guard<std::mutex> hold(g_zero_page_mutex);
+  if (!g_zero_page_ptr[device]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(zero_page)) != hipSuccess || !p) return WCN_ERR_LAUNCH;
+    g_zero_page_ptr[device] = p;
+  }
+  *ptr = g_zero_page_ptr[device];
+  return WCN_OK;
+}
+}  // namespace
+
 // Shared body of the forward product and the input gradient.  weight_as_stored / flip_offsets
 // choose how the caller's weight becomes the kernels' tiles (see conv_prep_weight).  With
 // `no_copy_commands` the call enqueues kernels only (the offsets must then fit the kernel
@@ -1358,9 +1382,14 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
                     const int32_t* group_start_or_null, void* out, int64_t num_out,
                     void* workspace, size_t workspace_bytes, int weight_as_stored,
                     int flip_offsets, bool no_copy_commands, void* stream,
-                    const void* residual_or_null = nullptr, int relu = 0) {
-  if (dtype < 0 || dtype > 2 || (weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32))
+                    const void* residual_or_null = nullptr, int relu = 0,
+                    const int64_t* device_offsets_of_prepared = nullptr) {
+  // With device_offsets_of_prepared, `weight` is the tiles wcn_conv_prepare_weight made and the
+  // call enqueues nothing but the contraction.
+  const bool prepared = device_offsets_of_prepared != nullptr;
+  if (dtype < 0 || dtype > 2 || (!prepared && weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32))
     return WCN_ERR_INVALID_ARGUMENT;
+  if (prepared && (!out_maps_ascend || !group_start_or_null)) return WCN_ERR_INVALID_ARGUMENT;
   if (num_in < 0 || num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || c_in < 1 ||
       c_out < 1 || !weight || !workspace || !host_offsets)
     return WCN_ERR_INVALID_ARGUMENT;
@@ -1383,7 +1412,7 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   // Up to 127 offsets reach the device in the arguments of the weight preparation, which is the
   // first launch of the call: no copy command.
   const bool offsets_by_value = num_offsets + 1 <= OFFSETS_BY_VALUE;
-  if (!offsets_by_value) {
+  if (!offsets_by_value && !prepared) {
     if (no_copy_commands) return WCN_ERR_INVALID_ARGUMENT;
     if (hipMemcpyAsync(w.offsets, host_offsets, sizeof(int64_t) * (size_t)(num_offsets + 1),
                        hipMemcpyHostToDevice, s) != hipSuccess)
@@ -1410,16 +1439,24 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   a.c_out_pad = w.c_out_pad;
   a.identity = identity_offset;
   const int64_t* by_value = offsets_by_value ? host_offsets : nullptr;
-  switch (dtype) {
-    case WCN_DTYPE_F32:
-      launch_prep<float>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, by_value, s);
-      break;
-    case WCN_DTYPE_F16:
-      launch_prep<_Float16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, by_value, s);
-      break;
-    default:
-      launch_prep<__bf16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, by_value, s);
-      break;
+  if (prepared) {
+    void* zero_page_address = nullptr;
+    if (const int st = static_zero_page(&zero_page_address)) return st;
+    a.Wt = weight;
+    a.zeros = zero_page_address;
+    a.offsets = device_offsets_of_prepared;
+  } else {
+    switch (dtype) {
+      case WCN_DTYPE_F32:
+        launch_prep<float>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, by_value, s);
+        break;
+      case WCN_DTYPE_F16:
+        launch_prep<_Float16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, by_value, s);
+        break;
+      default:
+        launch_prep<__bf16>(a, weight, weight_dtype, dtype, weight_as_stored, flip_offsets, by_value, s);
+        break;
+    }
   }
 
   a.in_maps = in_maps;
@@ -1562,6 +1599,56 @@ int wcn_sparse_conv_fwd_fused(const void* features, int64_t num_in, int32_t c_in
                   bias_or_null, in_maps, out_maps, host_offsets, identity_offset, out_maps_ascend,
                   group_start_or_null, out, num_out, workspace, workspace_bytes, 0, 0, false, stream,
                   residual_or_null, relu);
+}
+
+size_t wcn_conv_prepared_weight_bytes(int32_t num_offsets, int32_t c_in, int32_t c_out, int32_t dtype) {
+  if (num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || c_in < 1 || c_out < 1 || dtype < 0 || dtype > 2)
+    return 0;
+  return wcn_align256(elem_size(dtype) * (size_t)num_offsets * round_up(c_out, TN) *
+                      round_up(c_in, ck_of(dtype)));
+}
+
+int wcn_conv_prepare_weight(const void* weight, int32_t weight_dtype, int32_t num_offsets, int32_t c_in,
+                            int32_t c_out, int32_t dtype, void* prepared, size_t prepared_bytes,
+                            void* stream) {
+  const size_t need = wcn_conv_prepared_weight_bytes(num_offsets, c_in, c_out, dtype);
+  if (need == 0 || !weight || !prepared || (weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32))
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (prepared_bytes < need) return WCN_ERR_WORKSPACE;
+  ConvArgs a = {};
+  a.K = num_offsets;
+  a.c_in = c_in;
+  a.c_out = c_out;
+  a.c_in_pad = round_up(c_in, ck_of(dtype));
+  a.c_out_pad = round_up(c_out, TN);
+  a.Wt = prepared;  // zeros and offsets stay null: the kernel then writes the tiles only
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case WCN_DTYPE_F32: launch_prep<float>(a, weight, weight_dtype, dtype, 0, 0, nullptr, s); break;
+    case WCN_DTYPE_F16: launch_prep<_Float16>(a, weight, weight_dtype, dtype, 0, 0, nullptr, s); break;
+    default: launch_prep<__bf16>(a, weight, weight_dtype, dtype, 0, 0, nullptr, s); break;
+  }
+  return hipGetLastError() == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
+}
+
+int wcn_sparse_conv_fwd_prepared(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                                 const void* prepared_weight, size_t prepared_bytes,
+                                 int32_t num_offsets, int32_t c_out, const void* bias_or_null,
+                                 const int32_t* in_maps, const int32_t* out_maps,
+                                 const int64_t* host_offsets, const int64_t* device_offsets,
+                                 int32_t identity_offset, const int32_t* group_start,
+                                 const void* residual_or_null, int32_t relu, void* out,
+                                 int64_t num_out, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+  if (residual_or_null && residual_or_null == out) return WCN_ERR_INVALID_ARGUMENT;
+  if (!device_offsets || !group_start) return WCN_ERR_INVALID_ARGUMENT;
+  const size_t need = wcn_conv_prepared_weight_bytes(num_offsets, c_in, c_out, dtype);
+  if (need == 0) return WCN_ERR_INVALID_ARGUMENT;
+  if (prepared_bytes < need) return WCN_ERR_WORKSPACE;
+  return conv_run(features, num_in, c_in, dtype, prepared_weight, dtype, num_offsets, c_out,
+                  bias_or_null, in_maps, out_maps, host_offsets, identity_offset, 1, group_start, out,
+                  num_out, workspace, workspace_bytes, 0, 0, true, stream, residual_or_null, relu,
+                  device_offsets);
 }
 
 int wcn_sparse_conv_dgrad(const void* grad_out, int64_t num_out, int32_t c_out, int32_t dtype,

@@ -29,6 +29,7 @@ class IntSearchResult:
         # per-64-row group starts.
         self._out_ascend = False
         self._group_start = None
+        self._device_offsets = None  # (K + 1) int64 copy of `offsets` in device memory, when the builder left one
         # For the gradients: whether in_maps ascends inside every offset (the map of a transposed
         # convolution: a forward map with its lists exchanged), the group starts that belong to
         # that order, and whether exchanging in and out turns offset k into offset K - 1 - k

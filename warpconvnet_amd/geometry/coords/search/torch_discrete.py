@@ -117,8 +117,12 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
         # map (a copy of about K * M / 16 bytes; the workspace, whose probe results are K * M * 4
         # bytes, goes back to the allocator).  The copy is enqueued here, before the wait for the
         # result, so that nothing stands between that wait and what the caller launches next.
+        # The workspace begins with the map's K + 1 offsets as int64, which the scan leaves there for
+        # the fill pass: they ride along in the same copy, for contractions that take their offsets
+        # from device memory (wcn_sparse_conv_fwd_prepared).
         begin = L.wcn_kmap_group_start(ptr(ws), M, K) - ws.data_ptr()
-        groups = ws[begin:begin + 4 * K * ((M + 63) // 64 + 1)].clone()
+        kept = ws[:begin + 4 * K * ((M + 63) // 64 + 1)].clone()
+        groups = kept[begin:]
         status = L.wcn_kmap_read_result(ptr(ws), M, K, host_offsets, stream_ptr(device))
         if status == ERR_TABLE_OVERFLOW:
             table._grow()
@@ -142,6 +146,7 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     result._offsets64 = offsets64        # the memory behind that array
     result._out_ascend = True  # pairs ascend in output row inside every offset
     result._group_start = (groups, groups.data_ptr(), (K, M))
+    result._device_offsets = kept[:8 * (K + 1)].view(torch.int64)
     result._keys_unique = (L.wcn_kmap_last_table_flags() & 1) == 0
     return result
 

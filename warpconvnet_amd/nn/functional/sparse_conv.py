@@ -77,6 +77,39 @@ def _host_offsets_of(km: IntSearchResult):
     return kept
 
 
+def _device_offsets_of(km: IntSearchResult, device) -> Tensor:
+    """(K + 1) int64 copy of the map's offsets in device memory: left by the map builder, or made
+    here once per map object (one small copy)."""
+    kept = km._device_offsets
+    if kept is None or kept.device != device or kept.numel() != len(km.offsets):
+        kept = km.offsets.to(torch.int64).to(device)
+        km._device_offsets = kept
+    return kept
+
+
+@torch.no_grad()
+def _prepared_weight(weight: Tensor, make_w, dtype: torch.dtype, c_in: int) -> Tensor:
+    """The kernels' tiles of make_w() (the weight as the contraction would receive it: detached,
+    contiguous, its input channels zero-padded to c_in), made by wcn_conv_prepare_weight and kept
+    on the tensor object `weight` until its version counter, address, dtype or shape changes."""
+    key = (weight._version, weight.data_ptr(), weight.dtype, dtype, tuple(weight.shape), c_in)
+    kept = getattr(weight, "_wcn_prepared", None)
+    if kept is not None and kept[0] == key:
+        return kept[1]
+    L = lib()
+    w = make_w()
+    K, c_in, c_out = w.shape
+    nbytes = L.wcn_conv_prepared_weight_bytes(K, c_in, c_out, DTYPE_CODE[dtype])
+    tiles = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+    check(L.wcn_conv_prepare_weight(ptr(w), DTYPE_CODE[w.dtype], K, c_in, c_out, DTYPE_CODE[dtype],
+                                    ptr(tiles), nbytes, stream_ptr(w.device)), "wcn_conv_prepare_weight")
+    try:
+        weight._wcn_prepared = (key, tiles)
+    except AttributeError:
+        pass
+    return tiles
+
+
 @torch.no_grad()
 def _pairs_sorted(km: IntSearchResult, by: str, num_rows: int):
     """The map's pair lists re-ordered so that the `by` side ("out" or "in") ascends inside every
@@ -132,7 +165,8 @@ def _pairs_sorted(km: IntSearchResult, by: str, num_rows: int):
 def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSearchResult,
                         num_out_coords: int, bias: Optional[Tensor] = None,
                         compute_dtype: Optional[torch.dtype] = None,
-                        residual: Optional[Tensor] = None, relu: bool = False) -> Tensor:
+                        residual: Optional[Tensor] = None, relu: bool = False,
+                        keep_prepared_weight: bool = False) -> Tensor:
     """out = bias + sum_k scatter(X[in_k] @ W[k]) on the GPU (replaces the per-offset loops of
     sparse_conv.py:281-311 / :358-415 / :495-544 and the native GEMMs they call).
 
@@ -143,7 +177,14 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
 
     `residual` ((num_out_coords, c_out), added to the sums) and `relu` (clamp at zero) are done in
     the kernel's epilogue before the one rounding (wcn_sparse_conv_fwd_fused): what a residual
-    block does with two more elementwise kernels after the convolution.  Not in the reference."""
+    block does with two more elementwise kernels after the convolution.  Not in the reference.
+
+    `keep_prepared_weight` (not in the reference either): the kernels read the weight as zero-padded
+    transposed tiles, which every call makes anew with one more kernel.  With this flag the tiles
+    are kept on the tensor object `weight` and the call enqueues the contraction alone
+    (wcn_sparse_conv_fwd_prepared; same results bit for bit).  They are made again when the
+    tensor's version counter, address, dtype or shape changes; a change that the counter does not
+    see (through `weight.data`, say) is the caller's to avoid, which is why it is a flag."""
     require_device(in_features, "in_features")
     if in_features.ndim != 2 or weight.ndim != 3 or weight.shape[1] != in_features.shape[1]:
         raise ValueError(f"shape mismatch: features {tuple(in_features.shape)}, "
@@ -154,21 +195,26 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
     if x.dtype not in DTYPE_CODE:
         raise TypeError(f"unsupported feature dtype {x.dtype}")
     x = x.contiguous()
-    w = weight.detach()
-    if w.dtype != x.dtype and w.dtype != torch.float32:
-        w = w.to(x.dtype)
-    w = w.contiguous()
     b = None if bias is None else bias.detach().to(x.dtype).contiguous()
     # Feature rows that are not whole 16-byte vectors (the 3-channel input of a network's stem)
     # would take the library's slow general kernel: zero-pad the channels instead (the matching
     # weight rows are zero, the result is unchanged).
     vec = 16 // x.element_size()
+    pad = 0
     if x.shape[1] % vec != 0 and x.shape[0] > 0:
         pad = vec - x.shape[1] % vec
         x = torch.nn.functional.pad(x, (0, pad))
-        w = torch.nn.functional.pad(w, (0, 0, 0, pad))
+
+    def make_w():
+        w = weight.detach()
+        if w.dtype != x.dtype and w.dtype != torch.float32:
+            w = w.to(x.dtype)
+        if pad:
+            w = torch.nn.functional.pad(w, (0, 0, 0, pad))
+        return w.contiguous()
+
     km = kernel_map
-    K, c_in, c_out = w.shape
+    K, c_in, c_out = weight.shape[0], weight.shape[1] + pad, weight.shape[2]
     device = x.device
     out = torch.empty((num_out_coords, c_out), dtype=x.dtype, device=device)
     L = lib()
@@ -188,13 +234,23 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
                                         num_pairs, ascend)
     ws = workspace(nbytes, device)
     iden = -1 if km.identity_map_index is None else int(km.identity_map_index)
+    r = None
+    if residual is not None:
+        if tuple(residual.shape) != (num_out_coords, c_out):
+            raise ValueError(f"residual has shape {tuple(residual.shape)}, the output {(num_out_coords, c_out)}")
+        require_device(residual, "residual")
+        r = residual.detach().to(x.dtype).contiguous()
+    if keep_prepared_weight and group_start is not None and num_out_coords > 0:
+        tiles = _prepared_weight(weight, make_w, x.dtype, c_in)
+        check(L.wcn_sparse_conv_fwd_prepared(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(tiles),
+                                             tiles.numel(), K, c_out, ptr(b), ptr(in_maps), ptr(out_maps),
+                                             host_offsets, ptr(_device_offsets_of(km, device)), iden,
+                                             group_start, ptr(r), 1 if relu else 0, ptr(out),
+                                             num_out_coords, ptr(ws), ws.numel(), stream_ptr(device)),
+              "wcn_sparse_conv_fwd_prepared")
+        return out if out.dtype == in_features.dtype else out.to(in_features.dtype)
+    w = make_w()
     if residual is not None or relu:
-        r = None
-        if residual is not None:
-            if tuple(residual.shape) != (num_out_coords, c_out):
-                raise ValueError(f"residual has shape {tuple(residual.shape)}, the output {(num_out_coords, c_out)}")
-            require_device(residual, "residual")
-            r = residual.detach().to(x.dtype).contiguous()
         check(L.wcn_sparse_conv_fwd_fused(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(w),
                                           DTYPE_CODE[w.dtype], K, c_out, ptr(b), ptr(in_maps),
                                           ptr(out_maps), host_offsets, iden, ascend, group_start,
@@ -399,6 +455,7 @@ def generate_output_coords_and_kernel_map(
         kernel_map._in_group_start = forward_map._group_start
         kernel_map._keys_unique = getattr(forward_map, "_keys_unique", False)
         kernel_map._from_builder = getattr(forward_map, "_from_builder", False)
+        kernel_map._device_offsets = forward_map._device_offsets
     else:
         kernel_map = generate_kernel_map(in_coords, out_coords, stride, kernel_size,
                                          kernel_dilation, method=method,
@@ -435,6 +492,7 @@ def spatially_sparse_conv(
     implicit_matmul_bwd_block_size: Optional[int] = 16,
     residual: Optional[Union[Tensor, Voxels]] = None,
     relu: bool = False,
+    keep_prepared_weight: bool = False,
 ) -> Voxels:
     """Sparse convolution of a Voxels tensor with weight (K, C_in, C_out)
     (reference: sparse_conv.py:1662-1805).
@@ -442,7 +500,8 @@ def spatially_sparse_conv(
     `residual` (features of the output's shape, or a Voxels tensor holding them) and `relu` are not
     in the reference: out = act(conv(x) + bias + residual).  Without gradients they are carried out
     in the contraction's epilogue, on the fp32 sums before the one rounding; with gradients (and
-    for 1x1x1 kernels) they are the torch operations a caller would write after the call."""
+    for 1x1x1 kernels) they are the torch operations a caller would write after the call.
+    `keep_prepared_weight`: see sparse_conv_forward (used on the path without gradients)."""
     if not isinstance(input_sparse_tensor, Voxels):
         raise TypeError("Native spatially_sparse_conv expects input_sparse_tensor of type Voxels, "
                         f"got {type(input_sparse_tensor)}")
@@ -529,7 +588,8 @@ def spatially_sparse_conv(
         out_features = sparse_conv_forward(features, weight, kernel_map, num_out_coords, bias=bias,
                                            compute_dtype=effective_compute_dtype,
                                            residual=residual if fused else None,
-                                           relu=relu and fused)
+                                           relu=relu and fused,
+                                           keep_prepared_weight=keep_prepared_weight)
         if not fused:
             out_features = after(out_features)
 

@@ -85,6 +85,11 @@ class SpatiallySparseConv(nn.Module):
             s += ", bias=False"
         return s
 
+    # Set on an instance (or the class) whose weight stays the same between calls, or changes only in
+    # ways its version counter sees: the kernels' tiles of the weight are then kept with the
+    # parameter instead of being made by one more kernel in every call (see sparse_conv_forward).
+    keep_prepared_weight = False
+
     def forward(self, input_sparse_tensor: Voxels,
                 output_spatially_sparse_tensor: Optional[Voxels] = None, *,
                 residual=None, relu: bool = False) -> Voxels:
@@ -99,7 +104,7 @@ class SpatiallySparseConv(nn.Module):
             stride_mode=self.stride_mode, order=self.order, compute_dtype=self.compute_dtype,
             implicit_matmul_fwd_block_size=self.implicit_matmul_fwd_block_size,
             implicit_matmul_bwd_block_size=self.implicit_matmul_bwd_block_size,
-            residual=residual, relu=relu)
+            residual=residual, relu=relu, keep_prepared_weight=self.keep_prepared_weight)
 
 
 class SparseConv2d(SpatiallySparseConv):
