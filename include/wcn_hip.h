@@ -251,6 +251,12 @@ int wcn_sparse_conv_fwd_fused(const void* features, int64_t num_in, int32_t c_in
  * read the caller's weight as it is and need no such step). */
 size_t wcn_conv_prepared_weight_bytes(int32_t num_offsets, int32_t c_in, int32_t c_out, int32_t dtype);
 
+/* Workspace of wcn_sparse_conv_fwd_prepared: 0 (workspace may then be null) unless the problem's
+ * shape makes the library split the input channels over workgroups (few output rows, wide rows),
+ * then the fp32 partial sums of the slices. */
+size_t wcn_conv_prepared_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_in, int32_t c_out,
+                                         int32_t dtype);
+
 int wcn_conv_prepare_weight(const void* weight, int32_t weight_dtype, int32_t num_offsets, int32_t c_in,
                             int32_t c_out, int32_t dtype, void* prepared, size_t prepared_bytes,
                             void* stream);

@@ -47,6 +47,7 @@ SIGNATURES = {
     "wcn_sparse_conv_fwd_fused": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                                  _vp, _i64p, _i32, _i32, _vp, _vp, _i32, _vp, _i64, _vp, _sz, _vp]),
     "wcn_conv_prepared_weight_bytes": (_sz, [_i32, _i32, _i32, _i32]),
+    "wcn_conv_prepared_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i32]),
     "wcn_conv_prepare_weight": (ctypes.c_int, [_vp, _i32, _i32, _i32, _i32, _i32, _vp, _sz, _vp]),
     "wcn_sparse_conv_fwd_prepared": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _sz, _i32, _i32, _vp, _vp,
                                                     _vp, _i64p, _vp, _i32, _vp, _vp, _i32, _vp, _i64,
@@ -126,8 +127,10 @@ def stream_ptr(device) -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-def ptr(t) -> ctypes.c_void_p:
-    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+def ptr(t):
+    """A tensor's address as the void* argument of a library call (None: a null pointer); ctypes
+    converts the plain int itself."""
+    return None if t is None else t.data_ptr()
 
 
 def int3(values):

@@ -1371,6 +1371,16 @@ int static_zero_page(void** ptr) {
 }
 }  // namespace
 
+size_t wcn_conv_prepared_workspace_bytes(int64_t num_out, int32_t num_offsets, int32_t c_in, int32_t c_out,
+                                         int32_t dtype) {
+  if (num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || c_in < 1 || c_out < 1 ||
+      dtype < 0 || dtype > 2)
+    return 0;
+  const int cip = round_up(c_in, ck_of(dtype)), cop = round_up(c_out, TN);
+  if (!conv_wants_split(num_out, cip, cop, ck_of(dtype))) return 0;
+  return wcn_align256(sizeof(float) * (size_t)(cip / ck_of(dtype)) * (size_t)num_out * cop);
+}
+
 // Shared body of the forward product and the input gradient.  weight_as_stored / flip_offsets
 // choose how the caller's weight becomes the kernels' tiles (see conv_prep_weight).  With
 // `no_copy_commands` the call enqueues kernels only (the offsets must then fit the kernel
@@ -1391,7 +1401,7 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
     return WCN_ERR_INVALID_ARGUMENT;
   if (prepared && (!out_maps_ascend || !group_start_or_null)) return WCN_ERR_INVALID_ARGUMENT;
   if (num_in < 0 || num_out < 0 || num_offsets < 1 || num_offsets > WCN_MAX_OFFSETS || c_in < 1 ||
-      c_out < 1 || !weight || !workspace || !host_offsets)
+      c_out < 1 || !weight || (!workspace && !prepared) || !host_offsets)
     return WCN_ERR_INVALID_ARGUMENT;
   if (num_in >= (1ll << 31) || num_out >= (1ll << 31)) return WCN_ERR_INVALID_ARGUMENT;
   if (identity_offset >= num_offsets) return WCN_ERR_INVALID_ARGUMENT;
@@ -1403,12 +1413,21 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   if (L > 0 && (!in_maps || !out_maps)) return WCN_ERR_INVALID_ARGUMENT;
   if (num_out == 0) return WCN_OK;
   if (!out || (num_in > 0 && !features)) return WCN_ERR_INVALID_ARGUMENT;
-  if (workspace_bytes <
-      wcn_conv_workspace_bytes(num_out, num_offsets, c_in, c_out, dtype, L, out_maps_ascend))
-    return WCN_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   ConvWorkspace w;
-  conv_layout(workspace, num_out, num_offsets, c_in, c_out, dtype, out_maps_ascend ? -1 : L, &w);
+  if (prepared) {
+    // tiles, zeros, offsets and group starts all come from elsewhere: the workspace is the partial
+    // sums of split input-channel slices, where the problem's shape asks for them, and nothing else
+    const size_t need = wcn_conv_prepared_workspace_bytes(num_out, num_offsets, c_in, c_out, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return WCN_ERR_WORKSPACE;
+    conv_layout(nullptr, num_out, num_offsets, c_in, c_out, dtype, -1, &w);
+    w.partial = need > 0 ? (float*)workspace : nullptr;
+  } else {
+    if (workspace_bytes <
+        wcn_conv_workspace_bytes(num_out, num_offsets, c_in, c_out, dtype, L, out_maps_ascend))
+      return WCN_ERR_WORKSPACE;
+    conv_layout(workspace, num_out, num_offsets, c_in, c_out, dtype, out_maps_ascend ? -1 : L, &w);
+  }
   // Up to 127 offsets reach the device in the arguments of the weight preparation, which is the
   // first launch of the call: no copy command.
   const bool offsets_by_value = num_offsets + 1 <= OFFSETS_BY_VALUE;

@@ -33,7 +33,10 @@ class BatchedTensor:
         if isinstance(offsets, (list, tuple)):
             offsets = torch.LongTensor(list(offsets))
         elif isinstance(offsets, Tensor):
-            offsets = offsets.detach().cpu()
+            # a CPU tensor outside autograd is taken as it is: the coordinates and features of one
+            # geometry then share one offsets object, which later checks recognise at once
+            if offsets.is_cuda or offsets.requires_grad:
+                offsets = offsets.detach().cpu()
         else:
             raise ValueError(f"Invalid offsets type {type(offsets)}")
         if device is not None:

@@ -50,7 +50,8 @@ class Geometry:
         self.batched_coordinates = batched_coordinates
         self.batched_features = to_batched_features(batched_features, batched_coordinates.offsets,
                                                     device=kwargs.get("device", None))
-        assert (batched_coordinates.offsets == self.batched_features.offsets).all()
+        assert batched_coordinates.offsets is self.batched_features.offsets or \
+            (batched_coordinates.offsets == self.batched_features.offsets).all()
         if "_extra_attributes" in kwargs:  # flattened, as dataclasses.replace would pass it
             attr = kwargs.pop("_extra_attributes")
             assert isinstance(attr, dict), f"_extra_attributes must be a dictionary, got {attr}"

@@ -3,18 +3,28 @@
 The key is what the reference keys on: kernel size, dilation, transposed, generative, stride
 mode, skip-symmetric flag and the input / output batch offsets.
 """
-from typing import Optional, Sequence, Tuple
+from typing import Optional, Tuple
 
+import torch
 from torch import Tensor
 
 from .search_results import IntSearchResult
 
 
-def _seq_hash(values: Sequence[int]) -> int:
-    h = 0x345678
-    for v in values:
-        h = ((h * 1000003) ^ hash(int(v))) & 0xFFFFFFFFFFFFFFFF
-    return h
+def _as_tuple(offsets) -> Tuple[int, ...]:
+    """The batch offsets as a tuple of ints.  Network layers pass the same offsets tensor object over
+    and over, so the tuple is kept on it (together with its version counter)."""
+    if not isinstance(offsets, Tensor):
+        return tuple(int(v) for v in offsets)
+    kept = getattr(offsets, "_wcn_tuple", None)
+    if kept is not None and kept[0] == offsets._version:
+        return kept[1]
+    values = tuple(offsets.detach().cpu().tolist())
+    try:
+        offsets._wcn_tuple = (offsets._version, values)
+    except AttributeError:
+        pass
+    return values
 
 
 class IntSearchCacheKey:
@@ -27,28 +37,32 @@ class IntSearchCacheKey:
         self.generative = bool(generative)
         self.stride_mode = str(stride_mode)
         self.skip_symmetric_kernel_map = bool(skip_symmetric_kernel_map)
-        self.in_offsets = in_offsets.detach().cpu().int()
-        self.out_offsets = out_offsets.detach().cpu().int()
+        # compared and hashed as tuples of ints (a look-up per layer call: no tensor operations)
+        self._in = _as_tuple(in_offsets)
+        self._out = _as_tuple(out_offsets)
+        self._all = (self.kernel_size, self.kernel_dilation, self.transposed, self.generative,
+                     self.stride_mode, self.skip_symmetric_kernel_map, self._in, self._out)
 
-    def _scalars(self):
-        return (self.kernel_size, self.kernel_dilation, self.transposed, self.generative,
-                self.stride_mode, self.skip_symmetric_kernel_map)
+    @property
+    def in_offsets(self) -> Tensor:
+        return torch.tensor(self._in, dtype=torch.int32)
+
+    @property
+    def out_offsets(self) -> Tensor:
+        return torch.tensor(self._out, dtype=torch.int32)
 
     def __hash__(self) -> int:
-        return hash((self._scalars(), _seq_hash(self.in_offsets.tolist()),
-                     _seq_hash(self.out_offsets.tolist())))
+        return hash(self._all)
 
     def __eq__(self, other) -> bool:
-        return (isinstance(other, IntSearchCacheKey) and self._scalars() == other._scalars()
-                and self.in_offsets.equal(other.in_offsets)
-                and self.out_offsets.equal(other.out_offsets))
+        return isinstance(other, IntSearchCacheKey) and self._all == other._all
 
     def __repr__(self) -> str:
         return (f"IntSearchCacheKey(kernel_size={self.kernel_size}, "
                 f"kernel_dilation={self.kernel_dilation}, transposed={self.transposed}, "
                 f"generative={self.generative}, stride_mode={self.stride_mode}, "
                 f"skip_symmetric_kernel_map={self.skip_symmetric_kernel_map}, "
-                f"num_in={int(self.in_offsets[-1])}, num_out={int(self.out_offsets[-1])})")
+                f"num_in={self._in[-1]}, num_out={self._out[-1]})")
 
 
 class IntSearchCache(dict):

@@ -13,9 +13,10 @@ the map with in and out exchanged; `wcn_sparse_conv_wgrad`: per-offset X^T dY ov
 reference: sparse_conv.py:314-355).
 """
 import ctypes
-import warnings
 import enum
+import math
 import os
+import warnings
 from typing import List, Optional, Tuple, Union
 
 import numpy as np
@@ -195,7 +196,13 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
     if x.dtype not in DTYPE_CODE:
         raise TypeError(f"unsupported feature dtype {x.dtype}")
     x = x.contiguous()
-    b = None if bias is None else bias.detach().to(x.dtype).contiguous()
+
+    def as_rows(t):  # another tensor of the call, in the features' dtype and contiguous
+        if t is None or (t.dtype == x.dtype and t.is_contiguous()):
+            return t
+        return t.detach().to(x.dtype).contiguous()
+
+    b = as_rows(bias)
     # Feature rows that are not whole 16-byte vectors (the 3-channel input of a network's stem)
     # would take the library's slow general kernel: zero-pad the channels instead (the matching
     # weight rows are zero, the result is unchanged).
@@ -229,26 +236,28 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
         group_start = ctypes.c_void_p(km._group_start[1])
     ascend = 1
     host_offsets = _host_offsets_of(km)
-    num_pairs = int(host_offsets[K])
-    nbytes = L.wcn_conv_workspace_bytes(num_out_coords, K, c_in, c_out, DTYPE_CODE[x.dtype],
-                                        num_pairs, ascend)
-    ws = workspace(nbytes, device)
     iden = -1 if km.identity_map_index is None else int(km.identity_map_index)
     r = None
     if residual is not None:
         if tuple(residual.shape) != (num_out_coords, c_out):
             raise ValueError(f"residual has shape {tuple(residual.shape)}, the output {(num_out_coords, c_out)}")
         require_device(residual, "residual")
-        r = residual.detach().to(x.dtype).contiguous()
+        r = as_rows(residual)
+    code = DTYPE_CODE[x.dtype]
     if keep_prepared_weight and group_start is not None and num_out_coords > 0:
         tiles = _prepared_weight(weight, make_w, x.dtype, c_in)
-        check(L.wcn_sparse_conv_fwd_prepared(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(tiles),
+        nbytes = L.wcn_conv_prepared_workspace_bytes(num_out_coords, K, c_in, c_out, code)
+        ws = workspace(nbytes, device) if nbytes else None
+        check(L.wcn_sparse_conv_fwd_prepared(ptr(x), x.shape[0], c_in, code, ptr(tiles),
                                              tiles.numel(), K, c_out, ptr(b), ptr(in_maps), ptr(out_maps),
                                              host_offsets, ptr(_device_offsets_of(km, device)), iden,
                                              group_start, ptr(r), 1 if relu else 0, ptr(out),
-                                             num_out_coords, ptr(ws), ws.numel(), stream_ptr(device)),
+                                             num_out_coords, ptr(ws), nbytes, stream_ptr(device)),
               "wcn_sparse_conv_fwd_prepared")
         return out if out.dtype == in_features.dtype else out.to(in_features.dtype)
+    num_pairs = int(host_offsets[K])
+    nbytes = L.wcn_conv_workspace_bytes(num_out_coords, K, c_in, c_out, code, num_pairs, ascend)
+    ws = workspace(nbytes, device)
     w = make_w()
     if residual is not None or relu:
         check(L.wcn_sparse_conv_fwd_fused(ptr(x), x.shape[0], c_in, DTYPE_CODE[x.dtype], ptr(w),
@@ -523,7 +532,7 @@ def spatially_sparse_conv(
             out_features = out_features + residual.to(out_features.dtype)
         return torch.relu(out_features) if relu else out_features
 
-    if int(np.prod(_kernel_size)) == 1 and int(np.prod(_stride)) == 1:
+    if math.prod(_kernel_size) == 1 and math.prod(_stride) == 1:
         out_features = input_sparse_tensor.feature_tensor @ weight[0]
         if bias is not None:
             out_features = out_features + bias.to(out_features.dtype)
