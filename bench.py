@@ -404,9 +404,10 @@ class _UNet:
         return y
 
 
-def unet_config(dev, steps, warmup):
+def unet_config(dev, steps, warmup, compare=True):
     """One inference pass per step over a fresh Voxels (every kernel map is rebuilt, as for a new
-    input): 4 x 250k voxels, 3-channel features, bf16, random-init weights."""
+    input): 4 x 250k voxels, 3-channel features, bf16, random-init weights.  `compare`: the same
+    network timed again with the weights' tiles made in every call, and the outputs compared."""
     from warpconvnet_amd.geometry.types.voxels import Voxels
     from warpconvnet_amd.utils import synthetic
     items, offsets = synthetic.indoor_batch(4, 250_000, 0.02, seed=0)
@@ -428,14 +429,17 @@ def unet_config(dev, steps, warmup):
 
     net = _UNet(dev, torch.bfloat16)
     ms, out = timed(net)
-    ms_every_call, out_every_call = timed(_UNet(dev, torch.bfloat16, keep_tiles=False))
     assert out.feature_tensor.shape == (n, 32) and bool(torch.isfinite(out.feature_tensor).all())
-    assert torch.equal(out.feature_tensor, out_every_call.feature_tensor)
+    extra = {}
+    if compare:
+        ms_every_call, out_every_call = timed(_UNet(dev, torch.bfloat16, keep_tiles=False))
+        assert torch.equal(out.feature_tensor, out_every_call.feature_tensor)
+        extra["ms_per_pass_weight_tiles_made_in_every_call"] = ms_every_call
     convs = [net.stem] + net.down + net.up + [m for stage in net.enc_blocks + net.dec_blocks
                                              for blk in stage for m in blk if m is not None]
     sparse = sum(1 for m in convs if int(np.prod(m.kernel_size)) > 1)
     return {"num_voxels": n, "sparse_convolutions": sparse, "pointwise_convolutions": len(convs) - sparse,
-            "ms_per_pass": ms, "ms_per_pass_weight_tiles_made_in_every_call": ms_every_call,
+            "ms_per_pass": ms, **extra,
             "voxels_per_s": n / (ms * 1e-3)}
 
 
@@ -452,6 +456,9 @@ def main():
                          "the headline value stays the forward path)")
     ap.add_argument("--all-configs", action="store_true",
                     help="also time the other single-layer configurations (config.other_configs)")
+    ap.add_argument("--network-only", action="store_true",
+                    help="run nothing but passes of configs[3]'s network (--steps of them after --warmup) and "
+                         "print their timing: the command to put under a profiler for a pass's kernels")
     ap.add_argument("--gather-floor", action="store_true",
                     help="also time a kernel that only gathers the map's rows (roofline.gather_floor)")
     ap.add_argument("--sorted-voxels", action="store_true",
@@ -470,6 +477,10 @@ def main():
     from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
 
     dev = torch.device("cuda:0")
+    if args.network_only:
+        print(json.dumps({"configs[3]: MinkUNet18-style encoder-decoder, bf16, 1M voxels":
+                          unet_config(dev, args.steps, args.warmup, compare=False)}))
+        return
     bcoords, offsets, feats, weight = make_workload()
     n = len(bcoords)
     coords_d = torch.as_tensor(bcoords, device=dev)
