@@ -977,40 +977,61 @@ __global__ void __launch_bounds__(256) rows_fill(const int32_t* __restrict__ in_
   atomicMin(&row_in[row_ptr[o] + rank], in_maps[p]);
 }
 
-// Output-row form -> pair lists that ascend in output row inside every offset, plus their
-// group_start table.  Same two-pass scheme as the map builder: per (offset, 64-row group) hit
-// counts by ballot, row-wise scan, then every hit lane writes its pair at start + prefix.
-template <bool FILL>
-__global__ void __launch_bounds__(256) rows_to_pairs(const uint32_t* __restrict__ row_mask,
-                                                     const int32_t* __restrict__ row_ptr,
-                                                     const int32_t* __restrict__ row_in, int K,
-                                                     int words, int64_t num_out,
-                                                     const int64_t* __restrict__ offsets,
-                                                     int32_t* __restrict__ gs, int64_t G,
-                                                     int32_t* __restrict__ in_sorted,
-                                                     int32_t* __restrict__ out_sorted) {
+// The re-ordering of pair lists (pairs_sort_by_out) needs no row form in between.  First the rows of
+// every 64-row group that carry offset k, as a count (scanned afterwards into group_start) and as a
+// 64-bit mask ...
+__global__ void __launch_bounds__(256) pairs_group_hits(const uint32_t* __restrict__ row_mask, int K,
+                                                        int words, int64_t num_out,
+                                                        int32_t* __restrict__ gs, int64_t G,
+                                                        unsigned long long* __restrict__ hits) {
   const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t group = m >> 6;
   if (group >= G) return;
   const int lane = wcn_lane();
   const bool live = m < num_out;
-  int rank = live ? row_ptr[m] : 0;
   for (int w = 0; w < words; ++w) {
     const uint32_t word = live ? row_mask[m * words + w] : 0u;
     const int nbits = K - w * 32 < 32 ? K - w * 32 : 32;
     for (int b = 0; b < nbits; ++b) {
       const int k = w * 32 + b;
-      const bool hit = (word >> b) & 1u;
-      const unsigned long long hits = __ballot(hit);
-      if (!FILL) {
-        if (lane == 0) gs[(int64_t)k * (G + 1) + group] = __popcll(hits);
-      } else if (hit) {
-        const int64_t p = offsets[k] + gs[(int64_t)k * (G + 1) + group] +
-                          __popcll(hits & ((1ull << lane) - 1ull));
-        in_sorted[p] = row_in[rank++];
-        out_sorted[p] = (int32_t)m;
+      const unsigned long long h = __ballot((word >> b) & 1u);
+      if (lane == 0) {
+        gs[(int64_t)k * (G + 1) + group] = __popcll(h);
+        hits[group * K + k] = h;
       }
     }
+  }
+}
+
+// ... from which every pair finds its place by itself: behind the pairs of its offset whose output
+// row is lower.  in_sorted starts at INT32_MAX everywhere: of several pairs with the same (offset,
+// output row), which a kernel map never holds but a caller's lists may, the lowest input row
+// survives, whatever order the threads run in.
+__global__ void __launch_bounds__(256) pairs_place(const int32_t* __restrict__ in_maps,
+                                                   const int32_t* __restrict__ out_maps,
+                                                   const int64_t* __restrict__ offsets, int K,
+                                                   int64_t num_out, const int32_t* __restrict__ gs,
+                                                   int64_t G, const unsigned long long* __restrict__ hits,
+                                                   int32_t* __restrict__ in_sorted,
+                                                   int32_t* __restrict__ out_sorted) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= offsets[K]) return;
+  const int k = offset_of_pair(offsets, K, p);
+  const int32_t o = out_maps[p];
+  if ((uint32_t)o >= (uint64_t)num_out) return;
+  const int64_t group = o >> 6;
+  const unsigned long long h = hits[group * K + k];
+  const int64_t dest = offsets[k] + gs[(int64_t)k * (G + 1) + group] + __popcll(h & ((1ull << (o & 63)) - 1ull));
+  atomicMin(&in_sorted[dest], in_maps[p]);
+  out_sorted[dest] = o;
+}
+
+// Two ranges of words set to two values in one launch.
+__global__ void __launch_bounds__(256) rows_clear_two(uint32_t* __restrict__ a, int64_t n_a, uint32_t value_a,
+                                                      uint32_t* __restrict__ b, int64_t n_b, uint32_t value_b) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_a + n_b;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    if (i < n_a) a[i] = value_a; else b[i - n_a] = value_b;
   }
 }
 
@@ -1032,9 +1053,7 @@ struct ConvWorkspace {
   int32_t* group_start;  // (K, G+1), when not supplied by the caller
   int64_t* row_total;    // K+1 scratch of the scans
   uint32_t* row_mask;    // the rest only when the pair lists have to be re-ordered here
-  int32_t* row_ptr;
-  int32_t* row_in;
-  int32_t* groups;
+  unsigned long long* hits;
   int32_t* in_sorted;
   int32_t* out_sorted;
   float* partial;        // (slices, num_out, c_out_pad) when the input-channel slices are split
@@ -1067,12 +1086,8 @@ inline size_t conv_layout(void* base, int64_t num_out, int K, int c_in, int c_ou
   if (resort_pairs >= 0) {
     if (w) w->row_mask = (uint32_t*)(p + off);
     off += wcn_align256(sizeof(uint32_t) * (size_t)num_out * words);
-    if (w) w->row_ptr = (int32_t*)(p + off);
-    off += wcn_align256(sizeof(int32_t) * (size_t)(num_out + 1));
-    if (w) w->row_in = (int32_t*)(p + off);
-    off += wcn_align256(sizeof(int32_t) * (size_t)resort_pairs);
-    if (w) w->groups = (int32_t*)(p + off);
-    off += wcn_align256(sizeof(int32_t) * (size_t)(G + 1));
+    if (w) w->hits = (unsigned long long*)(p + off);
+    off += wcn_align256(sizeof(unsigned long long) * (size_t)K * (size_t)G);
     if (w) w->in_sorted = (int32_t*)(p + off);
     off += wcn_align256(sizeof(int32_t) * (size_t)resort_pairs);
     if (w) w->out_sorted = (int32_t*)(p + off);
@@ -1269,49 +1284,36 @@ int wcn_conv_set_timing_events(void* start_event, void* stop_event) {
   return WCN_OK;
 }
 
-// pair lists -> output-row form -> pair lists ascending in output row inside every offset, with
-// their group_start table.  Of several pairs with the same (offset, output row) one is kept.
+// pair lists -> pair lists ascending in output row inside every offset, with their group_start
+// table.  Of several pairs with the same (offset, output row) one is kept.  Five launches: clear,
+// mark the (row, offset) bits, per-group counts and masks, scan, place.
 static void pairs_sort_by_out(const int32_t* in_maps, const int32_t* out_maps, const int64_t* offsets_dev,
-                              int K, int64_t num_out, int64_t L, uint32_t* row_mask, int32_t* row_ptr,
-                              int32_t* row_in, int32_t* groups, int64_t* row_total, int32_t* in_sorted,
+                              int K, int64_t num_out, int64_t L, uint32_t* row_mask,
+                              unsigned long long* hits, int64_t* row_total, int32_t* in_sorted,
                               int32_t* out_sorted, int32_t* group_start, hipStream_t s) {
   const int words = (K + 31) / 32;
   const int64_t G = (num_out + 63) / 64;
   const unsigned rows_grid = (unsigned)((num_out + 255) / 256);
   const int64_t mask_words = num_out * words;
-  hipLaunchKernelGGL(rows_clear, dim3((unsigned)std::min<int64_t>(4096, (mask_words + 255) / 256)),
-                     dim3(256), 0, s, row_mask, mask_words, 0u);
-  if (L > 0) {
-    hipLaunchKernelGGL(rows_clear, dim3((unsigned)std::min<int64_t>(4096, (L + 255) / 256)), dim3(256),
-                       0, s, (uint32_t*)row_in, L, 0x7fffffffu);
+  hipLaunchKernelGGL(rows_clear_two, dim3((unsigned)std::min<int64_t>(4096, (mask_words + L + 255) / 256)),
+                     dim3(256), 0, s, row_mask, mask_words, 0u, (uint32_t*)in_sorted, L, 0x7fffffffu);
+  if (L > 0)
     hipLaunchKernelGGL(rows_mark, dim3((unsigned)((L + 255) / 256)), dim3(256), 0, s, out_maps,
                        offsets_dev, K, words, num_out, row_mask);
-  }
-  hipLaunchKernelGGL(rows_count<false>, dim3(rows_grid), dim3(256), 0, s, (const uint32_t*)row_mask,
-                     words, num_out, groups, row_ptr);
-  wcn_scan_rows_launch(groups, G, 1, row_total, s);
-  hipLaunchKernelGGL(rows_count<true>, dim3(rows_grid), dim3(256), 0, s, (const uint32_t*)row_mask,
-                     words, num_out, groups, row_ptr);
-  if (L > 0)
-    hipLaunchKernelGGL(rows_fill, dim3((unsigned)((L + 255) / 256)), dim3(256), 0, s, in_maps, out_maps,
-                       offsets_dev, K, words, num_out, (const uint32_t*)row_mask,
-                       (const int32_t*)row_ptr, row_in);
-  hipLaunchKernelGGL(rows_to_pairs<false>, dim3(rows_grid), dim3(256), 0, s, (const uint32_t*)row_mask,
-                     (const int32_t*)row_ptr, (const int32_t*)row_in, K, words, num_out, offsets_dev,
-                     group_start, G, in_sorted, out_sorted);
+  hipLaunchKernelGGL(pairs_group_hits, dim3(rows_grid), dim3(256), 0, s, (const uint32_t*)row_mask, K,
+                     words, num_out, group_start, G, hits);
   wcn_scan_rows_launch(group_start, G, K, row_total, s);
-  hipLaunchKernelGGL(rows_to_pairs<true>, dim3(rows_grid), dim3(256), 0, s, (const uint32_t*)row_mask,
-                     (const int32_t*)row_ptr, (const int32_t*)row_in, K, words, num_out, offsets_dev,
-                     group_start, G, in_sorted, out_sorted);
+  if (L > 0)
+    hipLaunchKernelGGL(pairs_place, dim3((unsigned)((L + 255) / 256)), dim3(256), 0, s, in_maps, out_maps,
+                       offsets_dev, K, num_out, (const int32_t*)group_start, G,
+                       (const unsigned long long*)hits, in_sorted, out_sorted);
 }
 
 struct SortWorkspace {
   int64_t* offsets;
   int64_t* row_total;
   uint32_t* row_mask;
-  int32_t* row_ptr;
-  int32_t* row_in;
-  int32_t* groups;
+  unsigned long long* hits;
 };
 
 inline size_t sort_layout(void* base, int64_t num_out, int K, int64_t L, SortWorkspace* w) {
@@ -1325,12 +1327,8 @@ inline size_t sort_layout(void* base, int64_t num_out, int K, int64_t L, SortWor
   off += wcn_align256(sizeof(int64_t) * (size_t)(K + 1));
   if (w) w->row_mask = (uint32_t*)(p + off);
   off += wcn_align256(sizeof(uint32_t) * (size_t)num_out * words);
-  if (w) w->row_ptr = (int32_t*)(p + off);
-  off += wcn_align256(sizeof(int32_t) * (size_t)(num_out + 1));
-  if (w) w->row_in = (int32_t*)(p + off);
-  off += wcn_align256(sizeof(int32_t) * (size_t)L);
-  if (w) w->groups = (int32_t*)(p + off);
-  off += wcn_align256(sizeof(int32_t) * (size_t)(G + 1));
+  if (w) w->hits = (unsigned long long*)(p + off);
+  off += wcn_align256(sizeof(unsigned long long) * (size_t)K * (size_t)G);
   return off;
 }
 
@@ -1483,8 +1481,7 @@ static int conv_run(const void* features, int64_t num_in, int32_t c_in, int32_t 
   a.group_start = group_start_or_null;
   if (!out_maps_ascend) {
     pairs_sort_by_out(in_maps, out_maps, (const int64_t*)w.offsets, num_offsets, num_out, L, w.row_mask,
-                      w.row_ptr, w.row_in, w.groups, w.row_total, w.in_sorted, w.out_sorted,
-                      w.group_start, s);
+                      w.hits, w.row_total, w.in_sorted, w.out_sorted, w.group_start, s);
     a.in_maps = w.in_sorted;
     a.out_maps = w.out_sorted;
     a.group_start = w.group_start;
@@ -1588,8 +1585,8 @@ int wcn_pairs_sort_by_out(const int32_t* in_maps, const int32_t* out_maps, const
                             hipMemcpyHostToDevice, s) != hipSuccess) {
     return WCN_ERR_LAUNCH;
   }
-  pairs_sort_by_out(in_maps, out_maps, w.offsets, num_offsets, num_out, L, w.row_mask, w.row_ptr,
-                    w.row_in, w.groups, w.row_total, in_sorted, out_sorted, group_start, s);
+  pairs_sort_by_out(in_maps, out_maps, w.offsets, num_offsets, num_out, L, w.row_mask, w.hits,
+                    w.row_total, in_sorted, out_sorted, group_start, s);
   return hipGetLastError() == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
 }
 
