@@ -44,7 +44,7 @@ def test_size_queries_and_status_strings():
     assert L.wcn_kmap_workspace_bytes(10**6, 27) >= 27 * (10**6 // 64 + 1) * 4
     assert L.wcn_kmap_workspace_bytes(10, 0) == 0 and L.wcn_kmap_workspace_bytes(10, 5000) == 0
     assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 1, 5000, 1) >= 27 * 64 * 64 * 2
-    assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 1, 5000, 0) >= 27 * 64 * 64 * 2 + 12 * 5000 + 8 * 1000
+    assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 1, 5000, 0) >= 27 * 64 * 64 * 2 + 8 * 5000 + 4 * 1000 + 8 * 27 * 16
     assert L.wcn_conv_workspace_bytes(1000, 27, 64, 64, 7, 0, 1) == 0
     assert L.wcn_stride_unique_workspace_bytes(1000, 1024) > 16 * 1000
 
@@ -74,7 +74,7 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert L.wcn_kmap_count_dilated(fake, 10, 1024, fake, 5, bad, three, one, one, fake, null) == -1
     assert L.wcn_kmap_count_dilated(fake, 10, 1024, fake, 5, three, three, one, one, null, null) == -1
     offs = (ctypes.c_int64 * 28)(*([0] * 28))
-    assert L.wcn_pairs_sort_workspace_bytes(1000, 27, 5000) >= 4 * 1000 + 4 * 5000
+    assert L.wcn_pairs_sort_workspace_bytes(1000, 27, 5000) >= 4 * 1000 + 8 * 27 * 16   # row bits + per-group masks
     assert L.wcn_pairs_sort_workspace_bytes(1000, 0, 5000) == 0
     assert L.wcn_pairs_sort_by_out(fake, fake, offs, 27, 10, fake, fake, null, fake, 1 << 20, null) == -1   # no group table
     assert L.wcn_pairs_sort_by_out(fake, fake, None, 27, 10, fake, fake, fake, fake, 1 << 20, null) == -1
@@ -89,6 +89,25 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
         return L.wcn_sparse_conv_fwd(fake, 10, 64, dtype, fake, wdtype, 27, 64, null, fake, fake,
                                      offsets, -1, ascend, gs, fake, 10, fake, ws_bytes, null)
 
+    # weight tiles made ahead of the call
+    assert L.wcn_conv_prepared_weight_bytes(27, 64, 64, 1) >= 27 * 64 * 64 * 2
+    assert L.wcn_conv_prepared_weight_bytes(27, 3, 20, 2) >= 27 * 32 * 32 * 2    # channels padded to whole tiles
+    assert L.wcn_conv_prepared_weight_bytes(0, 64, 64, 1) == 0 and L.wcn_conv_prepared_weight_bytes(27, 64, 64, 5) == 0
+    assert L.wcn_conv_prepared_workspace_bytes(1_000_000, 27, 64, 64, 1) == 0   # no split of input-channel slices
+    assert L.wcn_conv_prepared_workspace_bytes(1500, 27, 256, 256, 1) >= 4 * 4 * 1500 * 256
+    assert L.wcn_conv_prepare_weight(fake, 1, 27, 64, 64, 1, null, 1 << 20, null) == -1
+    assert L.wcn_conv_prepare_weight(fake, 2, 27, 64, 64, 1, fake, 1 << 20, null) == -1   # bf16 weight, f16 tiles
+    assert L.wcn_conv_prepare_weight(fake, 1, 27, 64, 64, 1, fake, 16, null) == -6
+
+    def prepared(tile_bytes=1 << 20, dev_offsets=fake, gs=fake, ws=null, ws_bytes=0, c=64, n=10, residual=null, out=fake):
+        return L.wcn_sparse_conv_fwd_prepared(fake, 10, c, 1, fake, tile_bytes, 27, c, null, fake, fake, offs,
+                                              dev_offsets, -1, gs, residual, 0, out, n, ws, ws_bytes, null)
+
+    assert prepared(dev_offsets=null) == -1          # the offsets have to be in device memory as well
+    assert prepared(gs=null) == -1                   # and the group starts come with the map
+    assert prepared(tile_bytes=16) == -6
+    assert prepared(c=256, n=1500, tile_bytes=1 << 23) == -6   # this shape splits slices: partial sums need room
+    assert prepared(residual=fake, out=fake) == -1   # the residual may not be the output buffer
     assert conv(dtype=9) == -1
     assert conv(wdtype=2) == -1                      # f16 features with bf16 weights
     assert conv(ws_bytes=16) == -6                   # workspace too small
