@@ -62,6 +62,9 @@ CONV_CASES = [
     ("f16_128_128_k2", torch.float16, 128, 128, 3000, 1, (2, 2, 2)),
     ("f16_16_16_k5", torch.float16, 16, 16, 3000, 1, (5, 5, 5)),
     ("bf16_40_72_k2", torch.bfloat16, 40, 72, 3000, 1, (2, 2, 2)),
+    # fp32 rows that are not a whole 128-byte slice under more than 64 offsets: the pair-packed
+    # kernel's eight-wave instance
+    ("f32_24_40_k5", torch.float32, 24, 40, 2500, 1, (5, 5, 5)),
     # wide rows on both sides and at least 96 tiles of 256 output rows: the output-stationary kernel
     # (sums in registers), with and without an identity offset, last tile partly filled; tiles of
     # 192 rows (four 48-row waves, whose rows span two 64-row groups) and, for the map of 51,000

@@ -710,7 +710,10 @@ inline int device_cus() {
 // plus its steps.  Small tiles put more CUs to work on small maps; tall ones need fewer phases.
 template <typename T, int NL, bool FULL, bool K2, bool WIDE>
 int launch_shaped(const ConvArgs& a, hipStream_t s) {
-  constexpr int R = WCN_PACK_R, NW = WCN_PACK_NW;
+  // fp32 rows that are not whole 128-byte slices under more than 64 offsets need a few registers
+  // more than twelve waves leave a lane (the kernel's waits are counted by hand: nothing may spill);
+  // that instance runs with eight waves
+  constexpr int R = WCN_PACK_R, NW = (sizeof(T) == 4 && !FULL && K2) ? 7 : WCN_PACK_NW;
   const bool wide_out = a.c_out > 32;
   const int64_t ny = wide_out ? (a.c_out + 63) / 64 : 1;
   const int cus = device_cus();
