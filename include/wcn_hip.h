@@ -187,6 +187,14 @@ int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_strid
 int wcn_stride_unique_read_count(const void* workspace, int64_t n, int64_t capacity,
                                  int64_t* host_count, void* stream);
 
+/* wcn_stride_unique_read_count plus, in the same read, where the rows of every batch item begin:
+ * host_bounds[b], b = 0 .. 1024, is the first of the M output rows whose batch id is at least b.
+ * Meaningful for inputs whose batch column does not descend (the rows of a Voxels object), whose
+ * output rows then do not descend either.  Replaces the reference's offsets_from_batch_index over
+ * the strided rows (geometry/coords/ops/batch_index.py:143-161: a bincount and its own wait). */
+int wcn_stride_unique_read_bounds(const void* workspace, int64_t n, int64_t capacity,
+                                  int64_t* host_count, int64_t* host_bounds, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Feature contraction.  Replaces, in one launch sequence, the whole per-offset loop of the
  * reference forward (sparse_conv.py:281-311 / :358-415 / :495-544) and the native calls it

@@ -222,6 +222,13 @@ def test_batch_offsets_of_an_ascending_column_by_search():
     a, a_off = stride_coords(_dev(in_coords), (2, 2, 2))
     b, b_off = stride_coords(_dev(in_coords), (2, 2, 2), batch_sorted=True)
     assert torch.equal(a, b) and a_off.tolist() == b_off.tolist()
+    # batch items without rows in the middle: the bounds the library hands over with the row count
+    gaps = in_coords.copy()
+    gaps[:, 0] = np.array([0, 2, 5, 6])[gaps[:, 0]]
+    a, a_off = stride_coords(_dev(gaps), (2, 2, 2))
+    b, b_off = stride_coords(_dev(gaps), (2, 2, 2), batch_sorted=True)
+    assert torch.equal(a, b) and a_off.tolist() == b_off.tolist() and len(b_off) == 8
+    assert b_off[2] == b_off[1] and b_off[-1] == len(b)
 
 
 def test_kernel_map_invariants_full_size():

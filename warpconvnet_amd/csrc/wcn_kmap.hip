@@ -1024,8 +1024,10 @@ void launch_emit(int64_t num_out, const KmapGeom& g, const KmapWorkspace& w, int
 
 // ---- strided output coordinates -----------------------------------------------------------------
 
+constexpr int STRIDE_BATCH_MARKS = 1025;  // batch ids 0 .. 1024 whose first coarse row is looked up
+
 struct StrideWorkspace {
-  int64_t* result;   // [0] = M, [1] = table status bits
+  int64_t* result;   // [0] = M, [1] = table status bits, [4 + b] = first coarse row of batch id >= b
   int32_t* coarse;   // (n, 4) floor-divided coordinates
   int32_t* groups;   // (1, G+1) winners per 64-row group, then prefix sums
   void* table;       // block table over the coarse coordinates
@@ -1037,7 +1039,7 @@ inline size_t stride_layout(void* base, int64_t n, int64_t capacity, StrideWorks
   size_t off = 0;
   const int64_t G = (n + 63) / 64;
   if (w) w->result = (int64_t*)(p + off);
-  off += 256;
+  off += wcn_align256(sizeof(int64_t) * (size_t)(4 + STRIDE_BATCH_MARKS));
   if (w) w->coarse = (int32_t*)(p + off);
   off += wcn_align256(sizeof(int32_t) * 4 * (size_t)n);
   if (w) w->groups = (int32_t*)(p + off);
@@ -1106,6 +1108,22 @@ __global__ void stride_finish(int64_t* __restrict__ result, const int32_t* __res
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
   result[0] = groups[G];
   result[1] = hdr->status;
+}
+
+// Where the coarse rows of each batch item begin, for rows whose batch column does not descend
+// (the rows of a batch-sorted input): thread b finds the first of the M rows whose batch id is at
+// least b.  For other inputs the numbers mean nothing and nobody reads them.
+__global__ void __launch_bounds__(1024) stride_batch_bounds(const int4* __restrict__ out_coords,
+                                                            int64_t* __restrict__ result) {
+  const int64_t m = result[0];
+  for (int b = threadIdx.x; b < STRIDE_BATCH_MARKS; b += 1024) {
+    int64_t lo = 0, hi = m;
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (out_coords[mid].x < b) lo = mid + 1; else hi = mid;
+    }
+    result[4 + b] = lo;
+  }
 }
 
 }  // namespace
@@ -1355,9 +1373,22 @@ int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_strid
     hipLaunchKernelGGL(stride_pick<true>, dim3(grid_for(n, 256)), dim3(256), 0, s,
                        (const int4*)w.coarse, n, v.hdr, v.slots, v.slot_of, v.perm, w.groups, w.G,
                        (int4*)out_coords, first_index);
+    hipLaunchKernelGGL(stride_batch_bounds, dim3(1), dim3(1024), 0, s, (const int4*)out_coords, w.result);
   }
   WCN_LAUNCH_CHECK();
   return WCN_OK;
+}
+
+int wcn_stride_unique_read_bounds(const void* workspace, int64_t n, int64_t capacity,
+                                  int64_t* host_count, int64_t* host_bounds, void* stream) {
+  if (!workspace || !host_count || !host_bounds) return WCN_ERR_INVALID_ARGUMENT;
+  StrideWorkspace w;
+  stride_layout(const_cast<void*>(workspace), n, capacity, &w);
+  int64_t tmp[4 + STRIDE_BATCH_MARKS];
+  if (wcn_read_small(tmp, w.result, sizeof(tmp), (hipStream_t)stream) != WCN_OK) return WCN_ERR_LAUNCH;
+  *host_count = tmp[0];
+  for (int b = 0; b < STRIDE_BATCH_MARKS; ++b) host_bounds[b] = n > 0 ? tmp[4 + b] : 0;
+  return wcn_table_status_from_bits((int32_t)tmp[1]);
 }
 
 int wcn_stride_unique_read_count(const void* workspace, int64_t n, int64_t capacity,

@@ -31,7 +31,7 @@ def expand_coords(batch_indexed_coords: Tensor, kernel_size: Tuple[int, ...],
         raise ValueError("kernel size and coordinates disagree on the number of spatial dimensions")
     shifted = (batch_indexed_coords.unsqueeze(0) + offsets.unsqueeze(1)).reshape(-1, offsets.shape[1])
     rows = torch.cat([batch_indexed_coords, shifted.to(batch_indexed_coords.dtype)], dim=0)
-    out, count = unique_floor_div_rows(rows.contiguous(), (1,) * (rows.shape[1] - 1))
+    out, count, _ = unique_floor_div_rows(rows.contiguous(), (1,) * (rows.shape[1] - 1))
     unique = out[:count, : rows.shape[1]]
     order = torch.sort(unique[:, 0], stable=True).indices
     unique = unique[order].contiguous()

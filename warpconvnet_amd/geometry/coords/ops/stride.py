@@ -32,11 +32,19 @@ def stride_coords(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
          f"dimensions for but coordinates with {num_spatial_dims} spatial dimensions.")
     if all(s == 1 for s in stride):
         return batch_indexed_coords, offsets_from_batch_index(batch_indexed_coords[:, 0], ascending=batch_sorted)
-    out, count = unique_floor_div_rows(batch_indexed_coords, stride)
+    out, count, bounds = unique_floor_div_rows(batch_indexed_coords, stride, want_bounds=batch_sorted)
     unique_coords = out[:count, : num_spatial_dims + 1]
     if num_spatial_dims != 3:
         unique_coords = unique_coords.contiguous()
-    out_offsets = offsets_from_batch_index(unique_coords[:, 0], ascending=batch_sorted)
+    out_offsets = None
+    if bounds is not None and count > 0:
+        # the library looked the batch items' first rows up behind the compaction and handed them
+        # over with the row count: what offsets_from_batch_index(..., ascending=True) computes
+        batches = sum(1 for b in bounds if b < count)  # the last batch item with rows, plus one
+        if batches < len(bounds):
+            out_offsets = torch.tensor(list(bounds[:batches]) + [count], dtype=torch.int64)
+    if out_offsets is None:
+        out_offsets = offsets_from_batch_index(unique_coords[:, 0], ascending=batch_sorted)
     if str(getattr(order, "name", order)).lower() not in ("random", "point_ordering.random"):
         # The coarse voxels of every batch item along a space-filling curve.  (The reference hands
         # the four-column rows to `encode`, whose code function accepts three columns and raises,
@@ -49,9 +57,11 @@ def stride_coords(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
 
 
 @torch.no_grad()
-def unique_floor_div_rows(batch_indexed_coords: Tensor, stride: Tuple[int, ...]):
-    """((n, 4) buffer, M): the distinct rows of floor(coords / [1, *stride]) in its first M rows,
-    ascending in the first source row of each (one library call and one host read)."""
+def unique_floor_div_rows(batch_indexed_coords: Tensor, stride: Tuple[int, ...], want_bounds: bool = False):
+    """((n, 4) buffer, M, bounds): the distinct rows of floor(coords / [1, *stride]) in its first M
+    rows, ascending in the first source row of each (one library call and one host read).
+    `want_bounds`: for an input whose batch column does not descend, bounds[b] (b = 0 .. 1024) is
+    the first output row whose batch id is at least b, from the same read; otherwise None."""
     assert batch_indexed_coords.dtype == torch.int32
     num_spatial_dims = batch_indexed_coords.shape[1] - 1
     device = batch_indexed_coords.device
@@ -63,15 +73,20 @@ def unique_floor_div_rows(batch_indexed_coords: Tensor, stride: Tuple[int, ...])
     first = torch.empty(n, dtype=torch.int32, device=device)
     slots = L.wcn_table_default_capacity(n)
     count = ctypes.c_int64(0)
+    bounds = (ctypes.c_int64 * 1025)() if want_bounds else None
     while True:
         ws = workspace(L.wcn_stride_unique_workspace_bytes(n, slots), device)
         check(L.wcn_stride_unique(ptr(coords), n, st, ptr(ws), slots, ptr(out), ptr(first),
                                   stream_ptr(device)), "wcn_stride_unique")
-        status = L.wcn_stride_unique_read_count(ptr(ws), n, slots, ctypes.byref(count),
-                                                stream_ptr(device))
+        if want_bounds:
+            status = L.wcn_stride_unique_read_bounds(ptr(ws), n, slots, ctypes.byref(count), bounds,
+                                                     stream_ptr(device))
+        else:
+            status = L.wcn_stride_unique_read_count(ptr(ws), n, slots, ctypes.byref(count),
+                                                    stream_ptr(device))
         if status == ERR_TABLE_OVERFLOW and slots < (1 << 30):
             slots *= 4
             continue
         check(status, "wcn_stride_unique")
         break
-    return out, int(count.value)
+    return out, int(count.value), (list(bounds) if want_bounds else None)

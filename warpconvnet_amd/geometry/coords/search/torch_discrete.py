@@ -131,8 +131,10 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
         table._checked = True
         break
     total = int(host_offsets[K])
-    if 2 * total <= assumed:
-        # far fewer pairs than assumed: exact copies, so the map does not hold the large buffers
+    if 2 * total <= assumed and (assumed - total) * 4 > (32 << 20):
+        # far fewer pairs than assumed, and more than 32 MiB of each buffer unused: exact copies,
+        # so the map does not hold the large buffers (below that the two copy kernels cost more
+        # than the memory is worth)
         in_maps, out_maps = in_buf[:total].clone(), out_buf[:total].clone()
     elif total <= assumed:
         in_maps, out_maps = in_buf[:total], out_buf[:total]
