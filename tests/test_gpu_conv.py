@@ -370,6 +370,11 @@ def test_pair_lists_are_reordered_once_and_kept_on_the_map(oracle):
     want[1] += feats[1] @ weights[0]
     want[2] += feats[9] @ weights[1]
     assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
+    # and with kept weight tiles: a caller's map has no offsets in device memory yet (they are copied
+    # there on first use and kept on the map object)
+    assert clean._device_offsets is None
+    kept = sparse_conv_forward(feats, weights, clean, 3, keep_prepared_weight=True)
+    assert torch.equal(got, kept) and clean._device_offsets.tolist() == [0, 2, 3]
 
 
 def test_transposed_adjoint_identity():

@@ -268,53 +268,13 @@ __global__ void __launch_bounds__(256) kmap_pass_fixed(const WcnTableHeader* __r
   if (lane == 0) groups[(int64_t)K * (G + 1) + group] = group_hits;
 }
 
-// Emit pass: pair lists from the masks, scanned counts and parked rows of the probe pass.  This
-// kernel takes maps of any size (the launch uses it for more than 64 offsets): lane j fetches mask
-// and start of offset k0 + j for the whole group; the lanes then walk the offsets together.
-__global__ void __launch_bounds__(256) kmap_emit(const unsigned long long* __restrict__ hits,
-                                                 const int32_t* __restrict__ found,
-                                                 const int32_t* __restrict__ groups,
-                                                 const int64_t* __restrict__ offsets, int K,
-                                                 int64_t G, int64_t pair_capacity,
-                                                 int32_t* __restrict__ in_maps,
-                                                 int32_t* __restrict__ out_maps) {
-  const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t group = m >> 6;  // wave-uniform
-  if (group >= G) return;
-  // offsets[K] = number of pairs, offsets[K + 1] = table status bits (written by the scan): the
-  // pass may have been enqueued before the host has seen either, so it checks them itself
-  if (offsets[K] > pair_capacity || offsets[K + 1] != 0) return;
-  const int lane = wcn_lane();
-  const unsigned long long below = (1ull << lane) - 1ull;
-  const int32_t* parked = found + group * (64 * (int64_t)K);  // the group's rows, offset by offset
-  int parked_before = 0;                                       // rows of the offsets walked so far
-  for (int k0 = 0; k0 < K; k0 += 64) {
-    unsigned long long h = 0ull;
-    long long st = 0;
-    if (k0 + lane < K) {
-      h = hits[group * K + k0 + lane];
-      st = offsets[k0 + lane] + groups[(int64_t)(k0 + lane) * (G + 1) + group];
-    }
-    const int n = K - k0 < 64 ? K - k0 : 64;
-    for (int j = 0; j < n; ++j) {
-      const unsigned long long hj = __shfl(h, j, 64);
-      const long long sj = __shfl(st, j, 64);
-      if ((hj >> lane) & 1ull) {
-        const long long p = sj + __popcll(hj & below);
-        in_maps[p] = parked[parked_before + __popcll(hj & below)];
-        out_maps[p] = (int32_t)m;
-      }
-      parked_before += __popcll(hj);  // the same in every lane
-    }
-  }
-}
-
-// Emit pass for maps of at most 64 offsets, a lane per PAIR: the parked rows of a group already lie
-// in the order of its pairs (offset by offset, in lane order), so lane p of a round takes pair
-// p, p + 64, ... of the group, finds the offset it belongs to (binary search over the running counts
-// the lanes hold), its rank there, and from rank and mask the output row.  A group's ~270 pairs cost
-// five rounds of one load and two stores where a walk over the offsets costs one load and two
-// stores of a few lanes each per offset.
+// Emit pass: pair lists from the masks, scanned counts and parked rows of the probe pass, a lane per
+// PAIR.  The parked rows of a group already lie in the order of its pairs (offset by offset, in lane
+// order), so for 64 offsets at a time (lane j fetches mask and start of offset k0 + j) lane p of a
+// round takes pair p, p + 64, ... of those offsets, finds the offset it belongs to (binary search
+// over the running counts the lanes hold), its rank there, and from rank and mask the output row.
+// A group's ~270 pairs of a 3x3x3 map cost five rounds of one load and two stores where a walk over
+// the offsets costs one load and two stores of a few lanes each per offset (5x5x5: 154 -> 85 us).
 __device__ __forceinline__ int kmap_nth_set_bit(unsigned long long mask, int r) {  // position of the r-th set bit (r counts from 0)
   uint32_t w = (uint32_t)mask;
   int pos = 0;
@@ -349,38 +309,43 @@ __global__ void __launch_bounds__(256) kmap_emit_flat(const unsigned long long* 
   const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t group = m >> 6;  // wave-uniform
   if (group >= G) return;
-  if (offsets[K] > pair_capacity || offsets[K + 1] != 0) return;  // see kmap_emit
+  // offsets[K] = number of pairs, offsets[K + 1] = table status bits (written by the scan): the
+  // pass may have been enqueued before the host has seen either, so it checks them itself
+  if (offsets[K] > pair_capacity || offsets[K + 1] != 0) return;
   const int lane = wcn_lane();
   const int32_t* parked = found + group * (64 * (int64_t)K);
-  unsigned long long h = 0ull;
-  long long st = 0;
-  if (lane < K) {
-    h = hits[group * K + lane];
-    st = offsets[lane] + groups[(int64_t)lane * (G + 1) + group];
-  }
-  const int cnt = __popcll(h);
-  const int incl = wcn_wave_inclusive_sum(cnt);  // pairs of the offsets up to and including this lane's
-  const int total = __shfl(incl, 63, 64);
-  for (int p0 = 0; p0 < total; p0 += 64) {
-    const int p = p0 + lane;
-    const bool live = p < total;
-    // first offset whose running count exceeds p (the lanes past K hold the total: never chosen by a live p)
-    int lo = 0, hi = 63;
+  for (int k0 = 0; k0 < K; k0 += 64) {  // 64 offsets at a time, a lane per offset
+    unsigned long long h = 0ull;
+    long long st = 0;
+    if (k0 + lane < K) {
+      h = hits[group * K + k0 + lane];
+      st = offsets[k0 + lane] + groups[(int64_t)(k0 + lane) * (G + 1) + group];
+    }
+    const int cnt = __popcll(h);
+    const int incl = wcn_wave_inclusive_sum(cnt);  // pairs of these offsets up to and including this lane's
+    const int total = __shfl(incl, 63, 64);
+    for (int p0 = 0; p0 < total; p0 += 64) {
+      const int p = p0 + lane;
+      const bool live = p < total;
+      // first offset whose running count exceeds p (lanes past the last offset hold the total: never chosen by a live p)
+      int lo = 0, hi = 63;
 #pragma unroll
-    for (int step = 0; step < 6; ++step) {
-      const int mid = (lo + hi) >> 1;
-      const int v = __shfl(incl, mid, 64);
-      if (v <= p) lo = mid + 1; else hi = mid;
+      for (int step = 0; step < 6; ++step) {
+        const int mid = (lo + hi) >> 1;
+        const int v = __shfl(incl, mid, 64);
+        if (v <= p) lo = mid + 1; else hi = mid;
+      }
+      const int k = lo;
+      const unsigned long long hk = __shfl(h, k, 64);
+      const long long sk = __shfl(st, k, 64);
+      const int rank = p - (__shfl(incl, k, 64) - __popcll(hk));
+      if (live) {
+        const long long dst = sk + rank;
+        in_maps[dst] = parked[p];
+        out_maps[dst] = (int32_t)(group * 64 + kmap_nth_set_bit(hk, rank));
+      }
     }
-    const int k = lo;
-    const unsigned long long hk = __shfl(h, k, 64);
-    const long long sk = __shfl(st, k, 64);
-    const int rank = p - (__shfl(incl, k, 64) - __popcll(hk));
-    if (live) {
-      const long long dst = sk + rank;
-      in_maps[dst] = parked[p];
-      out_maps[dst] = (int32_t)(group * 64 + kmap_nth_set_bit(hk, rank));
-    }
+    parked += total;  // the next 64 offsets' rows follow
   }
 }
 
@@ -882,7 +847,7 @@ __global__ void __launch_bounds__(SELF_CHUNK) self_emit(const uint32_t* __restri
   __shared__ int s_start[WAVES][K];     // pairs of offset k below the wave's first row
   __shared__ uint32_t s_hm[WAVES][64][WORDS];
   __shared__ int32_t s_ptr[WAVES][64];
-  // see kmap_emit; the group starts are written whatever the room for pairs (the caller keeps them)
+  // as in kmap_emit_flat; the group starts are written whatever the room for pairs (the caller keeps them)
   if (offsets[K + 1] != 0) return;
   const bool room = offsets[K] <= pair_capacity;
   const int tid = threadIdx.x, lane = wcn_lane(), wave = tid >> 6;
@@ -1013,13 +978,8 @@ void launch_emit(int64_t num_out, const KmapGeom& g, const KmapWorkspace& w, int
                  int32_t* in_maps, int32_t* out_maps, hipStream_t s) {
   const dim3 grid(grid_for(num_out, 256)), block(256);
   const int64_t* offsets = (const int64_t*)w.result;
-  if (g.K <= 64) {
-    hipLaunchKernelGGL(kmap_emit_flat, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
-                       w.G, pair_capacity, in_maps, out_maps);
-  } else {
-    hipLaunchKernelGGL(kmap_emit, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
-                       w.G, pair_capacity, in_maps, out_maps);
-  }
+  hipLaunchKernelGGL(kmap_emit_flat, grid, block, 0, s, w.hits, w.found, w.groups, offsets, g.K,
+                     w.G, pair_capacity, in_maps, out_maps);
 }
 
 // ---- strided output coordinates -----------------------------------------------------------------
