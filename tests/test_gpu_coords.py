@@ -409,3 +409,63 @@ def test_kernel_map_with_more_pairs_than_assumed(oracle):
     assert int(km.offsets[-1]) == len(im) > 8 * len(bc)
     assert np.array_equal(km.in_maps.cpu().numpy(), im) and np.array_equal(km.out_maps.cpu().numpy(), om)
     assert np.array_equal(km.offsets.numpy().astype(np.int64), off)
+
+
+def _brute_force_map(in_rows, out_rows, stride, ksize, dilation=None):
+    """Kernel map over any number of columns by dictionary look-up: offsets enumerated with the last
+    dimension fastest, pairs of an offset in ascending output row (what the reference's offset probe
+    over all columns yields, discrete_kernels.cu:129-180)."""
+    import itertools
+    D = len(ksize)
+    dilation = dilation or [1] * D
+    where = {tuple(r): i for i, r in enumerate(in_rows.tolist())}
+    centres = [(k - 1) // 2 if k % 2 == 1 else 0 for k in ksize]
+    ins, outs, offsets = [], [], [0]
+    for idx in itertools.product(*[range(k) for k in ksize]):
+        off = [(i - c) * d for i, c, d in zip(idx, centres, dilation)]
+        for m, r in enumerate(out_rows.tolist()):
+            q = (r[0],) + tuple(r[1 + d] * stride[d] + off[d] for d in range(D))
+            hit = where.get(q)
+            if hit is not None:
+                ins.append(hit)
+                outs.append(m)
+        offsets.append(len(ins))
+    return np.array(ins, np.int32), np.array(outs, np.int32), np.array(offsets, np.int64)
+
+
+MORE_DIMS = [
+    # name, columns past the batch, rows, extent, kernel, stride, dilation
+    ("4d_k3", 4, 3000, 9, (3, 3, 3, 3), (1, 1, 1, 1), None),
+    ("4d_k2s2", 4, 3000, 10, (2, 2, 2, 2), (2, 2, 2, 2), None),
+    ("4d_mixed_dilated", 4, 2000, 12, (3, 1, 2, 3), (1, 1, 1, 1), (1, 1, 2, 2)),
+    ("5d", 5, 2500, 6, (3, 3, 1, 2, 3), (1, 1, 1, 1, 1), None),
+]
+
+
+@pytest.mark.parametrize("name,D,n,extent,ksize,stride,dilation", MORE_DIMS, ids=[c[0] for c in MORE_DIMS])
+def test_kernel_map_over_more_than_three_dimensions(name, D, n, extent, ksize, stride, dilation):
+    """Four and five spatial dimensions (folded into the batch column for the device kernels) against
+    a dictionary look-up over all columns: same pairs, same order, negative coordinates included."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    rng = np.random.default_rng(len(name))
+    rows = rng.integers(-extent // 2, extent // 2 + 1, size=(n, D + 1)).astype(np.int32)
+    rows[:, 0] = rng.integers(0, 3, size=n)
+    rows = np.unique(rows, axis=0)
+    rng.shuffle(rows)
+    if any(s != 1 for s in stride):
+        coarse = rows.copy()
+        coarse[:, 1:] = np.floor_divide(rows[:, 1:], np.array(stride, dtype=np.int32))
+        out_rows = np.unique(coarse, axis=0)
+    else:
+        out_rows = rows
+    km = generate_kernel_map(_dev(rows), _dev(out_rows), stride, ksize, kernel_dilation=dilation,
+                             method="offset" if dilation else "size")
+    want_in, want_out, want_off = _brute_force_map(rows, out_rows, stride, ksize, dilation)
+    assert np.array_equal(km.offsets.numpy().astype(np.int64), want_off)
+    assert np.array_equal(km.in_maps.cpu().numpy(), want_in)
+    assert np.array_equal(km.out_maps.cpu().numpy(), want_out)
+    all_odd = all(k % 2 == 1 for k in ksize)
+    assert km.identity_map_index == (int(np.prod(ksize)) // 2 if all_odd and len(rows) == len(out_rows) else None)
+    if km.identity_map_index is not None:
+        i, o = km[km.identity_map_index]
+        assert torch.equal(i, o) and len(i) == len(rows)

@@ -175,6 +175,84 @@ def _table_of(coords: Tensor, hash_method: HashMethod, device) -> TorchHashTable
 
 
 @torch.no_grad()
+def _kernel_map_more_dims(in_coords: Tensor, out_coords: Tensor, stride, kernel_size, kernel_dilation,
+                          kernel_center_offset, hash_method, skip_symmetric_kernel_map) -> IntSearchResult:
+    """Kernel maps over more than three spatial dimensions (the reference's offset probe takes up to
+    sixteen columns, discrete_kernels.cu:129-180; its size probe is four columns wide like the
+    device kernels here).  The dimensions past the third are folded into the batch column: a row
+    (b, x, y, z, t, u) becomes ((b T + t - t0) U + u - u0, x, y, z), with T and U wide enough for
+    every query, so that a step along t or u is a shift of the batch column and a query that leaves
+    the range of the inputs lands on a batch id no input has.  One three-dimensional map per
+    combination of offsets along the folded dimensions, over one table of the folded inputs; their
+    per-offset lists, put together with the last dimension fastest, are the map (same pairs in the
+    same order as a probe of all columns at once)."""
+    device = in_coords.device
+    D = out_coords.shape[1] - 1
+    stride = [int(v) for v in stride]
+    ks = [int(v) for v in kernel_size]
+    dil = [1] * D if kernel_dilation is None else [int(v) for v in kernel_dilation]
+    centres = _kernel_centres(ks, kernel_center_offset)
+    steps = [[(i - centres[d]) * dil[d] for i in range(ks[d])] for d in range(D)]  # offsets per dimension
+    # ranges of the folded columns over inputs and queries (two small reductions, one read)
+    ext_in = in_coords[:, 4:].long()
+    ext_out = out_coords[:, 4:].long() * torch.tensor(stride[3:], device=device)
+    lows, highs = [], []
+    if in_coords.shape[0] and out_coords.shape[0]:
+        stats = torch.stack([ext_in.amin(0), ext_in.amax(0), ext_out.amin(0), ext_out.amax(0),
+                             in_coords[:, 0].long().amax().expand(D - 3),
+                             out_coords[:, 0].long().amax().expand(D - 3)]).cpu()
+        batches = int(max(stats[4, 0], stats[5, 0])) + 1
+        for e in range(D - 3):
+            lows.append(min(int(stats[0, e]), int(stats[2, e]) + min(steps[3 + e])))
+            highs.append(max(int(stats[1, e]), int(stats[3, e]) + max(steps[3 + e])))
+    else:
+        batches = 1
+        lows, highs = [0] * (D - 3), [0] * (D - 3)
+    widths = [h - l + 1 for l, h in zip(lows, highs)]
+    if batches * int(np.prod(widths)) >= 2 ** 31:
+        raise ValueError("the range of the dimensions past the third does not fit the batch column "
+                         f"({batches} batch items x {widths})")
+
+    def folded(rows, ext, shift):
+        b = rows[:, 0].long()
+        for e in range(D - 3):
+            b = b * widths[e] + (ext[:, e] + shift[e] - lows[e])
+        return torch.cat([b.to(torch.int32).unsqueeze(1), rows[:, 1:4]], dim=1).contiguous()
+
+    in3 = folded(in_coords, ext_in, [0] * (D - 3))
+    K3 = int(np.prod(ks[:3]))
+    combos = [[]]
+    for e in range(D - 3):
+        combos = [c + [o] for c in combos for o in steps[3 + e]]
+    maps = []
+    for shift in combos:
+        out3 = folded(out_coords, ext_out, shift)
+        maps.append(generate_kernel_map(in3, out3, stride[:3], ks[:3], dil[:3], centres[:3],
+                                        method="offset", hash_method=hash_method))
+    counts = torch.stack([torch.diff(m.offsets) for m in maps], dim=1).reshape(-1)  # (K3, combos) -> k
+    offsets = torch.cat([torch.zeros(1, dtype=counts.dtype), counts.cumsum(0)]).to(torch.int32)
+    ins = [m.in_maps[int(m.offsets[k]):int(m.offsets[k + 1])] for k in range(K3) for m in maps]
+    outs = [m.out_maps[int(m.offsets[k]):int(m.offsets[k + 1])] for k in range(K3) for m in maps]
+    K = K3 * len(combos)
+    is_odd = all(k % 2 == 1 for k in ks)
+    same_count = in_coords.shape[0] == out_coords.shape[0]
+    identity_map_index = K // 2 if (is_odd and same_count and centres == _kernel_centres(ks)) else None
+    empty = torch.empty(0, dtype=torch.int32, device=device)
+    result = IntSearchResult(torch.cat(ins) if ins else empty, torch.cat(outs) if outs else empty,
+                             offsets, identity_map_index=identity_map_index)
+    result._out_ascend = True
+    result._from_builder = True
+    result._keys_unique = all(getattr(m, "_keys_unique", False) for m in maps)
+    if skip_symmetric_kernel_map and is_odd:
+        half = K // 2
+        end = int(result.offsets[half])
+        result = IntSearchResult(result.in_maps[:end], result.out_maps[:end],
+                                 result.offsets[: half + 1].clone(), identity_map_index=identity_map_index)
+        result._out_ascend = True
+    return result
+
+
+@torch.no_grad()
 def generate_kernel_map(
     batch_indexed_in_coords: Tensor,
     batch_indexed_out_coords: Tensor,
@@ -212,7 +290,9 @@ def generate_kernel_map(
         assert kernel_center_offset is None, \
             "Custom kernel_center_offset is not supported with method='size'. Use method='offset' instead."
     if num_spatial_dims > 3:
-        raise NotImplementedError("more than 3 spatial dimensions are not supported")
+        return _kernel_map_more_dims(batch_indexed_in_coords, batch_indexed_out_coords,
+                                     in_to_out_stride_ratio, kernel_size, kernel_dilation,
+                                     kernel_center_offset, hash_method, skip_symmetric_kernel_map)
 
     table = _table_of(batch_indexed_in_coords, hash_method, device)
 
