@@ -183,6 +183,20 @@ int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_strid
                       void* workspace, int64_t capacity, int32_t* out_coords,
                       int32_t* first_index, void* stream);
 
+/* The same result for strides of 1, 2 or 4 per dimension through a table that already exists: the
+ * wcn_table_build of `coords` itself (the one the kernel maps of that resolution use).  Such a
+ * coarse cell is a sub-box of one 4x4x4 block, so its voxels are bits of one slot and the lowest
+ * of their rows represents the cell: one slot look-up and a few loads per row, no table over the
+ * coarse rows (which wcn_stride_unique builds from n rows that repeat up to 64-fold).  `workspace`:
+ * wcn_stride_unique_cells_workspace_bytes(n_keys) bytes; the result is read with
+ * wcn_stride_unique_read_count / _read_bounds as after wcn_stride_unique (same n and capacity).
+ * Replaces the same reference path (geometry/coords/ops/stride.py:17-54 + utils/unique.py:125-144). */
+size_t wcn_stride_unique_cells_workspace_bytes(int64_t n);
+
+int wcn_stride_unique_cells(const void* table, int64_t n_keys, int64_t capacity, const int32_t* coords,
+                            const int32_t host_stride[3], void* workspace, int32_t* out_coords,
+                            int32_t* first_index, void* stream);
+
 /* Waits for the stream; host_count receives M.  Returns the table status. */
 int wcn_stride_unique_read_count(const void* workspace, int64_t n, int64_t capacity,
                                  int64_t* host_count, void* stream);

@@ -38,6 +38,8 @@ SIGNATURES = {
     "wcn_kmap_last_table_flags": (_i32, []),
     "wcn_stride_unique_workspace_bytes": (_sz, [_i64, _i64]),
     "wcn_stride_unique": (ctypes.c_int, [_vp, _i64, _i32p, _vp, _i64, _vp, _vp, _vp]),
+    "wcn_stride_unique_cells_workspace_bytes": (_sz, [_i64]),
+    "wcn_stride_unique_cells": (ctypes.c_int, [_vp, _i64, _i64, _vp, _i32p, _vp, _vp, _vp, _vp]),
     "wcn_stride_unique_read_count": (ctypes.c_int, [_vp, _i64, _i64, _i64p, _vp]),
     "wcn_stride_unique_read_bounds": (ctypes.c_int, [_vp, _i64, _i64, _i64p, _i64p, _vp]),
     "wcn_conv_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _i32, _i64, _i32]),

@@ -1063,6 +1063,64 @@ __global__ void __launch_bounds__(256) stride_pick(const int4* __restrict__ coar
   }
 }
 
+// The same selection through the table of the FINE coordinates, for strides of 1, 2 or 4 per
+// dimension: such a coarse cell is a sub-box of one 4x4x4 block (the blocks' origins are multiples
+// of 4), so its voxels are bits of one slot's mask, their rows stand next to each other in perm, and
+// the cell's representative is the lowest of them.  No table over the coarse rows is needed: one
+// slot look-up and at most sx * sy * sz loads of perm per row.  LOG: log2 of the strides.
+template <bool FILL>
+__global__ void __launch_bounds__(256) stride_pick_cells(const int4* __restrict__ coords, int64_t n,
+                                                         const WcnTableHeader* __restrict__ hdr,
+                                                         const WcnSlot* __restrict__ slots,
+                                                         uint32_t cap_mask,
+                                                         const int32_t* __restrict__ perm,
+                                                         int lx, int ly, int lz,
+                                                         int32_t* __restrict__ groups, int64_t G,
+                                                         int4* __restrict__ out_coords,
+                                                         int32_t* __restrict__ first_index) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t group = i >> 6;
+  if (group >= G) return;
+  const int lane = wcn_lane();
+  bool winner = false;
+  int4 c = make_int4(0, 0, 0, 0);
+  if (i < n) {
+    const WcnLayout L = wcn_make_layout(hdr);
+    c = coords[i];
+    uint32_t r[4];
+    if (L.ok && wcn_relative(L, c.x, c.y, c.z, c.w, r)) {
+      int32_t base = 0;
+      const unsigned long long mask = wcn_lookup_block(slots, cap_mask, wcn_block_key(L, r), &base);
+      // the bits of the block that lie in this row's coarse cell
+      const uint32_t x0 = (r[1] & 3u) >> lx << lx, y0 = (r[2] & 3u) >> ly << ly, z0 = (r[3] & 3u) >> lz << lz;
+      const unsigned long long zs = ((1ull << (1 << lz)) - 1ull) << z0;          // within a row of 4 bits
+      unsigned long long ys = 0ull, cell = 0ull;
+      for (int dy = 0; dy < (1 << ly); ++dy) ys |= zs << ((y0 + dy) * 4);       // within a plane of 16 bits
+      for (int dx = 0; dx < (1 << lx); ++dx) cell |= ys << ((x0 + dx) * 16);
+      unsigned long long siblings = mask & cell;
+      int32_t lowest = INT32_MAX;
+      while (siblings) {
+        const int b = __builtin_ctzll(siblings);
+        siblings &= siblings - 1ull;
+        const int64_t pos = (int64_t)base + wcn_rank_below(mask, (uint32_t)b);
+        if (pos >= 0 && pos < n) lowest = min(lowest, perm[pos]);
+      }
+      winner = lowest == (int32_t)i;
+      c.y = floor_div(c.y, 1 << lx);
+      c.z = floor_div(c.z, 1 << ly);
+      c.w = floor_div(c.w, 1 << lz);
+    }
+  }
+  const unsigned long long wins = __ballot(winner);
+  if (!FILL) {
+    if (lane == 0) groups[group] = __popcll(wins);
+  } else if (winner) {
+    const int64_t pos = (int64_t)groups[group] + __popcll(wins & ((1ull << lane) - 1ull));
+    out_coords[pos] = c;
+    first_index[pos] = (int32_t)i;
+  }
+}
+
 __global__ void stride_finish(int64_t* __restrict__ result, const int32_t* __restrict__ groups,
                               int64_t G, const WcnTableHeader* __restrict__ hdr) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
@@ -1334,6 +1392,52 @@ int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_strid
                        (const int4*)w.coarse, n, v.hdr, v.slots, v.slot_of, v.perm, w.groups, w.G,
                        (int4*)out_coords, first_index);
     hipLaunchKernelGGL(stride_batch_bounds, dim3(1), dim3(1024), 0, s, (const int4*)out_coords, w.result);
+  }
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+size_t wcn_stride_unique_cells_workspace_bytes(int64_t n) {
+  if (n < 0) return 0;
+  return wcn_align256(sizeof(int64_t) * (size_t)(4 + STRIDE_BATCH_MARKS)) +
+         wcn_align256(sizeof(int32_t) * (size_t)((n + 63) / 64 + 1));
+}
+
+int wcn_stride_unique_cells(const void* table, int64_t n_keys, int64_t capacity, const int32_t* coords,
+                            const int32_t host_stride[3], void* workspace, int32_t* out_coords,
+                            int32_t* first_index, void* stream) {
+  if (!table_args_ok(table, n_keys, capacity) || !workspace || !host_stride || n_keys >= (1ll << 31))
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (n_keys > 0 && (!coords || !out_coords || !first_index)) return WCN_ERR_INVALID_ARGUMENT;
+  int lg[3];
+  for (int d = 0; d < 3; ++d) {
+    if (host_stride[d] != 1 && host_stride[d] != 2 && host_stride[d] != 4) return WCN_ERR_INVALID_ARGUMENT;
+    lg[d] = host_stride[d] == 1 ? 0 : (host_stride[d] == 2 ? 1 : 2);
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t n = n_keys;
+  WcnTableView v;
+  wcn_table_layout(const_cast<void*>(table), n_keys, capacity, &v);
+  // the result block first, as in the workspace of wcn_stride_unique (the read calls find it there)
+  int64_t* result = (int64_t*)workspace;
+  int32_t* groups = (int32_t*)((char*)workspace + wcn_align256(sizeof(int64_t) * (size_t)(4 + STRIDE_BATCH_MARKS)));
+  const int64_t G = (n + 63) / 64;
+  const uint32_t cap_mask = (uint32_t)(capacity - 1);
+  if (n > 0) {
+    hipLaunchKernelGGL(stride_pick_cells<false>, dim3(grid_for(n, 256)), dim3(256), 0, s, (const int4*)coords,
+                       n, v.hdr, v.slots, cap_mask, v.perm, lg[0], lg[1], lg[2], groups, G, (int4*)nullptr,
+                       (int32_t*)nullptr);
+  }
+  {
+    const KmapFinish none = {nullptr, nullptr, nullptr, 0, nullptr, 0};
+    hipLaunchKernelGGL(kmap_scan_rows, dim3(1), dim3(1024), 0, s, groups, G, result + 2, none);
+  }
+  hipLaunchKernelGGL(stride_finish, dim3(1), dim3(64), 0, s, result, groups, G, v.hdr);
+  if (n > 0) {
+    hipLaunchKernelGGL(stride_pick_cells<true>, dim3(grid_for(n, 256)), dim3(256), 0, s, (const int4*)coords,
+                       n, v.hdr, v.slots, cap_mask, v.perm, lg[0], lg[1], lg[2], groups, G, (int4*)out_coords,
+                       first_index);
+    hipLaunchKernelGGL(stride_batch_bounds, dim3(1), dim3(1024), 0, s, (const int4*)out_coords, result);
   }
   WCN_LAUNCH_CHECK();
   return WCN_OK;

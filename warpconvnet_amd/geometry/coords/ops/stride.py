@@ -68,22 +68,45 @@ def unique_floor_div_rows(batch_indexed_coords: Tensor, stride: Tuple[int, ...],
     coords = _four_columns(batch_indexed_coords)
     n = coords.shape[0]
     L = lib()
-    st = int3(list(ntuple(stride, ndim=num_spatial_dims)) + [1] * (3 - num_spatial_dims))
+    strides = list(ntuple(stride, ndim=num_spatial_dims)) + [1] * (3 - num_spatial_dims)
+    st = int3(strides)
     out = torch.empty((n, 4), dtype=torch.int32, device=device)
     first = torch.empty(n, dtype=torch.int32, device=device)
-    slots = L.wcn_table_default_capacity(n)
     count = ctypes.c_int64(0)
     bounds = (ctypes.c_int64 * 1025)() if want_bounds else None
+
+    def read(ws, slots):
+        if want_bounds:
+            return L.wcn_stride_unique_read_bounds(ptr(ws), n, slots, ctypes.byref(count), bounds,
+                                                   stream_ptr(device))
+        return L.wcn_stride_unique_read_count(ptr(ws), n, slots, ctypes.byref(count), stream_ptr(device))
+
+    if all(int(v) in (1, 2, 4) for v in strides) and n > 0:
+        # Cells of 1, 2 or 4 voxels per dimension lie inside the 4x4x4 blocks of the table of the
+        # fine coordinates (the one this resolution's kernel maps use, kept on the tensor object):
+        # the distinct coarse rows come out of that table, no second table is built.
+        from ..search.torch_discrete import _table_of
+        from ..search.torch_hashmap import HashMethod
+        table = _table_of(batch_indexed_coords, HashMethod.CITY, device)
+        while True:
+            raw, n_keys, slots = table._raw()  # the table's own four-column copy of the rows
+            ws = workspace(L.wcn_stride_unique_cells_workspace_bytes(n), device)
+            check(L.wcn_stride_unique_cells(ptr(raw), n_keys, slots, ptr(table._keys4), st, ptr(ws), ptr(out),
+                                            ptr(first), stream_ptr(device)), "wcn_stride_unique_cells")
+            status = read(ws, slots)
+            if status == ERR_TABLE_OVERFLOW:
+                table._grow()
+                continue
+            check(status, "wcn_stride_unique_cells")
+            table._checked = True
+            return out, int(count.value), (list(bounds) if want_bounds else None)
+
+    slots = L.wcn_table_default_capacity(n)
     while True:
         ws = workspace(L.wcn_stride_unique_workspace_bytes(n, slots), device)
         check(L.wcn_stride_unique(ptr(coords), n, st, ptr(ws), slots, ptr(out), ptr(first),
                                   stream_ptr(device)), "wcn_stride_unique")
-        if want_bounds:
-            status = L.wcn_stride_unique_read_bounds(ptr(ws), n, slots, ctypes.byref(count), bounds,
-                                                     stream_ptr(device))
-        else:
-            status = L.wcn_stride_unique_read_count(ptr(ws), n, slots, ctypes.byref(count),
-                                                    stream_ptr(device))
+        status = read(ws, slots)
         if status == ERR_TABLE_OVERFLOW and slots < (1 << 30):
             slots *= 4
             continue
