@@ -1076,12 +1076,24 @@ __global__ void __launch_bounds__(256) stride_pick_cells(const int4* __restrict_
                                                          const int32_t* __restrict__ perm,
                                                          int lx, int ly, int lz,
                                                          int32_t* __restrict__ groups, int64_t G,
+                                                         unsigned long long* __restrict__ picked,
                                                          int4* __restrict__ out_coords,
                                                          int32_t* __restrict__ first_index) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t group = i >> 6;
   if (group >= G) return;
   const int lane = wcn_lane();
+  if (FILL) {
+    // the counting pass left the group's representatives as a mask: no second look-up
+    const unsigned long long wins = picked[group];
+    if ((wins >> lane) & 1ull) {
+      const int4 c = coords[i];
+      const int64_t pos = (int64_t)groups[group] + __popcll(wins & ((1ull << lane) - 1ull));
+      out_coords[pos] = make_int4(c.x, floor_div(c.y, 1 << lx), floor_div(c.z, 1 << ly), floor_div(c.w, 1 << lz));
+      first_index[pos] = (int32_t)i;
+    }
+    return;
+  }
   bool winner = false;
   int4 c = make_int4(0, 0, 0, 0);
   if (i < n) {
@@ -1106,18 +1118,12 @@ __global__ void __launch_bounds__(256) stride_pick_cells(const int4* __restrict_
         if (pos >= 0 && pos < n) lowest = min(lowest, perm[pos]);
       }
       winner = lowest == (int32_t)i;
-      c.y = floor_div(c.y, 1 << lx);
-      c.z = floor_div(c.z, 1 << ly);
-      c.w = floor_div(c.w, 1 << lz);
     }
   }
   const unsigned long long wins = __ballot(winner);
-  if (!FILL) {
-    if (lane == 0) groups[group] = __popcll(wins);
-  } else if (winner) {
-    const int64_t pos = (int64_t)groups[group] + __popcll(wins & ((1ull << lane) - 1ull));
-    out_coords[pos] = c;
-    first_index[pos] = (int32_t)i;
+  if (lane == 0) {
+    groups[group] = __popcll(wins);
+    picked[group] = wins;
   }
 }
 
@@ -1400,7 +1406,8 @@ int wcn_stride_unique(const int32_t* coords, int64_t n, const int32_t host_strid
 size_t wcn_stride_unique_cells_workspace_bytes(int64_t n) {
   if (n < 0) return 0;
   return wcn_align256(sizeof(int64_t) * (size_t)(4 + STRIDE_BATCH_MARKS)) +
-         wcn_align256(sizeof(int32_t) * (size_t)((n + 63) / 64 + 1));
+         wcn_align256(sizeof(int32_t) * (size_t)((n + 63) / 64 + 1)) +
+         wcn_align256(sizeof(unsigned long long) * (size_t)((n + 63) / 64));
 }
 
 int wcn_stride_unique_cells(const void* table, int64_t n_keys, int64_t capacity, const int32_t* coords,
@@ -1422,11 +1429,12 @@ int wcn_stride_unique_cells(const void* table, int64_t n_keys, int64_t capacity,
   int64_t* result = (int64_t*)workspace;
   int32_t* groups = (int32_t*)((char*)workspace + wcn_align256(sizeof(int64_t) * (size_t)(4 + STRIDE_BATCH_MARKS)));
   const int64_t G = (n + 63) / 64;
+  unsigned long long* picked = (unsigned long long*)((char*)groups + wcn_align256(sizeof(int32_t) * (size_t)(G + 1)));
   const uint32_t cap_mask = (uint32_t)(capacity - 1);
   if (n > 0) {
     hipLaunchKernelGGL(stride_pick_cells<false>, dim3(grid_for(n, 256)), dim3(256), 0, s, (const int4*)coords,
-                       n, v.hdr, v.slots, cap_mask, v.perm, lg[0], lg[1], lg[2], groups, G, (int4*)nullptr,
-                       (int32_t*)nullptr);
+                       n, v.hdr, v.slots, cap_mask, v.perm, lg[0], lg[1], lg[2], groups, G, picked,
+                       (int4*)nullptr, (int32_t*)nullptr);
   }
   {
     const KmapFinish none = {nullptr, nullptr, nullptr, 0, nullptr, 0};
@@ -1435,8 +1443,8 @@ int wcn_stride_unique_cells(const void* table, int64_t n_keys, int64_t capacity,
   hipLaunchKernelGGL(stride_finish, dim3(1), dim3(64), 0, s, result, groups, G, v.hdr);
   if (n > 0) {
     hipLaunchKernelGGL(stride_pick_cells<true>, dim3(grid_for(n, 256)), dim3(256), 0, s, (const int4*)coords,
-                       n, v.hdr, v.slots, cap_mask, v.perm, lg[0], lg[1], lg[2], groups, G, (int4*)out_coords,
-                       first_index);
+                       n, v.hdr, v.slots, cap_mask, v.perm, lg[0], lg[1], lg[2], groups, G, picked,
+                       (int4*)out_coords, first_index);
     hipLaunchKernelGGL(stride_batch_bounds, dim3(1), dim3(1024), 0, s, (const int4*)out_coords, result);
   }
   WCN_LAUNCH_CHECK();
