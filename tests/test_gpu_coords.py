@@ -469,3 +469,27 @@ def test_kernel_map_over_more_than_three_dimensions(name, D, n, extent, ksize, s
     if km.identity_map_index is not None:
         i, o = km[km.identity_map_index]
         assert torch.equal(i, o) and len(i) == len(rows)
+
+
+@pytest.mark.parametrize("stride", [(2, 2, 2), (4, 4, 4), (4, 2, 1), (1, 1, 2), (3, 2, 2)],
+                         ids=["s2", "s4", "s421", "s112", "s322_other_path"])
+def test_strided_coordinates_with_negative_coordinates_and_repeated_rows(oracle, stride):
+    """Strides of 1, 2, 4 take the distinct coarse rows out of the table of the fine rows (cells inside
+    4x4x4 blocks); any other stride builds a table over the coarse rows.  Both against the oracle, in
+    this implementation's order (ascending first source row), with coordinates on both sides of zero
+    and with fine rows that repeat."""
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    rng = np.random.default_rng(sum(stride))
+    rows = rng.integers(-37, 41, size=(30000, 4)).astype(np.int32)
+    rows[:, 0] = np.sort(rng.integers(0, 3, size=len(rows)))
+    rows = np.concatenate([rows, rows[rng.integers(0, len(rows), 2000)]])  # repeats, batch column no longer sorted
+    for batch_sorted in (False, True):
+        use = rows[np.argsort(rows[:, 0], kind="stable")] if batch_sorted else rows
+        got, got_off = stride_coords(_dev(use), stride, batch_sorted=batch_sorted)
+        ref_out, _, ref_off = oracle.stride_coords(use, stride, 3)
+        if batch_sorted:  # same rows in the same order, same offsets
+            assert np.array_equal(got.cpu().numpy(), ref_out), stride
+            assert np.array_equal(got_off.numpy().astype(np.int64), ref_off)
+        else:             # the oracle orders by batch item afterwards, as the reference does
+            assert np.array_equal(sort_rows(got.cpu().numpy()), sort_rows(ref_out)), stride
+            assert np.array_equal(got_off.numpy().astype(np.int64), ref_off)
