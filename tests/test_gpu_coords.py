@@ -398,17 +398,21 @@ def test_morton_codes_and_sort():
 def test_kernel_map_with_more_pairs_than_assumed(oracle):
     """A dense cube has ~27 pairs per voxel, more than the buffers the emit pass is first enqueued
     into hold: that pass must leave them untouched and the second, exact one produce the map."""
+    from warpconvnet_amd.geometry.coords.search import torch_discrete
     from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
     S = 24
     g = np.stack(np.meshgrid(np.arange(S), np.arange(S), np.arange(S), indexing="ij"), -1).reshape(-1, 3)
     rng = np.random.default_rng(0)
     rng.shuffle(g)
     bc = np.concatenate([np.zeros((len(g), 1), np.int32), g.astype(np.int32)], axis=1)
-    km = generate_kernel_map(_dev(bc), _dev(bc), (1, 1, 1), (3, 3, 3))
     im, om, off, iden = oracle.kernel_map(bc, bc, (3, 3, 3))
-    assert int(km.offsets[-1]) == len(im) > 8 * len(bc)
-    assert np.array_equal(km.in_maps.cpu().numpy(), im) and np.array_equal(km.out_maps.cpu().numpy(), om)
-    assert np.array_equal(km.offsets.numpy().astype(np.int64), off)
+    torch_discrete._PAIRS_PER_ROW.clear()  # nothing remembered: eight pairs per row are assumed
+    for attempt in range(2):               # the second build sizes its buffers by what the first one held
+        km = generate_kernel_map(_dev(bc), _dev(bc), (1, 1, 1), (3, 3, 3))
+        assert int(km.offsets[-1]) == len(im) > 8 * len(bc)
+        assert np.array_equal(km.in_maps.cpu().numpy(), im) and np.array_equal(km.out_maps.cpu().numpy(), om)
+        assert np.array_equal(km.offsets.numpy().astype(np.int64), off)
+    assert max(torch_discrete._PAIRS_PER_ROW.values()) > 8
 
 
 def _brute_force_map(in_rows, out_rows, stride, ksize, dilation=None):

@@ -58,6 +58,11 @@ def _pad_kernel_args(values: Sequence[int], fill: int):
     return values + [fill] * (3 - len(values))
 
 
+# pairs per output row of the last map built for (kernel size, stride, size class of the row count):
+# sizes the buffers the pairs are emitted into before their number is known
+_PAIRS_PER_ROW = {}
+
+
 @torch.no_grad()
 def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_size, stride,
                            identity_map_index: Optional[int], dilation=None,
@@ -78,7 +83,12 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
     # to the host (a voxel of a surface-like scene has a handful of neighbours, far from K); the
     # lists handed out are views of these buffers.  More pairs than assumed: the emit pass has
     # written nothing and runs again with exact buffers.
-    assumed = min(K * M, max(8 * M, 1 << 16))
+    # Eight per row unless a map of this kernel and size class was built before: then what that
+    # one held, with a quarter to spare (the resolutions of a network differ a lot: 4 pairs per
+    # voxel of a scene's surface at the finest level, 14 two levels down).
+    shape_key = (tuple(int(k) for k in kernel_size), tuple(int(v) for v in stride), M.bit_length())
+    per_row = _PAIRS_PER_ROW.get(shape_key, 8.0)
+    assumed = min(K * M, max(int(1.25 * per_row * M) + 4096, 1 << 16))
     in_buf = torch.empty(assumed, dtype=torch.int32, device=device)
     out_buf = torch.empty(assumed, dtype=torch.int32, device=device)
     # A coordinate set mapped onto itself can also be probed block by block (WCN_KMAP_PROBE=blocks:
@@ -131,6 +141,8 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
         table._checked = True
         break
     total = int(host_offsets[K])
+    if M > 0:
+        _PAIRS_PER_ROW[shape_key] = total / M
     if 2 * total <= assumed and (assumed - total) * 4 > (32 << 20):
         # far fewer pairs than assumed, and more than 32 MiB of each buffer unused: exact copies,
         # so the map does not hold the large buffers (below that the two copy kernels cost more
