@@ -35,11 +35,15 @@ def _run(cmd):
 # compiler spills (or otherwise moves) while such a load is still in flight would be overwritten
 # later by the landing data.  These files must compile without any scratch memory.
 NO_SCRATCH_SOURCES = ("wcn_conv_pack_f16.hip", "wcn_conv_pack_bf16.hip", "wcn_conv_pack_f32.hip")
+# Sources whose waits are the compiler's, so that a spill is safe, but whose instances are sized to
+# their register budget (waves per workgroup chosen so that nothing spills): scratch memory there is
+# a slower kernel that nobody asked for, and the build says so.
+NO_SPILL_SOURCES = ("wcn_conv_group.hip",)
 _REMARK = "-Rpass-analysis=kernel-resource-usage"
 
 
 def _extra_flags(src):
-    return [_REMARK] if os.path.basename(src) in NO_SCRATCH_SOURCES else []
+    return [_REMARK] if os.path.basename(src) in NO_SCRATCH_SOURCES + NO_SPILL_SOURCES else []
 
 
 def _without_remarks(log):
@@ -47,7 +51,7 @@ def _without_remarks(log):
 
 
 def _check_no_scratch(src, log):
-    if os.path.basename(src) not in NO_SCRATCH_SOURCES:
+    if os.path.basename(src) not in NO_SCRATCH_SOURCES + NO_SPILL_SOURCES:
         return
     name, seen = None, 0
     for line in log.splitlines():
@@ -57,9 +61,10 @@ def _check_no_scratch(src, log):
             seen += 1
             value = int(line.split(":")[-1].split("[")[0].strip())
             if value != 0:
+                why = ("its hand-counted loads make that unsafe" if os.path.basename(src) in NO_SCRATCH_SOURCES
+                       else "its instances are meant to fit their register budget")
                 raise RuntimeError(f"{os.path.basename(src)}: kernel {name} uses scratch memory / spills vector "
-                                   f"registers ({line.split('remark:')[1].strip()}); its hand-counted loads "
-                                   "make that unsafe")
+                                   f"registers ({line.split('remark:')[1].strip()}); {why}")
     if seen == 0:
         raise RuntimeError(f"{os.path.basename(src)}: no resource-usage remarks found; cannot vouch for its kernels")
 

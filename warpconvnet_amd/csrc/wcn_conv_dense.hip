@@ -42,7 +42,9 @@ using namespace wcn_mma;
 
 // NCB: 16-channel blocks of output channels (C_out / 16); DENSE_WAVES waves with DENSE_RB 16-row
 // blocks of output rows each: a tile is DENSE_WAVES * DENSE_RB * 16 output rows
-template <typename T, int NCB, int DENSE_WAVES, int DENSE_RB>
+// RES: the instance that reads a residual in its epilogue (those loads keep more registers alive
+// beside the sums, so calls without a residual get an instance without them)
+template <typename T, int NCB, int DENSE_WAVES, int DENSE_RB, bool RES>
 __global__ void __launch_bounds__(DENSE_WAVES * 64) conv_fwd_dense(ConvArgs a, int num_tiles) {
   constexpr int DENSE_THREADS = DENSE_WAVES * 64, DENSE_ROWS = DENSE_WAVES * DENSE_RB * 16;
   typedef typename Mma<T>::V V;
@@ -245,7 +247,7 @@ __global__ void __launch_bounds__(DENSE_WAVES * 64) conv_fwd_dense(ConvArgs a, i
         if (row < tile_rows) {
           T t[4];
           float r[4] = {0.f, 0.f, 0.f, 0.f};  // rows are whole 16-byte vectors here: 128 or 256 channels
-          if (a.residual) load_floats<T, 4>(static_cast<const T*>(a.residual) + (m0 + row) * a.c_out + col, r);
+          if (RES) load_floats<T, 4>(static_cast<const T*>(a.residual) + (m0 + row) * a.c_out + col, r);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float f = acc[rb][cb][e] + b[e] + r[e];
@@ -273,12 +275,12 @@ inline int dense_cus() {
   return cus[device];
 }
 
-template <typename T, int NCB, int WAVES, int RB>
-int launch_dense(const ConvArgs& a, hipStream_t s) {
+template <typename T, int NCB, int WAVES, int RB, bool RES>
+int launch_dense_instance(const ConvArgs& a, hipStream_t s) {
   constexpr int ROWS = WAVES * RB * 16;
   constexpr int lds = 2 * NCB * 16 * 8 * 16 + WAVES * RB * 16 * 4;
   static_assert(lds <= 160 * 1024, "LDS of one workgroup");
-  const void* fn = (const void*)conv_fwd_dense<T, NCB, WAVES, RB>;
+  const void* fn = (const void*)conv_fwd_dense<T, NCB, WAVES, RB, RES>;
   // more than 64 KiB of dynamic LDS has to be allowed once per device and kernel
   static std::mutex mu;
   static bool allowed[64] = {};
@@ -295,9 +297,15 @@ int launch_dense(const ConvArgs& a, hipStream_t s) {
   const int64_t tiles = (a.num_out + ROWS - 1) / ROWS;
   if (tiles <= 0 || tiles > INT32_MAX) return WCN_ERR_INVALID_ARGUMENT;
   const unsigned grid = (unsigned)std::min<int64_t>(tiles, dense_cus());
-  hipLaunchKernelGGL((conv_fwd_dense<T, NCB, WAVES, RB>), dim3(grid), dim3(WAVES * 64), lds, s, a, (int)tiles);
-  wcn_conv_note_kernel("conv_fwd_dense<%s, %d, %d, %d>", wcn_type_text<T>(), NCB, WAVES, RB);
+  hipLaunchKernelGGL((conv_fwd_dense<T, NCB, WAVES, RB, RES>), dim3(grid), dim3(WAVES * 64), lds, s, a, (int)tiles);
+  wcn_conv_note_kernel("conv_fwd_dense<%s, %d, %d, %d, %s>", wcn_type_text<T>(), NCB, WAVES, RB, RES ? "true" : "false");
   return hipGetLastError() == hipSuccess ? WCN_OK : WCN_ERR_LAUNCH;
+}
+
+template <typename T, int NCB, int WAVES, int RB>
+int launch_dense(const ConvArgs& a, hipStream_t s) {
+  return a.residual ? launch_dense_instance<T, NCB, WAVES, RB, true>(a, s)
+                    : launch_dense_instance<T, NCB, WAVES, RB, false>(a, s);
 }
 
 // Two tile shapes: 256 rows (eight waves of 32 rows, two per SIMD) and 192 rows (four waves of 48

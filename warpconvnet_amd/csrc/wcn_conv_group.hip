@@ -373,11 +373,12 @@ int launch_group_waves(const ConvArgs& a, hipStream_t s) {
 
 // Sixteen waves per workgroup (four per SIMD) where the sums of sixteen groups fit LDS beside the
 // weights, twelve otherwise (3x3x3 with 32 channels on both sides: 54 KB of weights and 8 KB of
-// sums per wave).  The one instance that does not stay within 128 registers has weights that fit
-// LDS for no kernel of more than 64 offsets and is not built.
+// sums per wave).  The instances for 32 input channels under more than 64 offsets do not stay
+// within the 128 registers of sixteen waves (one has weights that fit LDS for no such kernel anyway,
+// the other would spill a few registers): they are built for twelve waves only.
 template <typename T, int NCB, bool HALF_K, int NCH>
 int launch_group_chunks(const ConvArgs& a, hipStream_t s) {
-  if constexpr (!(NCB == 2 && !HALF_K && NCH == 2)) {
+  if constexpr (!(!HALF_K && NCH == 2)) {
     if (group_lds<T, NCB, HALF_K>(a.K, 16) <= GROUP_LDS_MAX) return launch_group_waves<T, NCB, HALF_K, NCH, 16>(a, s);
   }
   return launch_group_waves<T, NCB, HALF_K, NCH, 12>(a, s);
