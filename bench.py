@@ -236,9 +236,18 @@ def secondary_configs(dev, steps, warmup):
     t_map, (coarse, km) = timed(build)
     m = len(coarse)
     t_down, y = timed(lambda: sparse_conv_forward(x, wd, km, m))
+    # the transposed convolution's map as spatially_sparse_conv makes it: the forward map with its lists
+    # exchanged; kernel = stride over voxels without repeats, so every fine voxel has exactly one pair
     up = IntSearchResult(km.out_maps, km.in_maps, km.offsets)
     up._in_ascend, up._in_group_start = km._out_ascend, km._group_start
-    t_up, _ = timed(lambda: sparse_conv_forward(y, wu, up, n))
+    up._keys_unique, up._from_builder = km._keys_unique, True
+    up._single_out = bool(km._keys_unique and int(km.offsets[-1]) == n)
+    t_up, y_up = timed(lambda: sparse_conv_forward(y, wu, up, n))
+    # the same product by the general path (lists re-ordered once, sums in LDS), for comparison
+    up_general = IntSearchResult(km.out_maps, km.in_maps, km.offsets)
+    up_general._keys_unique, up_general._from_builder = km._keys_unique, True
+    t_up_general, y_general = timed(lambda: sparse_conv_forward(y, wu, up_general, n))
+    assert float((y_up.float() - y_general.float()).abs().max()) <= 2e-2 * float(y_general.float().abs().max())
     # consumers of the same maps: depthwise 3x3x3 over the 1M-voxel map, 2x2x2 stride-2 max pooling
     from warpconvnet_amd.nn.functional.sparse_conv_depth import spatially_sparse_depthwise_conv
     km3 = generate_kernel_map(c, c, (1, 1, 1), (3, 3, 3))
@@ -329,7 +338,7 @@ def secondary_configs(dev, steps, warmup):
     out["configs[2]: 2x2x2 s2 96->128 + transposed 128->96 bf16, 1M fine voxels"] = {
         "num_voxels": n, "num_coarse": m, "num_pairs": int(km.offsets[-1]),
         "coords_and_kernel_map_build_ms": t_map, "down_contraction_call_ms": t_down,
-        "up_contraction_call_ms": t_up, "voxels_per_s": n / ((t_map + t_down + t_up) * 1e-3)}
+        "up_contraction_call_ms": t_up, "up_contraction_call_general_path_ms": t_up_general, "voxels_per_s": n / ((t_map + t_down + t_up) * 1e-3)}
     return out
 
 

@@ -293,6 +293,30 @@ int wcn_sparse_conv_fwd_prepared(const void* features, int64_t num_in, int32_t c
                                  int64_t num_out, void* workspace, size_t workspace_bytes,
                                  void* stream);
 
+/* The forward contraction over a map in which EVERY OUTPUT ROW HAS EXACTLY ONE PAIR
+ * (host_offsets[num_offsets] == num_out, which is checked, and no output row twice, which the caller
+ * vouches for): the transposed convolution that undoes a strided convolution whose kernel is as large
+ * as its stride, where every fine voxel has one parent at one offset.  Nothing is accumulated across
+ * pairs, so the lists may be in any order inside an offset (a forward map with its lists exchanged is
+ * taken as it is, not re-ordered) and need no group-start table:
+ *
+ *   out[out_maps[p], :] = act(bias + features[in_maps[p], :] @ W[k(p)] + residual[out_maps[p], :])
+ *
+ * wcn_conv_single_supported says whether a shape is taken (16-bit features, c_in of 32, 64, 96, 128,
+ * 192 or 256, c_out a multiple of 8 up to 256, at most 64 offsets).  weight_is_prepared != 0: `weight`
+ * is the block wcn_conv_prepare_weight made (no workspace needed); otherwise W (K, c_in, c_out) as
+ * stored and a workspace of wcn_conv_prepared_weight_bytes bytes.  Replaces the same reference path as
+ * wcn_sparse_conv_fwd (sparse_conv.py:495-544 over the map of sparse_conv.py:1916-1939). */
+int wcn_conv_single_supported(int32_t dtype, int32_t c_in, int32_t c_out, int32_t num_offsets);
+
+int wcn_sparse_conv_fwd_single(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                               const void* weight, int32_t weight_dtype, int32_t weight_is_prepared,
+                               int32_t num_offsets, int32_t c_out, const void* bias_or_null,
+                               const int32_t* in_maps, const int32_t* out_maps,
+                               const int64_t* host_offsets, const void* residual_or_null, int32_t relu,
+                               void* out, int64_t num_out, void* workspace, size_t workspace_bytes,
+                               void* stream);
+
 /* wcn_sparse_conv_fwd for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
  * Same arguments and results as wcn_sparse_conv_fwd, minus the workspace: the scratch memory is a

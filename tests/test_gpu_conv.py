@@ -298,6 +298,65 @@ def test_strided_then_transposed_pair(oracle, dtype):
     assert rel_err(back.feature_tensor.float().cpu().numpy(), want) <= TOL[dtype]
 
 
+SINGLE_CASES = [
+    # name, dtype, coarse channels, fine channels, kernel = stride, voxels per item
+    ("bf16_32_32", torch.bfloat16, 32, 32, (2, 2, 2), 6000),
+    ("f16_64_32", torch.float16, 64, 32, (2, 2, 2), 6000),
+    ("bf16_128_96", torch.bfloat16, 128, 96, (2, 2, 2), 6000),
+    ("f16_256_128", torch.float16, 256, 128, (2, 2, 2), 3000),
+    ("bf16_96_200", torch.bfloat16, 96, 200, (2, 1, 2), 5000),   # 25 channel blocks: the last column group partly there
+    ("f16_192_8_k4", torch.float16, 192, 8, (4, 4, 4), 5000),    # 64 offsets, most of them with a handful of pairs
+]
+
+
+@pytest.mark.parametrize("name,dtype,c_coarse,c_fine,ks,n", SINGLE_CASES, ids=[c[0] for c in SINGLE_CASES])
+def test_transposed_convolution_with_one_pair_per_output_row(oracle, name, dtype, c_coarse, c_fine, ks, n):
+    """The transposed convolution that undoes a strided one with kernel = stride: every fine voxel has one
+    parent, so nothing is summed and the exchanged lists are used as they are (conv_fwd_single).  Against
+    the fp64 oracle, against the general path over the re-ordered lists, with residual and clamp in the
+    epilogue and with kept weight tiles."""
+    from warpconvnet_amd._lib import lib
+    from warpconvnet_amd.nn.functional.sparse_conv import (generate_output_coords_and_kernel_map,
+                                                         spatially_sparse_conv)
+    items = [synthetic.random_cloud(40 + b, n, 36)[:, 1:] for b in range(2)]
+    bc = synthetic.batch_indexed(items)
+    fine = _voxels(items, normal_features(len(bc), 8, seed=3, dtype=dtype))
+    wd = kaiming_weight(int(np.prod(ks)), 8, c_coarse, seed=4, dtype=dtype).to(DEV)
+    wu = kaiming_weight(int(np.prod(ks)), c_coarse, c_fine, seed=5, dtype=dtype).to(DEV)
+    bias = (torch.randn(c_fine, generator=torch.Generator().manual_seed(6)) * 0.1).to(dtype).to(DEV)
+    res = normal_features(len(bc), c_fine, seed=7, dtype=dtype).to(DEV)
+    with torch.no_grad():
+        coarse = spatially_sparse_conv(fine, wd, ks, stride=ks)
+        coarse = coarse.replace(batched_features=normal_features(len(coarse.feature_tensor), c_coarse, seed=8, dtype=dtype).to(DEV))
+        back = spatially_sparse_conv(coarse, wu, ks, stride=ks, bias=bias, transposed=True,
+                                     output_spatially_sparse_tensor=fine)
+        assert lib().wcn_conv_last_kernel().decode().startswith("conv_fwd_single<"), lib().wcn_conv_last_kernel()
+        _, _, km = generate_output_coords_and_kernel_map(coarse, ks, (1,) * 3, ks, False, True, fine)
+        assert km._single_out and km._by_out is None  # no re-ordered lists were made
+        # oracle: the forward map with its lists exchanged
+        coarse_bc = coarse.batch_indexed_coordinates.cpu().numpy()
+        im, om, off, _ = oracle.kernel_map(bc, coarse_bc, ks, ks)
+        want = oracle.explicit_conv_f64(coarse.feature_tensor.double().cpu().numpy(), wu.double().cpu().numpy(),
+                                        om, im, off, None, len(bc)) + bias.double().cpu().numpy()
+        got = back.feature_tensor.float().cpu().numpy()
+        assert rel_err(got, want) <= TOL[dtype] and elementwise_rel_err(got, want) <= 5e-2  # one product per entry
+        # residual, clamp and kept tiles
+        fused = spatially_sparse_conv(coarse, wu, ks, stride=ks, bias=bias, transposed=True,
+                                      output_spatially_sparse_tensor=fine, residual=res, relu=True)
+        ref = np.maximum(want + res.double().cpu().numpy(), 0.0)
+        assert rel_err(fused.feature_tensor.float().cpu().numpy(), ref) <= TOL[dtype]
+        kept = spatially_sparse_conv(coarse, wu, ks, stride=ks, bias=bias, transposed=True,
+                                     output_spatially_sparse_tensor=fine, keep_prepared_weight=True)
+        assert torch.equal(kept.feature_tensor, back.feature_tensor)
+        # the general path over the same map (lists re-ordered, sums in LDS): same result up to rounding
+        km._single_out = False
+        general = spatially_sparse_conv(coarse, wu, ks, stride=ks, bias=bias, transposed=True,
+                                        output_spatially_sparse_tensor=fine)
+        assert not lib().wcn_conv_last_kernel().decode().startswith("conv_fwd_single<")
+        assert rel_err(general.feature_tensor.float().cpu().numpy(), want) <= TOL[dtype]
+        km._single_out = True
+
+
 def test_pair_lists_are_reordered_once_and_kept_on_the_map(oracle):
     """The map of a transposed convolution does not ascend in output row: its re-ordered lists
     are made on the first product and the very same tensors serve the second one."""

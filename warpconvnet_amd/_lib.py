@@ -55,6 +55,9 @@ SIGNATURES = {
     "wcn_sparse_conv_fwd_prepared": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _sz, _i32, _i32, _vp, _vp,
                                                     _vp, _i64p, _vp, _i32, _vp, _vp, _i32, _vp, _i64,
                                                     _vp, _sz, _vp]),
+    "wcn_conv_single_supported": (ctypes.c_int, [_i32, _i32, _i32, _i32]),
+    "wcn_sparse_conv_fwd_single": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _vp, _vp,
+                                                  _vp, _i64p, _vp, _i32, _vp, _i64, _vp, _sz, _vp]),
     "wcn_sparse_conv_fwd_static": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp,
                                                   _vp, _i64p, _i32, _i32, _vp, _vp, _i64, _vp]),
     "wcn_pairs_sort_workspace_bytes": (_sz, [_i64, _i32, _i64]),

@@ -1667,6 +1667,64 @@ int wcn_sparse_conv_fwd_prepared(const void* features, int64_t num_in, int32_t c
                   device_offsets);
 }
 
+int wcn_conv_single_supported(int32_t dtype, int32_t c_in, int32_t c_out, int32_t num_offsets) {
+  return wcn_conv_single_takes(dtype, c_in, c_out, num_offsets) ? 1 : 0;
+}
+
+int wcn_sparse_conv_fwd_single(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,
+                               const void* weight, int32_t weight_dtype, int32_t weight_is_prepared,
+                               int32_t num_offsets, int32_t c_out, const void* bias_or_null,
+                               const int32_t* in_maps, const int32_t* out_maps,
+                               const int64_t* host_offsets, const void* residual_or_null, int32_t relu,
+                               void* out, int64_t num_out, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+  if (!wcn_conv_single_takes(dtype, c_in, c_out, num_offsets) || !features || !weight || !host_offsets || !out ||
+      num_in <= 0 || num_out <= 0 || num_in >= (1ll << 31) || num_out >= (1ll << 31))
+    return WCN_ERR_INVALID_ARGUMENT;
+  if (residual_or_null && residual_or_null == out) return WCN_ERR_INVALID_ARGUMENT;
+  if (!weight_is_prepared && weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32) return WCN_ERR_INVALID_ARGUMENT;
+  const int64_t L = host_offsets[num_offsets];
+  if (host_offsets[0] != 0 || L != num_out || !in_maps || !out_maps) return WCN_ERR_INVALID_ARGUMENT;  // one pair per output row
+  for (int k = 0; k < num_offsets; ++k)
+    if (host_offsets[k + 1] < host_offsets[k]) return WCN_ERR_INVALID_ARGUMENT;
+  const size_t es = elem_size(dtype);
+  if ((uintptr_t)features % 16 != 0 || (uintptr_t)out % 16 != 0 || ((size_t)c_out * es) % 16 != 0 ||
+      (bias_or_null && (uintptr_t)bias_or_null % 8 != 0) || (residual_or_null && (uintptr_t)residual_or_null % 16 != 0))
+    return WCN_ERR_INVALID_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  ConvArgs a = {};
+  a.X = features;
+  a.bias = bias_or_null;
+  a.residual = residual_or_null;
+  a.relu = relu ? 1 : 0;
+  a.in_maps = in_maps;
+  a.out_maps = out_maps;
+  a.out = out;
+  a.num_in = num_in;
+  a.num_out = num_out;
+  a.num_pairs = L;
+  a.K = num_offsets;
+  a.c_in = c_in;
+  a.c_out = c_out;
+  a.c_in_pad = round_up(c_in, ck_of(dtype));
+  a.c_out_pad = round_up(c_out, TN);
+  a.identity = -1;
+  if (weight_is_prepared) {
+    a.Wt = weight;
+  } else {
+    const size_t need = wcn_conv_prepared_weight_bytes(num_offsets, c_in, c_out, dtype);
+    if (!workspace || workspace_bytes < need) return WCN_ERR_WORKSPACE;
+    a.Wt = workspace;
+    if (dtype == WCN_DTYPE_F16) launch_prep<_Float16>(a, weight, weight_dtype, dtype, 0, 0, nullptr, s);
+    else launch_prep<__bf16>(a, weight, weight_dtype, dtype, 0, 0, nullptr, s);
+  }
+  if (g_time_start) (void)hipEventRecord(g_time_start, s);
+  const int rc = wcn_conv_single_launch(a, dtype, host_offsets, s);
+  if (g_time_stop) (void)hipEventRecord(g_time_stop, s);
+  g_time_start = g_time_stop = nullptr;
+  return rc;
+}
+
 int wcn_sparse_conv_dgrad(const void* grad_out, int64_t num_out, int32_t c_out, int32_t dtype,
                           const void* weight, int32_t weight_dtype, int32_t num_offsets,
                           int32_t c_in, const int32_t* in_maps, const int32_t* out_maps,

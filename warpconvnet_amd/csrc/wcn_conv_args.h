@@ -45,6 +45,18 @@ int wcn_conv_pack_launch(const ConvArgs& a, int dtype, hipStream_t stream);
 bool wcn_conv_dense_takes(const ConvArgs& a, int dtype);
 int wcn_conv_dense_launch(const ConvArgs& a, int dtype, hipStream_t stream);
 
+// The contraction for maps with exactly one pair per output row (wcn_conv_single.hip): whether it
+// takes a problem's shape, and its launch over pair lists in any order (`host_offsets`: the K + 1
+// offsets; X, Wt, bias, residual, relu, out, the lists and the sizes are read from `a`).
+constexpr int WCN_SINGLE_MAX_OFFSETS = 64;
+struct WcnSingleTiles {  // tiles of 256 pairs of one offset, in offset order
+  int32_t first_tile[WCN_SINGLE_MAX_OFFSETS + 1];
+  int32_t first_pair[WCN_SINGLE_MAX_OFFSETS + 1];
+  int32_t total;
+};
+bool wcn_conv_single_takes(int dtype, int c_in, int c_out, int num_offsets);
+int wcn_conv_single_launch(const ConvArgs& a, int dtype, const int64_t* host_offsets, hipStream_t stream);
+
 #endif  // WCN_CONV_ARGS_H_
 
 // The contraction for narrow layers (wcn_conv_group.hip): a wave per group of 64 output rows.

@@ -45,6 +45,10 @@ class IntSearchResult:
         # group-start table, row count) or None until first needed.
         self._by_out = None
         self._by_in = None
+        # every output row occurs in exactly one pair (the map of a transposed convolution that
+        # undoes a strided one with kernel size = stride over duplicate-free voxels): the
+        # contraction then needs neither an order of the pairs nor sums
+        self._single_out = False
 
     @torch.no_grad()
     def __getitem__(self, idx: int) -> Tuple[Tensor, Tensor]:

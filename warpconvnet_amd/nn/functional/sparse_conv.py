@@ -226,6 +226,34 @@ def sparse_conv_forward(in_features: Tensor, weight: Tensor, kernel_map: IntSear
     out = torch.empty((num_out_coords, c_out), dtype=x.dtype, device=device)
     L = lib()
     in_maps, out_maps = km.in_maps, km.out_maps
+    if km._single_out and num_out_coords > 0 and x.shape[0] > 0 and x.dtype in (torch.float16, torch.bfloat16) \
+            and int(km.offsets[-1]) == num_out_coords \
+            and L.wcn_conv_single_supported(DTYPE_CODE[x.dtype], c_in, c_out, K):
+        # one pair per output row: nothing is summed, the lists are taken in the order they have
+        host_offsets = _host_offsets_of(km)
+        r = None
+        if residual is not None:
+            if tuple(residual.shape) != (num_out_coords, c_out):
+                raise ValueError(f"residual has shape {tuple(residual.shape)}, the output {(num_out_coords, c_out)}")
+            require_device(residual, "residual")
+            r = as_rows(residual)
+        code = DTYPE_CODE[x.dtype]
+        if keep_prepared_weight:
+            tiles = _prepared_weight(weight, make_w, x.dtype, c_in)
+            check(L.wcn_sparse_conv_fwd_single(ptr(x), x.shape[0], c_in, code, ptr(tiles), code, 1, K, c_out, ptr(b),
+                                               ptr(in_maps), ptr(out_maps), host_offsets, ptr(r), 1 if relu else 0,
+                                               ptr(out), num_out_coords, None, 0, stream_ptr(device)),
+                  "wcn_sparse_conv_fwd_single")
+        else:
+            w = make_w()
+            nbytes = L.wcn_conv_prepared_weight_bytes(K, c_in, c_out, code)
+            ws = workspace(nbytes, device)
+            check(L.wcn_sparse_conv_fwd_single(ptr(x), x.shape[0], c_in, code, ptr(w), DTYPE_CODE[w.dtype], 0, K, c_out,
+                                               ptr(b), ptr(in_maps), ptr(out_maps), host_offsets, ptr(r),
+                                               1 if relu else 0, ptr(out), num_out_coords, ptr(ws), nbytes,
+                                               stream_ptr(device)),
+                  "wcn_sparse_conv_fwd_single")
+        return out if out.dtype == in_features.dtype else out.to(in_features.dtype)
     group_start = None
     if not km._out_ascend and num_out_coords > 0:
         # a map whose out_maps does not ascend (transposed convolution, caller-made lists) is
@@ -465,6 +493,13 @@ def generate_output_coords_and_kernel_map(
         kernel_map._keys_unique = getattr(forward_map, "_keys_unique", False)
         kernel_map._from_builder = getattr(forward_map, "_from_builder", False)
         kernel_map._device_offsets = forward_map._device_offsets
+        # kernel as large as the stride, no dilation, a forward map of the builder's over fine voxels
+        # without repeats: every fine row has its one parent, at one offset
+        kernel_map._single_out = bool(
+            tuple(int(k) for k in kernel_size) == tuple(int(v) for v in stride)
+            and all(int(d) == 1 for d in kernel_dilation) and not generative
+            and kernel_map._from_builder and kernel_map._keys_unique
+            and int(forward_map.offsets[-1]) == out_coords.shape[0])
     else:
         kernel_map = generate_kernel_map(in_coords, out_coords, stride, kernel_size,
                                          kernel_dilation, method=method,
