@@ -108,6 +108,23 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert prepared(tile_bytes=16) == -6
     assert prepared(c=256, n=1500, tile_bytes=1 << 23) == -6   # this shape splits slices: partial sums need room
     assert prepared(residual=fake, out=fake) == -1   # the residual may not be the output buffer
+    # one pair per output row
+    assert L.wcn_conv_single_supported(1, 128, 96, 8) == 1 and L.wcn_conv_single_supported(2, 32, 8, 64) == 1
+    assert L.wcn_conv_single_supported(0, 128, 96, 8) == 0      # fp32 features
+    assert L.wcn_conv_single_supported(1, 40, 96, 8) == 0       # rows that are not whole 32-channel steps
+    assert L.wcn_conv_single_supported(1, 160, 96, 8) == 0      # no instance for five steps
+    assert L.wcn_conv_single_supported(1, 128, 260, 8) == 0 and L.wcn_conv_single_supported(1, 128, 96, 65) == 0
+    eight = (ctypes.c_int64 * 9)(0, 1, 2, 3, 4, 5, 6, 7, 10)
+
+    def single(num_out=10, offsets=eight, c_in=128, ws=fake, ws_bytes=1 << 20, prepared=0, residual=null, out=fake):
+        return L.wcn_sparse_conv_fwd_single(fake, 10, c_in, 1, fake, 1, prepared, 8, 96, null, fake, fake, offsets,
+                                            residual, 0, out, num_out, ws, ws_bytes, null)
+
+    assert single(num_out=11) == -1                  # as many pairs as output rows, or it is not this kind of map
+    assert single(c_in=40) == -1
+    assert single(ws_bytes=16) == -6                 # room for the weight tiles
+    assert single(offsets=None) == -1
+    assert single(residual=fake, out=fake) == -1
     assert conv(dtype=9) == -1
     assert conv(wdtype=2) == -1                      # f16 features with bf16 weights
     assert conv(ws_bytes=16) == -6                   # workspace too small
