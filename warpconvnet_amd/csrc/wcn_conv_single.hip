@@ -161,8 +161,9 @@ int launch_single(const ConvArgs& a, const WcnSingleTiles& tt, hipStream_t s) {
       allowed[device] = true;
     }
   }
-  // workgroups per CU: two where registers (up to 180 a lane for rows of up to 128 channels, 244 beyond) and LDS admit them
-  const int per_cu = std::max(1, std::min(KS <= 4 ? 2 : 1, (160 * 1024) / lds));
+  // workgroups per CU: what the registers admit (130 to 166 a lane for rows of up to 96 channels: three
+  // waves per SIMD; 180 for 128 channels: two; 214 and 244 beyond: one) and LDS holds
+  const int per_cu = std::max(1, std::min(KS <= 3 ? 3 : (KS <= 4 ? 2 : 1), (160 * 1024) / lds));
   const unsigned grid = (unsigned)std::min<int64_t>(tt.total, (int64_t)single_cus() * per_cu);
   hipLaunchKernelGGL((conv_fwd_single<T, KS>), dim3(grid), dim3(SINGLE_WAVES * 64), lds, s, a, tt);
   wcn_conv_note_kernel("conv_fwd_single<%s, %d>", wcn_type_text<T>(), KS);
