@@ -173,6 +173,7 @@ def cpu_baseline(bcoords, feats, weight):
 def secondary_configs(dev, steps, warmup):
     """The other single-layer configurations (parity-test cases; reported under config.other_configs
     with --all-configs, never as the headline value): cold map build + contraction per step."""
+    from warpconvnet_amd._lib import lib
     from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
     from warpconvnet_amd.geometry.coords.search.search_results import IntSearchResult
     from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
@@ -248,6 +249,17 @@ def secondary_configs(dev, steps, warmup):
     up_general._keys_unique, up_general._from_builder = km._keys_unique, True
     t_up_general, y_general = timed(lambda: sparse_conv_forward(y, wu, up_general, n))
     assert float((y_up.float() - y_general.float()).abs().max()) <= 2e-2 * float(y_general.float().abs().max())
+    # the same two paths over the same map for other channel counts (whole calls, warm map)
+    up_shapes = {}
+    for c_coarse, c_fine in ((32, 32), (64, 32), (256, 128)):
+        ys = torch.randn(m, c_coarse, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(dev)
+        ws = weights(8, c_coarse, c_fine, torch.bfloat16, 10)
+        t_single, _ = timed(lambda: sparse_conv_forward(ys, ws, up, n))
+        kernel_single = lib().wcn_conv_last_kernel().decode()
+        t_general, _ = timed(lambda: sparse_conv_forward(ys, ws, up_general, n))
+        up_shapes[f"{c_coarse}->{c_fine}"] = {"one_pair_per_row_call_ms": t_single, "kernel": kernel_single,
+                                              "general_path_call_ms": t_general,
+                                              "general_path_kernel": lib().wcn_conv_last_kernel().decode()}
     # consumers of the same maps: depthwise 3x3x3 over the 1M-voxel map, 2x2x2 stride-2 max pooling
     from warpconvnet_amd.nn.functional.sparse_conv_depth import spatially_sparse_depthwise_conv
     km3 = generate_kernel_map(c, c, (1, 1, 1), (3, 3, 3))
@@ -338,7 +350,8 @@ def secondary_configs(dev, steps, warmup):
     out["configs[2]: 2x2x2 s2 96->128 + transposed 128->96 bf16, 1M fine voxels"] = {
         "num_voxels": n, "num_coarse": m, "num_pairs": int(km.offsets[-1]),
         "coords_and_kernel_map_build_ms": t_map, "down_contraction_call_ms": t_down,
-        "up_contraction_call_ms": t_up, "up_contraction_call_general_path_ms": t_up_general, "voxels_per_s": n / ((t_map + t_down + t_up) * 1e-3)}
+        "up_contraction_call_ms": t_up, "up_contraction_call_general_path_ms": t_up_general,
+        "up_other_channel_counts_bf16": up_shapes, "voxels_per_s": n / ((t_map + t_down + t_up) * 1e-3)}
     return out
 
 
