@@ -303,10 +303,13 @@ int wcn_sparse_conv_fwd_prepared(const void* features, int64_t num_in, int32_t c
  *   out[out_maps[p], :] = act(bias + features[in_maps[p], :] @ W[k(p)] + residual[out_maps[p], :])
  *
  * wcn_conv_single_supported says whether a shape is taken (16-bit features, c_in of 32, 64, 96, 128,
- * 192 or 256, c_out a multiple of 8 up to 256, at most 64 offsets).  weight_is_prepared != 0: `weight`
- * is the block wcn_conv_prepare_weight made (no workspace needed); otherwise W (K, c_in, c_out) as
- * stored and a workspace of wcn_conv_prepared_weight_bytes bytes.  Replaces the same reference path as
- * wcn_sparse_conv_fwd (sparse_conv.py:495-544 over the map of sparse_conv.py:1916-1939). */
+ * 192 or 256, c_out a multiple of 8 up to 256, at most 64 offsets).  weight_is_prepared: 0 = W
+ * (K, c_in, c_out) as stored, 2 = W (K, c_out, c_in) (the product is then with W[k]^T: the input
+ * gradient of a strided convolution with kernel = stride over voxels without repeats is a map of this
+ * kind, dX[in_maps] = dY[out_maps] @ W[k]^T, sparse_conv.py:547-627), both with a workspace of
+ * wcn_conv_prepared_weight_bytes bytes; 1 = `weight` is the block wcn_conv_prepare_weight made (no
+ * workspace).  Replaces the same reference path as wcn_sparse_conv_fwd (sparse_conv.py:495-544 over
+ * the map of sparse_conv.py:1916-1939). */
 int wcn_conv_single_supported(int32_t dtype, int32_t c_in, int32_t c_out, int32_t num_offsets);
 
 int wcn_sparse_conv_fwd_single(const void* features, int64_t num_in, int32_t c_in, int32_t dtype,

@@ -100,16 +100,18 @@ def test_gradients_with_duplicate_voxels_use_the_general_path(oracle):
     assert rel_err(gx.cpu().numpy()[defined], want_x.numpy()[defined]) <= 1e-5
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_gradients_of_strided_and_transposed_pair(oracle, dtype):
+@pytest.mark.parametrize("dtype,c1,c2", [(torch.float32, 24, 40), (torch.bfloat16, 24, 40), (torch.bfloat16, 32, 64)],
+                         ids=["f32_24_40", "bf16_24_40", "bf16_32_64_one_pair_per_row"])
+def test_gradients_of_strided_and_transposed_pair(oracle, dtype, c1, c2):
     """2x2x2 stride-2 convolution followed by its transposed convolution back onto the fine
-    voxels: the gradient of the first exchanges an unsorted map (re-ordered by the library), the
-    gradient of the second a map whose input list ascends."""
+    voxels: the gradient of the first exchanges an unsorted map (re-ordered by the library, or, for
+    16-bit rows of whole 32-channel steps, taken as it is: every fine row is in one pair, so its
+    gradient is one product), the gradient of the second a map whose input list ascends."""
+    from warpconvnet_amd._lib import lib
     from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
     from oracle.explicit_conv import explicit_gemm_forward
     items = [synthetic.indoor_scene(seed=50 + b, n_target=6000, voxel_size=0.05) for b in range(2)]
     bc = synthetic.batch_indexed(items)
-    c1, c2 = 24, 40
     x = normal_features(len(bc), c1, seed=9, dtype=dtype)
     w_down = kaiming_weight(8, c1, c2, seed=10, dtype=dtype)
     w_up = kaiming_weight(8, c2, c1, seed=11, dtype=dtype)
@@ -121,6 +123,8 @@ def test_gradients_of_strided_and_transposed_pair(oracle, dtype):
     back = spatially_sparse_conv(coarse, wu, (2, 2, 2), stride=(2, 2, 2), transposed=True,
                                  output_spatially_sparse_tensor=fine)
     back.feature_tensor.backward(gy.to(DEV))
+    took_single = lib().wcn_conv_last_kernel().decode().startswith("conv_fwd_single<")
+    assert took_single == (c1 % 32 == 0 and dtype != torch.float32), lib().wcn_conv_last_kernel()
 
     # float64 chain on the CPU over the library's own coarse coordinates (their order is free)
     coarse_bc = coarse.batch_indexed_coordinates.cpu().numpy()

@@ -1682,7 +1682,8 @@ int wcn_sparse_conv_fwd_single(const void* features, int64_t num_in, int32_t c_i
       num_in <= 0 || num_out <= 0 || num_in >= (1ll << 31) || num_out >= (1ll << 31))
     return WCN_ERR_INVALID_ARGUMENT;
   if (residual_or_null && residual_or_null == out) return WCN_ERR_INVALID_ARGUMENT;
-  if (!weight_is_prepared && weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32) return WCN_ERR_INVALID_ARGUMENT;
+  if (weight_is_prepared < 0 || weight_is_prepared > 2) return WCN_ERR_INVALID_ARGUMENT;
+  if (weight_is_prepared != 1 && weight_dtype != dtype && weight_dtype != WCN_DTYPE_F32) return WCN_ERR_INVALID_ARGUMENT;
   const int64_t L = host_offsets[num_offsets];
   if (host_offsets[0] != 0 || L != num_out || !in_maps || !out_maps) return WCN_ERR_INVALID_ARGUMENT;  // one pair per output row
   for (int k = 0; k < num_offsets; ++k)
@@ -1709,14 +1710,15 @@ int wcn_sparse_conv_fwd_single(const void* features, int64_t num_in, int32_t c_i
   a.c_in_pad = round_up(c_in, ck_of(dtype));
   a.c_out_pad = round_up(c_out, TN);
   a.identity = -1;
-  if (weight_is_prepared) {
+  if (weight_is_prepared == 1) {
     a.Wt = weight;
   } else {
     const size_t need = wcn_conv_prepared_weight_bytes(num_offsets, c_in, c_out, dtype);
     if (!workspace || workspace_bytes < need) return WCN_ERR_WORKSPACE;
     a.Wt = workspace;
-    if (dtype == WCN_DTYPE_F16) launch_prep<_Float16>(a, weight, weight_dtype, dtype, 0, 0, nullptr, s);
-    else launch_prep<__bf16>(a, weight, weight_dtype, dtype, 0, 0, nullptr, s);
+    const int as_stored = weight_is_prepared == 2 ? 1 : 0;  // 2: W is (K, c_out, c_in): rows of the tiles already
+    if (dtype == WCN_DTYPE_F16) launch_prep<_Float16>(a, weight, weight_dtype, dtype, as_stored, 0, nullptr, s);
+    else launch_prep<__bf16>(a, weight, weight_dtype, dtype, as_stored, 0, nullptr, s);
   }
   if (g_time_start) (void)hipEventRecord(g_time_start, s);
   const int rc = wcn_conv_single_launch(a, dtype, host_offsets, s);

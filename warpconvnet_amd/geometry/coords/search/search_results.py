@@ -49,6 +49,9 @@ class IntSearchResult:
         # undoes a strided one with kernel size = stride over duplicate-free voxels): the
         # contraction then needs neither an order of the pairs nor sums
         self._single_out = False
+        # the same for the input rows (the forward map of such a strided convolution): its input
+        # gradient is a product of that kind
+        self._single_in = False
 
     @torch.no_grad()
     def __getitem__(self, idx: int) -> Tuple[Tensor, Tensor]:

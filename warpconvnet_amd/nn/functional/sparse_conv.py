@@ -352,7 +352,18 @@ def sparse_conv_backward(grad_output: Tensor, in_features: Tensor, weight: Tenso
             symmetric = 1 if (km._symmetric and km._out_ascend and n_in == n_out) else 0
             in_maps, out_maps = km.in_maps, km.out_maps
             group_start = None
-            if not symmetric and not km._in_ascend:
+            if km._single_in and num_pairs == n_in and dtype in (torch.float16, torch.bfloat16) \
+                    and L.wcn_conv_single_supported(code, c_out, c_in, K):
+                # every input row is in exactly one pair: dX[in] = dY[out] @ W[k]^T, nothing summed, the
+                # lists in the order they have
+                nbytes = L.wcn_conv_prepared_weight_bytes(K, c_out, c_in, code)
+                ws = workspace(nbytes, device)
+                grad_x = torch.empty((n_in, c_in), dtype=dtype, device=device)
+                check(L.wcn_sparse_conv_fwd_single(ptr(gy), n_out, c_out, code, ptr(w), DTYPE_CODE[w.dtype], 2, K,
+                                                   c_in, None, ptr(out_maps), ptr(in_maps), host_offsets, None, 0,
+                                                   ptr(grad_x), n_in, ptr(ws), nbytes, stream_ptr(device)),
+                      "wcn_sparse_conv_fwd_single")
+            elif not symmetric and not km._in_ascend:
                 # general map: the lists ascending in input row are made once per map object
                 out_maps, in_maps, groups = _pairs_sorted(km, "in", n_in)
                 group_start = ptr(groups)
@@ -361,14 +372,15 @@ def sparse_conv_backward(grad_output: Tensor, in_features: Tensor, weight: Tenso
                 if gs is not None and gs[2] == (K, n_in):
                     group_start = ctypes.c_void_p(gs[1])
             ascend = 1
-            ws = workspace(L.wcn_conv_workspace_bytes(n_in, K, c_out, c_in, code, num_pairs, ascend),
-                           device)
-            grad_x = torch.empty((n_in, c_in), dtype=dtype, device=device)
-            check(L.wcn_sparse_conv_dgrad(ptr(gy), n_out, c_out, code, ptr(w), DTYPE_CODE[w.dtype], K,
-                                          c_in, ptr(in_maps), ptr(out_maps), host_offsets, iden,
-                                          symmetric, 1, group_start,
-                                          ptr(grad_x), n_in, ptr(ws), ws.numel(), stream_ptr(device)),
-                  "wcn_sparse_conv_dgrad")
+            if grad_x is None:
+                ws = workspace(L.wcn_conv_workspace_bytes(n_in, K, c_out, c_in, code, num_pairs, ascend),
+                               device)
+                grad_x = torch.empty((n_in, c_in), dtype=dtype, device=device)
+                check(L.wcn_sparse_conv_dgrad(ptr(gy), n_out, c_out, code, ptr(w), DTYPE_CODE[w.dtype], K,
+                                              c_in, ptr(in_maps), ptr(out_maps), host_offsets, iden,
+                                              symmetric, 1, group_start,
+                                              ptr(grad_x), n_in, ptr(ws), ws.numel(), stream_ptr(device)),
+                      "wcn_sparse_conv_dgrad")
         grad_x = grad_x.to(in_features.dtype)
 
     if need_weight_grad:
@@ -504,6 +516,12 @@ def generate_output_coords_and_kernel_map(
         kernel_map = generate_kernel_map(in_coords, out_coords, stride, kernel_size,
                                          kernel_dilation, method=method,
                                          skip_symmetric_kernel_map=False)
+        # kernel as large as the stride over voxels without repeats: every input row is in one pair
+        kernel_map._single_in = bool(
+            tuple(int(k) for k in kernel_size) == tuple(int(v) for v in stride)
+            and any(int(v) != 1 for v in stride) and all(int(d) == 1 for d in kernel_dilation)
+            and not generative and getattr(kernel_map, "_keys_unique", False)
+            and int(kernel_map.offsets[-1]) == in_coords.shape[0])
 
     if input_sparse_tensor.cache is None:
         input_sparse_tensor._extra_attributes["_cache"] = IntSearchCache()
