@@ -357,6 +357,36 @@ def test_transposed_convolution_with_one_pair_per_output_row(oracle, name, dtype
         km._single_out = True
 
 
+def test_transposed_convolution_onto_voxels_without_a_parent_takes_the_general_path(oracle):
+    """An output tensor with voxels that no coarse voxel covers: fewer pairs than output rows, so the map
+    is not of the one-pair-per-row kind; those rows get the bias alone."""
+    from warpconvnet_amd._lib import lib
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    dtype = torch.bfloat16
+    items = [synthetic.random_cloud(61, 5000, 30)[:, 1:]]
+    fine = _voxels(items, normal_features(len(items[0]), 8, seed=3, dtype=dtype))
+    far = (items[0][:400] + np.array([64, 64, 64], dtype=items[0].dtype))  # a second cloud no coarse voxel covers
+    wider_items = [np.concatenate([items[0], far])]
+    wider = _voxels(wider_items, normal_features(len(wider_items[0]), 8, seed=4, dtype=dtype))
+    wd = kaiming_weight(8, 8, 64, seed=5, dtype=dtype).to(DEV)
+    wu = kaiming_weight(8, 64, 32, seed=6, dtype=dtype).to(DEV)
+    bias = (torch.randn(32, generator=torch.Generator().manual_seed(7)) * 0.1).to(dtype).to(DEV)
+    with torch.no_grad():
+        coarse = spatially_sparse_conv(fine, wd, 2, stride=2)
+        back = spatially_sparse_conv(coarse, wu, 2, stride=2, bias=bias, transposed=True,
+                                     output_spatially_sparse_tensor=wider)
+    assert not lib().wcn_conv_last_kernel().decode().startswith("conv_fwd_single<")
+    bc_w = synthetic.batch_indexed(wider_items)
+    coarse_bc = coarse.batch_indexed_coordinates.cpu().numpy()
+    im, om, off, _ = oracle.kernel_map(bc_w, coarse_bc, (2, 2, 2), (2, 2, 2))
+    assert int(off[-1]) == len(items[0]) < len(bc_w)
+    want = oracle.explicit_conv_f64(coarse.feature_tensor.double().cpu().numpy(), wu.double().cpu().numpy(),
+                                    om, im, off, None, len(bc_w)) + bias.double().cpu().numpy()
+    got = back.feature_tensor.float().cpu().numpy()
+    assert rel_err(got, want) <= TOL[dtype]
+    assert np.allclose(got[len(items[0]):], bias.float().cpu().numpy(), atol=1e-6)
+
+
 def test_pair_lists_are_reordered_once_and_kept_on_the_map(oracle):
     """The map of a transposed convolution does not ascend in output row: its re-ordered lists
     are made on the first product and the very same tensors serve the second one."""
