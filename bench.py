@@ -610,6 +610,23 @@ def main():
     finally:
         gc.enable()
     module_max_diff = float((mod_out.feature_tensor.float() - out.float()).abs().max())
+    # the same with the weight's tiles kept on the parameter (an option for weights that stay put:
+    # the call then enqueues the contraction alone); reported beside, never as the headline value
+    module.keep_prepared_weight = True
+    for _ in range(5):
+        module_step()
+    torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            kept_out = module_step()
+        torch.cuda.synchronize()
+        module_kept_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    finally:
+        gc.enable()
+    assert torch.equal(kept_out.feature_tensor, mod_out.feature_tensor)
     if os.environ.get("WCN_BENCH_TRACE"):  # per-step device times, for looking into an odd average
         for i in range(args.steps):
             print(f"step {i}: map {starts[i].elapsed_time(mids[i]):.3f} ms, contraction call "
@@ -653,6 +670,7 @@ def main():
             "contraction_call_ms": conv_call_ms,
             "contraction_kernel_ms": conv_kernel_ms,
             "module_forward_ms": module_ms,
+            "module_forward_kept_weight_tiles_ms": module_kept_ms,
             "module_forward_note": ("SparseConv3d.forward on a Voxels object made anew per step (cold table and "
                                     "map, cache lookups, output Voxels); wall clock / K; max |difference| to the "
                                     f"direct path's output: {module_max_diff:.3g}"),
