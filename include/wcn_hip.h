@@ -524,6 +524,16 @@ int wcn_voxel_rows(const float* points, int64_t num_points, const int64_t* host_
                    const int64_t* device_batch_offsets_or_null, int32_t batch_size, double voxel_size,
                    int32_t* rows, void* stream);
 
+/* wcn_batch_indexed_rows replaces `torch.cat([batch_index.unsqueeze(1), batched_coords], dim=1)`
+ * over `batch_index_from_offset(offsets)` (warpconvnet/geometry/coords/ops/batch_index.py:22-36 and
+ * :110-117): rows (n, dims + 1) int32 receives [b, coords[i][0..dims)] with b the batch item whose
+ * range [host_batch_offsets[b], host_batch_offsets[b + 1]) holds i.  The offsets (batch_size + 1
+ * values, the first 0, the last n, not descending) are read on the host and travel with the launch;
+ * batch_size is at most WCN_VOXEL_MAX_BATCH. */
+int wcn_batch_indexed_rows(const int32_t* coords, int64_t num_rows, int32_t dims,
+                           const int64_t* host_batch_offsets, int32_t batch_size, int32_t* rows,
+                           void* stream);
+
 size_t wcn_unique_rows_workspace_bytes(int64_t num_rows);
 
 int wcn_unique_rows_csr(const int32_t* rows, int64_t num_rows, int32_t columns, void* workspace,

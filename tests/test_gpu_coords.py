@@ -497,3 +497,22 @@ def test_strided_coordinates_with_negative_coordinates_and_repeated_rows(oracle,
         else:             # the oracle orders by batch item afterwards, as the reference does
             assert np.array_equal(sort_rows(got.cpu().numpy()), sort_rows(ref_out)), stride
             assert np.array_equal(got_off.numpy().astype(np.int64), ref_off)
+
+
+@pytest.mark.parametrize("dims", [1, 2, 3, 4])
+@pytest.mark.parametrize("counts", [(5,), (3, 0, 4, 0), (0, 0, 7), tuple(range(64)), tuple([2] * 65)],
+                         ids=["one_item", "empty_items", "leading_empty", "64_items", "65_items"])
+def test_batch_indexed_coordinates_against_the_formula(dims, counts):
+    """[batch item, coordinates] rows against the reference's formula, the batch column expanded
+    from the offsets with repeat_interleave (batch_index.py:22-36, 110-117); 65 batch items are
+    beyond what travels with the library's launch and take the torch path."""
+    from warpconvnet_amd.geometry.coords.ops.batch_index import batch_indexed_coordinates
+    g = torch.Generator().manual_seed(len(counts) * 10 + dims)
+    n = sum(counts)
+    coords = torch.randint(-50, 50, (n, dims), generator=g, dtype=torch.int32)
+    offsets = torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int64)
+    got = batch_indexed_coordinates(coords.cuda(), offsets)
+    batch = torch.arange(len(counts)).repeat_interleave(torch.tensor(counts))
+    want = torch.cat([batch.to(torch.int32).unsqueeze(1), coords], dim=1)
+    assert got.dtype == torch.int32 and got.shape == want.shape
+    assert torch.equal(got.cpu(), want)

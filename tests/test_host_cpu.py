@@ -389,7 +389,14 @@ def test_voxelisation_entry_points_reject_bad_arguments():
         assert L.wcn_voxel_rows(fake, 10, offsets, null, batch, size, fake, null) == -1
         assert L.wcn_voxelize_points_csr(fake, 10, offsets, null, batch, size, fake, 1 << 30, null, null, null,
                                          null, null, ctypes.byref(count), null) == -1
+    for offsets, rows, dims, batch in ((ok, 10, 0, 2), (ok, 9, 3, 2), (ok, 10, 3, 0), (None, 10, 3, 2),
+                                       ((ctypes.c_int64 * 3)(1, 4, 10), 10, 3, 2),
+                                       ((ctypes.c_int64 * 3)(0, 11, 10), 10, 3, 2), (ok, -1, 3, 2)):
+        assert L.wcn_batch_indexed_rows(fake, rows, dims, offsets, batch, fake, null) == -1
+    assert L.wcn_batch_indexed_rows(null, 10, 3, ok, 2, fake, null) == -1
+    assert L.wcn_batch_indexed_rows(null, 0, 3, (ctypes.c_int64 * 2)(0, 0), 1, null, null) == 0  # nothing to do
     many = (ctypes.c_int64 * 102)(*range(0, 102))  # 101 batch items: the offsets must also be on the device
+    assert L.wcn_batch_indexed_rows(fake, 101, 3, many, 101, fake, null) == -1  # more than travel with a launch
     assert L.wcn_voxel_rows(fake, 101, many, null, 101, 0.1, fake, null) == -1
     assert L.wcn_voxelize_points_csr(fake, 10, ok, null, 2, 0.1, fake, 64, null, null, null, null, null,
                                      ctypes.byref(count), null) == -6

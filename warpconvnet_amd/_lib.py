@@ -81,6 +81,7 @@ SIGNATURES = {
                                              _i32, _i32, _vp, _i32, _vp, _sz, _vp]),
     "wcn_probe_gather_rows": (ctypes.c_int, [_vp, _i64, _i32, _vp, _i64, _vp, _vp]),
     "wcn_voxel_rows": (ctypes.c_int, [_vp, _i64, _i64p, _vp, _i32, ctypes.c_double, _vp, _vp]),
+    "wcn_batch_indexed_rows": (ctypes.c_int, [_vp, _i64, _i32, _i64p, _i32, _vp, _vp]),
     "wcn_unique_rows_workspace_bytes": (_sz, [_i64]),
     "wcn_unique_rows_csr": (ctypes.c_int, [_vp, _i64, _i32, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _i64p, _vp]),
     "wcn_voxelize_points_csr": (ctypes.c_int, [_vp, _i64, _i64p, _vp, _i32, ctypes.c_double, _vp, _sz, _vp, _vp,

@@ -159,6 +159,28 @@ __global__ void __launch_bounds__(256) voxel_rows(PointRows src, int64_t n, int4
 }
 
 // ---- bounding box of the rows --------------------------------------------------------------------
+// The batch column put in front of integer coordinates: row i = [batch item of row i, c[i][0..dims)].
+// One thread per row; with three spatial columns the row goes out as one 16-byte store.
+__global__ void __launch_bounds__(256) batch_indexed_rows(const int32_t* __restrict__ coords, int64_t n,
+                                                          int dims, BatchStarts starts, int batch_size,
+                                                          int32_t* __restrict__ rows) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int lo = 0, hi = batch_size;  // the item lies in [lo, hi)
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (starts.start[mid] <= i) lo = mid; else hi = mid;
+  }
+  if (dims == 3) {
+    const int32_t* c = coords + 3 * i;
+    reinterpret_cast<int4*>(rows)[i] = make_int4(lo, c[0], c[1], c[2]);
+  } else {
+    int32_t* r = rows + i * (dims + 1);
+    r[0] = lo;
+    for (int d = 0; d < dims; ++d) r[d + 1] = coords[i * dims + d];
+  }
+}
+
 __global__ void unique_init(UniqueHeader* __restrict__ h) {
   const int t = threadIdx.x;
   if (t < 4) {
@@ -416,6 +438,27 @@ int wcn_voxel_rows(const float* points, int64_t num_points, const int64_t* host_
   if (!rows) return WCN_ERR_INVALID_ARGUMENT;
   hipLaunchKernelGGL(voxel_rows, dim3((unsigned)((num_points + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, src, num_points, (int4*)rows);
+  WCN_LAUNCH_CHECK();
+  return WCN_OK;
+}
+
+int wcn_batch_indexed_rows(const int32_t* coords, int64_t num_rows, int32_t dims,
+                           const int64_t* host_batch_offsets, int32_t batch_size, int32_t* rows,
+                           void* stream) {
+  if (num_rows < 0 || dims < 1 || batch_size < 1 || batch_size > WCN_VOXEL_MAX_BATCH ||
+      !host_batch_offsets)
+    return WCN_ERR_INVALID_ARGUMENT;
+  BatchStarts starts;
+  for (int b = 0; b <= batch_size; ++b) {
+    starts.start[b] = host_batch_offsets[b];
+    if (b > 0 && starts.start[b] < starts.start[b - 1]) return WCN_ERR_INVALID_ARGUMENT;
+  }
+  for (int b = batch_size + 1; b <= WCN_VOXEL_MAX_BATCH; ++b) starts.start[b] = num_rows;
+  if (starts.start[0] != 0 || starts.start[batch_size] != num_rows) return WCN_ERR_INVALID_ARGUMENT;
+  if (num_rows == 0) return WCN_OK;
+  if (!coords || !rows) return WCN_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(batch_indexed_rows, dim3((unsigned)((num_rows + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, coords, num_rows, (int)dims, starts, (int)batch_size, rows);
   WCN_LAUNCH_CHECK();
   return WCN_OK;
 }

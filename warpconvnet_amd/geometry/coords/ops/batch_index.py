@@ -1,6 +1,12 @@
 """Batch index / offsets conversions (reference: warpconvnet/geometry/coords/ops/batch_index.py)."""
+import ctypes
+
 import torch
 from torch import Tensor
+
+from ...._lib import check, lib, ptr, stream_ptr
+
+_BY_VALUE_BATCHES = 64  # batch items whose offsets travel with the launch (WCN_VOXEL_MAX_BATCH)
 
 
 @torch.no_grad()
@@ -19,6 +25,18 @@ def batch_indexed_coordinates(batched_coords: Tensor, offsets: Tensor) -> Tensor
     instead of being expanded on the host and copied."""
     if batched_coords.is_cuda:
         n = batched_coords.shape[0]
+        host = offsets.tolist()
+        batch = len(host) - 1
+        if (batched_coords.dtype == torch.int32 and batched_coords.ndim == 2 and n > 0
+                and 1 <= batch <= _BY_VALUE_BATCHES and host[0] == 0 and host[-1] == n):
+            # one launch of the library instead of arange + searchsorted + cast + cat
+            coords = batched_coords.contiguous()
+            dims = coords.shape[1]
+            rows = torch.empty((n, dims + 1), dtype=torch.int32, device=coords.device)
+            host_offsets = (ctypes.c_int64 * (batch + 1))(*[int(v) for v in host])
+            check(lib().wcn_batch_indexed_rows(ptr(coords), n, dims, host_offsets, batch, ptr(rows),
+                                               stream_ptr(coords.device)), "wcn_batch_indexed_rows")
+            return rows
         bounds = offsets[1:].to(dtype=torch.int64, device="cpu")
         staged = torch.empty(bounds.shape, dtype=torch.int64, pin_memory=True)
         staged.copy_(bounds)
