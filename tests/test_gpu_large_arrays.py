@@ -1,0 +1,167 @@
+"""Feature arrays of more than 2^31 elements (and more than 4 GiB): the sizes 288 GB of HBM invite.
+Row indices stay below 2^31, but `row * channels` and the byte offsets behind it do not, so every
+address in the kernels has to be formed in 64 bits.  The CPU oracle does not finish at these sizes:
+sampled output rows (the first, the last, and those either side of element 2^31) are checked against
+plain torch fp32 operations over the same map, the maps themselves against their invariants."""
+import pytest
+import torch
+
+from helpers import kaiming_weight
+from warpconvnet_amd._lib import lib
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _random_voxels(n, extent, seed):
+    """n distinct voxels of an extent^3 box in random order, four batch items of n / 4 rows."""
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    return _voxels_of_cells(torch.randperm(extent ** 3, generator=g, device=DEV)[:n], extent)
+
+
+def _scattered_voxels(n, gap, extent, seed):
+    """n distinct voxels, one in every run of `gap` cells of an extent^3 box, in random order: with
+    a large gap nearly every voxel is alone in its 4x4x4 block."""
+    assert n * gap <= extent ** 3
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    cells = torch.arange(n, device=DEV) * gap + torch.randint(0, gap, (n,), generator=g, device=DEV)
+    return _voxels_of_cells(cells[torch.randperm(n, generator=g, device=DEV)], extent)
+
+
+def _voxels_of_cells(cells, extent):
+    n = cells.numel()
+    rows = torch.empty((n, 4), dtype=torch.int32, device=DEV)
+    rows[:, 0] = (torch.arange(n, device=DEV) * 4 // n).to(torch.int32)
+    rows[:, 1] = (cells // (extent * extent)).to(torch.int32)
+    rows[:, 2] = (cells // extent % extent).to(torch.int32)
+    rows[:, 3] = (cells % extent).to(torch.int32)
+    return rows
+
+
+def _sample_rows(n, channels):
+    edge = (1 << 31) // channels  # the row that holds element 2^31
+    assert 256 < edge < n - 256
+    picks = torch.cat([torch.arange(0, 256), torch.arange(edge - 128, edge + 128), torch.arange(n - 256, n)])
+    return picks.to(DEV)
+
+
+def _sampled_scatter(src, w_of, km, from_rows, to_rows, picks, n_to, width):
+    """sum over pairs whose `to` row is in picks of src[from] @ w_of(k), in fp32, as (len(picks), width)."""
+    place = torch.full((n_to,), -1, dtype=torch.int64, device=DEV)
+    place[picks] = torch.arange(len(picks), device=DEV)
+    out = torch.zeros(len(picks), width, dtype=torch.float32, device=DEV)
+    for k in range(len(km)):
+        im, om = km[k]
+        f, t = (im, om) if from_rows == "in" else (om, im)
+        where = place[t.long()]
+        keep = where >= 0
+        if bool(keep.any()):
+            out.index_add_(0, where[keep], src[f[keep].long()].float() @ w_of(k))
+    return out
+
+
+def _check_map(km, n):
+    offs = km.offsets.cpu()
+    assert int(offs[-1]) == km.in_maps.numel() == km.out_maps.numel()
+    assert int(km.in_maps.min()) >= 0 and int(km.in_maps.max()) < n
+    assert int(km.out_maps.min()) >= 0 and int(km.out_maps.max()) < n
+    centre = len(km) // 2
+    im, om = km[centre]
+    assert im.numel() == n and torch.equal(im, om)  # every voxel meets itself once at the centre offset
+    for k in (0, len(km) - 1):
+        a, b = km[k]
+        assert bool((b[1:] > b[:-1]).all())           # output rows ascend inside an offset
+
+
+def _check_pair_count(km, n, extent):
+    """Voxels drawn uniformly from the box, a quarter of them per batch item: a voxel meets itself
+    and, in each of 26 directions, another voxel of its item with the item's density (a little less
+    at the faces of the box)."""
+    expected = n + 26 * n * (n / 4) / extent ** 3
+    assert 0.98 * expected < km.in_maps.numel() < 1.005 * expected
+
+
+def _close(got, want, tol=1e-2):
+    scale = float(want.abs().max())
+    return float((got.float() - want).abs().max()) <= tol * scale
+
+
+def test_wide_rows_beyond_two_to_the_31_elements():
+    """3x3x3, 256 -> 256, fp16, 8.5 M voxels: 2.18 G elements and 4.35 GB per feature array (the
+    output-stationary kernel for wide rows), with both gradients."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_backward, sparse_conv_forward
+    n, c = 8_500_000, 256
+    assert n * c > (1 << 31)
+    coords = _random_voxels(n, 400, seed=3)
+    km = generate_kernel_map(coords, coords, (1, 1, 1), (3, 3, 3))
+    _check_map(km, n)
+    _check_pair_count(km, n, 400)
+    g = torch.Generator(device=DEV).manual_seed(4)
+    x = torch.randn(n, c, generator=g, device=DEV, dtype=torch.float16)
+    w = kaiming_weight(27, c, c, seed=5, dtype=torch.float16).to(DEV)
+    picks = _sample_rows(n, c)
+    got = sparse_conv_forward(x, w, km, n)
+    assert lib().wcn_conv_last_kernel().decode().startswith("conv_fwd_dense<"), lib().wcn_conv_last_kernel()
+    want = _sampled_scatter(x, lambda k: w[k].float(), km, "in", "out", picks, n, c)
+    assert _close(got[picks], want)
+    gy = torch.randn(n, c, generator=g, device=DEV, dtype=torch.float16)
+    gx, gw = sparse_conv_backward(gy, x, w, km)
+    want = _sampled_scatter(gy, lambda k: w[k].float().t(), km, "out", "in", picks, n, c)
+    assert _close(gx[picks], want)
+    del want, gx
+    want = torch.stack([x[km[k][0].long()].float().t() @ gy[km[k][1].long()].float() for k in range(27)])
+    assert _close(gw, want)
+
+
+def test_one_slice_rows_beyond_two_to_the_31_elements():
+    """3x3x3, 64 -> 64, fp16, 34 M voxels: 2.18 G elements per feature array (the pair-packed
+    kernel of the headline configuration) over a map of some 150 M pairs."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    n, c = 34_000_000, 64
+    assert n * c > (1 << 31)
+    coords = _random_voxels(n, 640, seed=6)
+    km = generate_kernel_map(coords, coords, (1, 1, 1), (3, 3, 3))
+    _check_map(km, n)
+    g = torch.Generator(device=DEV).manual_seed(7)
+    x = torch.randn(n, c, generator=g, device=DEV, dtype=torch.float16)
+    w = kaiming_weight(27, c, c, seed=8, dtype=torch.float16).to(DEV)
+    picks = _sample_rows(n, c)
+    got = sparse_conv_forward(x, w, km, n)
+    assert lib().wcn_conv_last_kernel().decode().startswith("conv_fwd_pack<"), lib().wcn_conv_last_kernel()
+    want = _sampled_scatter(x, lambda k: w[k].float(), km, "in", "out", picks, n, c)
+    assert _close(got[picks], want)
+    _check_pair_count(km, n, 640)
+    eye = torch.zeros(27, c, c, dtype=torch.float16, device=DEV)
+    eye[13] = torch.eye(c, dtype=torch.float16, device=DEV)
+    assert torch.equal(sparse_conv_forward(x, eye, km, n), x)  # centre tap only: a copy of every row
+
+
+def test_table_of_scattered_voxels_with_many_bins():
+    """12 M voxels that are nearly all alone in their block: 12 M blocks, which the build sorts into
+    more bins than its small form has (an LDS counter per bin, a bin's blocks in an LDS table).
+    Every voxel is found again at its own row, absent neighbours are not found, and the map of the
+    set onto itself holds the centre pairs and little else."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.geometry.coords.search.torch_hashmap import TorchHashTable
+    n = 12_000_000
+    coords = _scattered_voxels(n, 500, 1900, seed=9)
+    table = TorchHashTable.from_keys(coords)
+    assert lib().wcn_table_default_capacity(n) // 2048 > 4096  # more bins than the small form takes
+    found = table.search(coords)
+    assert torch.equal(found.long(), torch.arange(n, device=DEV))
+    shifted = coords.clone()
+    shifted[:, 1] += 2000  # outside the box of the set
+    assert int((table.search(shifted) >= 0).sum()) == 0
+    km = generate_kernel_map(coords, coords, (1, 1, 1), (3, 3, 3))
+    _check_map(km, n)
+    pairs = km.in_maps.numel()
+    assert n <= pairs < n + n // 10
+    # every pair joins two voxels one step apart, in the direction of its offset
+    for k in (0, 5, 26):
+        im, om = km[k]
+        if im.numel():
+            d = coords[im.long()] - coords[om.long()]
+            want = torch.tensor([0, k // 9 - 1, k // 3 % 3 - 1, k % 3 - 1], dtype=torch.int32, device=DEV)
+            assert bool((d == want).all())

@@ -78,10 +78,11 @@ static inline size_t wcn_align256(size_t x) { return (x + 255) & ~(size_t)255; }
 // rebuild with more slots also re-deals the bins.
 #define WCN_BIN_SLOTS 2048      // distinct blocks a bin can hold (its table in LDS)
 #define WCN_PART_KEYS 4096      // keys per workgroup of the histogram and scatter passes
+#define WCN_MAX_BINS 32768      // a counter per bin in LDS during the build: 128 KB
 static inline int32_t wcn_table_bins(int64_t capacity) {
   int64_t b = capacity / 2048;
   if (b < 16) b = 16;
-  if (b > 4096) b = 4096;
+  if (b > WCN_MAX_BINS) b = WCN_MAX_BINS;
   return (int32_t)b;
 }
 static inline int32_t wcn_table_parts(int64_t n_keys) {

@@ -46,7 +46,10 @@ __device__ __forceinline__ PartRange part_range(int64_t n_keys) {
   return r;
 }
 
-constexpr int MAX_BINS = 4096;
+// Bins: capacity / 2048, at most WCN_MAX_BINS.  The histogram and scatter passes keep one counter
+// per bin in LDS (dynamic: 4 bytes per bin, 128 KB at the most), and a thread of the scatter pass
+// scans BINS_PER_THREAD bin totals: 4 up to 4096 bins, 32 beyond.
+constexpr int SMALL_BINS = 4096;
 
 // Keys per bin of one part of the keys, the part's bounding box; the part's share of the slots is
 // set to empty on the way (each slot is two 16-byte stores, {EMPTY, 0} and {0, 0, 0, 0}).
@@ -54,7 +57,7 @@ __global__ void __launch_bounds__(1024) table_hist(const int4* __restrict__ keys
                                                    int32_t bins, int32_t* __restrict__ hist,
                                                    int32_t* __restrict__ part_box,
                                                    WcnSlot* __restrict__ slots, int64_t capacity) {
-  __shared__ int s_cnt[MAX_BINS];
+  extern __shared__ int s_cnt[];  // [bins]
   __shared__ int s_mn[16][4];
   __shared__ int s_mx[16][4];
   const int tid = threadIdx.x, parts = gridDim.x, part = blockIdx.x;
@@ -139,8 +142,9 @@ __global__ void __launch_bounds__(256) table_colscan(int32_t* __restrict__ hist,
 }
 
 // Every key and its row to its place in its bin.  Each workgroup scans the bin totals into bin
-// starts for itself (at most MAX_BINS numbers); workgroup 0 also stores them for the next pass,
+// starts for itself (1024 x BPT numbers); workgroup 0 also stores them for the next pass,
 // merges the parts' bounding boxes and writes the header.
+template <int BPT>
 __global__ void __launch_bounds__(1024) table_scatter(const int4* __restrict__ keys, int64_t n_keys,
                                                       int32_t bins, const int32_t* __restrict__ hist,
                                                       const int32_t* __restrict__ bin_total,
@@ -150,7 +154,7 @@ __global__ void __launch_bounds__(1024) table_scatter(const int4* __restrict__ k
                                                       int64_t stats_offset,
                                                       int4* __restrict__ bin_coords,
                                                       int32_t* __restrict__ bin_row) {
-  __shared__ int s_cur[MAX_BINS];
+  extern __shared__ int s_cur[];  // [bins]
   __shared__ int s_wave[16];
   const int tid = threadIdx.x, lane = wcn_lane(), wave = tid >> 6;
   const int parts = gridDim.x, part = blockIdx.x;
@@ -162,10 +166,10 @@ __global__ void __launch_bounds__(1024) table_scatter(const int4* __restrict__ k
     const int64_t i = r.lo + tid + t * 1024;
     c[t] = i < r.hi ? keys[i] : make_int4(0, 0, 0, 0);
   }
-  int v[4], mine[4], sum = 0;
+  int v[BPT], mine[BPT], sum = 0;
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int b = tid * 4 + t;
+  for (int t = 0; t < BPT; ++t) {
+    const int b = tid * BPT + t;
     v[t] = b < bins ? bin_total[b] : 0;
     mine[t] = b < bins ? hist[(int64_t)b * parts + part] : 0;
     sum += v[t];
@@ -176,8 +180,8 @@ __global__ void __launch_bounds__(1024) table_scatter(const int4* __restrict__ k
   int run = incl - sum;
   for (int w = 0; w < wave; ++w) run += s_wave[w];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int b = tid * 4 + t;
+  for (int t = 0; t < BPT; ++t) {
+    const int b = tid * BPT + t;
     if (b < bins) {
       s_cur[b] = run + mine[t];
       if (part == 0) bin_start[b] = run;
@@ -557,18 +561,14 @@ int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView
                          bool want_slot_of, hipStream_t s) {
   const uint32_t cap_mask = (uint32_t)(v.capacity - 1);
   const int4* k4 = (const int4*)keys;
-  hipLaunchKernelGGL(table_hist, dim3(v.parts), dim3(1024), 0, s, k4, n_keys, v.bins, v.hist,
-                     v.part_box, v.slots, v.capacity);
-  hipLaunchKernelGGL(table_colscan, dim3((v.bins + 3) / 4), dim3(256), 0, s, v.hist, v.bins,
-                     v.parts, v.bin_total);
-  hipLaunchKernelGGL(table_scatter, dim3(v.parts), dim3(1024), 0, s, k4, n_keys, v.bins, v.hist,
-                     v.bin_total, v.bin_start, v.part_box, v.hdr,
-                     (int64_t)((const char*)v.bin_stats - (const char*)v.hdr), (int4*)v.bin_coords,
-                     v.bin_row);
+  if (v.bins < 1 || v.bins > WCN_MAX_BINS || (v.bins & (v.bins - 1))) return WCN_ERR_INVALID_ARGUMENT;
+  const bool many_bins = v.bins > SMALL_BINS;
+  const size_t counters = sizeof(int) * (size_t)v.bins;
+  auto scatter = many_bins ? table_scatter<WCN_MAX_BINS / 1024> : table_scatter<SMALL_BINS / 1024>;
   auto fn = want_slot_of ? table_bins<true> : table_bins<false>;
-  {  // the kernel's LDS exceeds the default limit: lift it once per device and instance
+  {  // LDS beyond the default limit: lifted once per device and kernel
     static std::mutex mu;
-    static bool allowed[2][64] = {};
+    static bool allowed[4][64] = {};
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return WCN_ERR_LAUNCH;
     std::lock_guard<std::mutex> hold(mu);
@@ -578,7 +578,24 @@ int wcn_table_build_impl(const int32_t* keys, int64_t n_keys, const WcnTableView
         return WCN_ERR_LAUNCH;
       allowed[want_slot_of][device] = true;
     }
+    if (many_bins && !allowed[2][device]) {
+      const int most = (int)(sizeof(int) * WCN_MAX_BINS);
+      if (hipFuncSetAttribute((const void*)table_hist, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              most) != hipSuccess ||
+          hipFuncSetAttribute((const void*)scatter, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              most) != hipSuccess)
+        return WCN_ERR_LAUNCH;
+      allowed[2][device] = true;
+    }
   }
+  hipLaunchKernelGGL(table_hist, dim3(v.parts), dim3(1024), counters, s, k4, n_keys, v.bins, v.hist,
+                     v.part_box, v.slots, v.capacity);
+  hipLaunchKernelGGL(table_colscan, dim3((v.bins + 3) / 4), dim3(256), 0, s, v.hist, v.bins,
+                     v.parts, v.bin_total);
+  hipLaunchKernelGGL(scatter, dim3(v.parts), dim3(1024), counters, s, k4, n_keys, v.bins, v.hist,
+                     v.bin_total, v.bin_start, v.part_box, v.hdr,
+                     (int64_t)((const char*)v.bin_stats - (const char*)v.hdr), (int4*)v.bin_coords,
+                     v.bin_row);
   hipLaunchKernelGGL(fn, dim3(v.bins), dim3(1024), sizeof(BinLds), s, v.hdr, v.slots, cap_mask,
                      v.bin_start, (const int4*)v.bin_coords, v.bin_row, v.order_tag, v.order_row,
                      v.block_list, v.perm, v.slot_of, v.bin_stats);
