@@ -39,10 +39,11 @@ def _voxels_of_cells(cells, extent):
 
 
 def _sample_rows(n, channels):
-    edge = (1 << 31) // channels  # the row that holds element 2^31
-    assert 256 < edge < n - 256
-    picks = torch.cat([torch.arange(0, 256), torch.arange(edge - 128, edge + 128), torch.arange(n - 256, n)])
-    return picks.to(DEV)
+    edge = (1 << 31) // channels  # the row that holds element 2^31, where the array is that long
+    parts = [torch.arange(0, 256), torch.arange(n - 256, n)]
+    if 512 < edge < n - 512:
+        parts.insert(1, torch.arange(edge - 128, edge + 128))
+    return torch.cat(parts).to(DEV)
 
 
 def _sampled_scatter(src, w_of, km, from_rows, to_rows, picks, n_to, width):
@@ -75,9 +76,9 @@ def _check_map(km, n):
 
 def _check_pair_count(km, n, extent):
     """Voxels drawn uniformly from the box, a quarter of them per batch item: a voxel meets itself
-    and, in each of 26 directions, another voxel of its item with the item's density (a little less
-    at the faces of the box)."""
-    expected = n + 26 * n * (n / 4) / extent ** 3
+    and, in each of the other directions, another voxel of its item with the item's density (a
+    little less at the faces of the box)."""
+    expected = n + (len(km) - 1) * n * (n / 4) / extent ** 3
     assert 0.98 * expected < km.in_maps.numel() < 1.005 * expected
 
 
@@ -165,3 +166,108 @@ def test_table_of_scattered_voxels_with_many_bins():
             d = coords[im.long()] - coords[om.long()]
             want = torch.tensor([0, k // 9 - 1, k // 3 % 3 - 1, k % 3 - 1], dtype=torch.int32, device=DEV)
             assert bool((d == want).all())
+
+
+def test_down_and_up_sampling_beyond_two_to_the_31_elements():
+    """2x2x2 stride 2, 64 -> 128, and its transposed 128 -> 64 back onto the fine voxels, fp16, 34 M
+    fine voxels: the coarse array (some 30 M rows of 128) and the fine ones are beyond 2^31
+    elements; the up-sampling takes the kernel for maps with one pair per output row."""
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    from warpconvnet_amd.nn.functional.sparse_conv import spatially_sparse_conv
+    n = 34_000_000
+    rows = _random_voxels(n, 640, seed=10)
+    g = torch.Generator(device=DEV).manual_seed(11)
+    x = torch.randn(n, 64, generator=g, device=DEV, dtype=torch.float16)
+    offsets = torch.tensor([0, n // 4, n // 2, 3 * n // 4, n])
+    fine = Voxels(rows[:, 1:].contiguous(), x, offsets=offsets)
+    wd = kaiming_weight(8, 64, 128, seed=12, dtype=torch.float16).to(DEV)
+    wu = kaiming_weight(8, 128, 64, seed=13, dtype=torch.float16).to(DEV)
+    coarse = spatially_sparse_conv(fine, wd, 2, stride=2)
+    m = len(coarse)
+    assert m * 128 > (1 << 31)
+    km = next(iter(fine.cache.values()))
+    assert int(km.offsets[-1]) == n
+    assert torch.equal(torch.sort(km.in_maps).values, torch.arange(n, dtype=torch.int32, device=DEV))
+    assert int(km.out_maps.max()) == m - 1
+    picks = _sample_rows(m, 128)
+    want = _sampled_scatter(x, lambda k: wd[k].float(), km, "in", "out", picks, m, 128)
+    assert _close(coarse.feature_tensor[picks], want)
+    back = spatially_sparse_conv(coarse, wu, 2, stride=2, transposed=True, output_spatially_sparse_tensor=fine)
+    assert lib().wcn_conv_last_kernel().decode().startswith("conv_fwd_single<"), lib().wcn_conv_last_kernel()
+    picks = _sample_rows(n, 64)
+    want = _sampled_scatter(coarse.feature_tensor, lambda k: wu[k].float(), km, "out", "in", picks, n, 64)
+    assert _close(back.feature_tensor[picks], want)
+
+
+def test_map_of_125_offsets_over_20_million_voxels():
+    """5x5x5 over 20 M voxels: offsets x voxels = 2.5 G entries of parked rows (10 GB), 16 -> 16 fp16
+    over the map's 99 M pairs (the kernel for narrow rows takes up to 2^24 input rows; beyond that
+    the pair-packed kernel runs)."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    n = 20_000_000
+    assert 125 * n > (1 << 31)
+    coords = _random_voxels(n, 540, seed=14)
+    km = generate_kernel_map(coords, coords, (1, 1, 1), (5, 5, 5))
+    assert len(km) == 125 and km.identity_map_index == 62
+    _check_map(km, n)
+    _check_pair_count(km, n, 540)
+    counts = torch.diff(km.offsets)
+    assert torch.equal(counts, counts.flip(0))
+    for k in (0, 57, 124):  # every pair joins two voxels of one item, apart by its offset
+        im, om = km[k]
+        d = coords[im.long()] - coords[om.long()]
+        want = torch.tensor([0, k // 25 - 2, k // 5 % 5 - 2, k % 5 - 2], dtype=torch.int32, device=DEV)
+        assert im.numel() > 0 and bool((d == want).all())
+    g = torch.Generator(device=DEV).manual_seed(15)
+    x = torch.randn(n, 16, generator=g, device=DEV, dtype=torch.float16)
+    w = kaiming_weight(125, 16, 16, seed=16, dtype=torch.float16).to(DEV)
+    got = sparse_conv_forward(x, w, km, n)
+    assert lib().wcn_conv_last_kernel().decode().startswith("conv_fwd_pack<"), lib().wcn_conv_last_kernel()
+    picks = _sample_rows(n, 16)
+    want = _sampled_scatter(x, lambda k: w[k].float(), km, "in", "out", picks, n, 16)
+    assert _close(got[picks], want)
+
+
+def test_pooling_and_depthwise_beyond_two_to_the_31_elements():
+    """34 M voxels x 64 channels fp16 through the depthwise 3x3x3 convolution (centre tap: a copy;
+    all taps one: the neighbours' sum on sampled rows) and through 2x2x2 stride-2 pooling (the sum of
+    ones counts every fine voxel once, the mean of ones is one, the maximum on sampled coarse rows)."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    from warpconvnet_amd.nn.functional.sparse_conv_depth import spatially_sparse_depthwise_conv
+    from warpconvnet_amd.nn.functional.sparse_pool import sparse_reduce
+    n, c = 34_000_000, 64
+    rows = _random_voxels(n, 640, seed=17)
+    g = torch.Generator(device=DEV).manual_seed(18)
+    x = torch.randn(n, c, generator=g, device=DEV, dtype=torch.float16)
+    km = generate_kernel_map(rows, rows, (1, 1, 1), (3, 3, 3))
+    w = torch.zeros(27, c, dtype=torch.float16, device=DEV)
+    w[13] = 1
+    assert torch.equal(spatially_sparse_depthwise_conv(x, w, km, n), x)
+    w[:] = 1
+    got = spatially_sparse_depthwise_conv(x, w, km, n)
+    picks = _sample_rows(n, c)
+    eye = torch.eye(c, dtype=torch.float32, device=DEV)
+    want = _sampled_scatter(x, lambda k: eye, km, "in", "out", picks, n, c)
+    assert _close(got[picks], want)
+    del got, km
+
+    offsets = torch.tensor([0, n // 4, n // 2, 3 * n // 4, n])
+    fine = Voxels(rows[:, 1:].contiguous(), x, offsets=offsets)
+    top = sparse_reduce(fine, 2, 2, "max")
+    m = len(top)
+    pool_map = next(iter(fine.cache.values()))
+    assert int(pool_map.offsets[-1]) == n and int(pool_map.out_maps.max()) == m - 1
+    picks = _sample_rows(m, c)
+    place = torch.full((m,), -1, dtype=torch.int64, device=DEV)
+    place[picks] = torch.arange(len(picks), device=DEV)
+    where = place[pool_map.out_maps.long()]
+    keep = where >= 0
+    want = torch.full((len(picks), c), float("-inf"), device=DEV)
+    want.scatter_reduce_(0, where[keep][:, None].expand(-1, c), x[pool_map.in_maps[keep].long()].float(), "amax")
+    assert torch.equal(top.feature_tensor[picks].float(), want)
+    ones = fine.replace(batched_features=torch.ones_like(x))
+    counts = sparse_reduce(ones, 2, 2, "sum").feature_tensor
+    assert int(counts[:, 0].double().sum()) == n and float(counts.max()) <= 8 and float(counts.min()) >= 1
+    assert bool((sparse_reduce(ones, 2, 2, "mean").feature_tensor == 1).all())
