@@ -3,6 +3,8 @@ Row indices stay below 2^31, but `row * channels` and the byte offsets behind it
 address in the kernels has to be formed in 64 bits.  The CPU oracle does not finish at these sizes:
 sampled output rows (the first, the last, and those either side of element 2^31) are checked against
 plain torch fp32 operations over the same map, the maps themselves against their invariants."""
+import math
+
 import pytest
 import torch
 
@@ -271,3 +273,44 @@ def test_pooling_and_depthwise_beyond_two_to_the_31_elements():
     counts = sparse_reduce(ones, 2, 2, "sum").feature_tensor
     assert int(counts[:, 0].double().sum()) == n and float(counts.max()) <= 8 and float(counts.min()) >= 1
     assert bool((sparse_reduce(ones, 2, 2, "mean").feature_tensor == 1).all())
+
+
+def test_points_to_voxels_of_120_million_points():
+    """120 M points (4 items) -> some 104 M voxels of 2 cm, and the per-voxel sums of 32 fp32 features
+    per point (3.84 G elements): sorted distinct voxels, the grouping a permutation of the points,
+    every point in the group of its own cell, exact sums of small integers."""
+    from warpconvnet_amd.geometry.coords.ops.voxel import voxel_downsample_csr_mapping
+    from warpconvnet_amd.ops.reductions import segment_reduction
+    from warpconvnet_amd.utils.gather import take_rows
+    g = torch.Generator(device=DEV).manual_seed(19)
+    n, c = 120_000_000, 32
+    assert n * c > (1 << 31)
+    pts = torch.rand((n, 3), device=DEV, generator=g) * torch.tensor([20.0, 20.0, 2.0], device=DEV)
+    offsets = torch.tensor([0, n // 4, n // 2, 3 * n // 4, n])
+    unique, voffsets, csr_indices, csr_offsets, tu = voxel_downsample_csr_mapping(pts, offsets, 0.02)
+    m = len(unique)
+    expected = 4 * 1e8 * (1 - math.exp(-(n / 4) / 1e8))  # occupied cells of 10^8 per item, uniform points
+    assert 0.995 * expected < m < 1.005 * expected
+    assert unique.shape[1] == 4 and int(voffsets[-1]) == m and int(csr_offsets[-1]) == n
+    key = ((unique[:, 0].long() * 1024 + unique[:, 1].long()) * 1024 + unique[:, 2].long()) * 1024 + unique[:, 3].long()
+    assert bool((key[1:] > key[:-1]).all())  # strictly ascending: sorted and distinct
+    del key
+    assert torch.equal(torch.sort(csr_indices).values, torch.arange(n, device=DEV))  # a permutation
+    cells = torch.floor(pts / 0.02).int()
+    # rows are picked with the package's take_rows: `unique[index]` itself returns wrong rows for the
+    # last 2^26 of more than 2^26 indices into 16-byte rows with this PyTorch build
+    assert torch.equal(tu.to_original(unique)[:, 1:], cells)
+    by_column = torch.stack([unique[:, j].contiguous()[tu.to_orig_indices] for j in range(4)], dim=1)
+    assert torch.equal(take_rows(unique, tu.to_orig_indices), by_column)
+    del by_column
+    assert torch.equal(take_rows(cells, tu.to_unique_indices), unique[:, 1:])
+    del cells
+    counts = csr_offsets.diff()
+    assert int(counts.min()) >= 1
+    marks = ((torch.arange(n, device=DEV).view(-1, 1) + torch.arange(c, device=DEV).view(1, -1)) % 3).float()
+    per_voxel = segment_reduction(marks, csr_offsets, "sum", indices=csr_indices)
+    assert per_voxel.shape == (m, c)
+    for col in (0, c - 1):  # integers, exact in fp32 per voxel and in fp64 over all of them
+        assert float(per_voxel[:, col].double().sum()) == float(marks[:, col].double().sum())
+    last = csr_indices[int(csr_offsets[m - 1]):]   # the last voxel's points: beyond element 2^31 of `marks`
+    assert torch.equal(per_voxel[m - 1], marks[last].sum(dim=0))

@@ -450,3 +450,19 @@ def test_points_reductions_and_unique_host_logic():
     info = UniqueInfo(None, torch.tensor([2, 0, 3, 1, 4]), torch.tensor([0, 2, 3, 5]), None)
     assert info.to_orig_indices.tolist() == [0, 2, 0, 1, 2]
     assert info.to_orig_indices is info.to_orig_indices
+
+
+def test_take_rows_in_pieces_equals_plain_indexing(monkeypatch):
+    from warpconvnet_amd.utils import gather
+    g = torch.Generator().manual_seed(0)
+    src = torch.randn(50, 4, generator=g, requires_grad=True)
+    index = torch.randint(0, 50, (1000,), generator=g)
+    whole = gather.take_rows(src, index)
+    monkeypatch.setattr(gather, "_PIECE", 64)
+    pieces = gather.take_rows(src, index)
+    assert torch.equal(pieces, src[index]) and torch.equal(pieces, whole)
+    pieces.sum().backward()  # the gradient counts how often every row was picked
+    assert torch.equal(src.grad[:, 0], torch.bincount(index, minlength=50).float())
+    mask = torch.arange(50) % 2 == 0
+    assert torch.equal(gather.take_rows(src, mask), src[mask])
+    assert torch.equal(gather.take_rows(src[:, 0], index), src[:, 0][index])

@@ -7,6 +7,7 @@ from torch import Tensor
 
 from ..search.torch_discrete import kernel_offsets_from_size
 from .stride import unique_floor_div_rows
+from ....utils.gather import take_rows
 
 
 @torch.no_grad()
@@ -34,7 +35,7 @@ def expand_coords(batch_indexed_coords: Tensor, kernel_size: Tuple[int, ...],
     out, count, _ = unique_floor_div_rows(rows.contiguous(), (1,) * (rows.shape[1] - 1))
     unique = out[:count, : rows.shape[1]]
     order = torch.sort(unique[:, 0], stable=True).indices
-    unique = unique[order].contiguous()
+    unique = take_rows(unique, order).contiguous()
     counts = torch.bincount(unique[:, 0]).cpu()
     out_offsets = torch.cat([torch.zeros(1, dtype=torch.int32), counts.cumsum(dim=0)], dim=0)
     return unique, out_offsets

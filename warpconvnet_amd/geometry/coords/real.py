@@ -2,6 +2,7 @@
 Neighbour search and sorting of points are not part of this package."""
 from ..base.coords import Coords
 from .ops.voxel import voxel_downsample_random_indices
+from ...utils.gather import take_rows
 
 
 class RealCoords(Coords):
@@ -13,4 +14,4 @@ class RealCoords(Coords):
         assert self.device.type != "cpu", "Voxel downsample is only supported on GPU"
         perm, down_offsets = voxel_downsample_random_indices(self.batched_tensor, self.offsets,
                                                              voxel_size=voxel_size)
-        return self.__class__(self.batched_tensor[perm], offsets=down_offsets)
+        return self.__class__(take_rows(self.batched_tensor, perm), offsets=down_offsets)

@@ -15,6 +15,7 @@ from ...geometry.coords.ops.voxel import (voxel_downsample_csr_mapping,
 from ...geometry.coords.real import RealCoords
 from ...geometry.coords.search.search_results import RealSearchResult
 from ...ops.reductions import REDUCTIONS, segment_reduction
+from ...utils.gather import take_rows
 
 __all__ = ["point_pool"]
 
@@ -25,12 +26,12 @@ def _pool_by_random_sample(pc, downsample_voxel_size: Optional[float], return_ty
     from ...geometry.types.voxels import Voxels
     keep, unique_offsets = voxel_downsample_random_indices(pc.coordinate_tensor, pc.offsets,
                                                            voxel_size=downsample_voxel_size)
-    feats = pc.features[keep]
+    feats = take_rows(pc.features, keep)
     if return_type == "voxel":
-        coords = IntCoords(torch.floor(pc.coordinate_tensor[keep] / downsample_voxel_size).int(),
+        coords = IntCoords(torch.floor(take_rows(pc.coordinate_tensor, keep) / downsample_voxel_size).int(),
                            offsets=unique_offsets)
         return Voxels(coords, feats, voxel_size=downsample_voxel_size)
-    coords = RealCoords(pc.coordinate_tensor[keep], offsets=unique_offsets)
+    coords = RealCoords(take_rows(pc.coordinate_tensor, keep), offsets=unique_offsets)
     return Points(coords, feats, voxel_size=downsample_voxel_size)
 
 
@@ -78,7 +79,7 @@ def point_pool(pc, reduction: Union[REDUCTIONS, str], downsample_max_num_points:
             xyz = segment_reduction(pc.coordinate_tensor, csr_offsets, REDUCTIONS.MEAN,
                                     indices=csr_indices, segment_of=lambda: to_unique.to_orig_indices)
         else:
-            xyz = pc.coordinate_tensor[to_unique.to_unique_indices]
+            xyz = take_rows(pc.coordinate_tensor, to_unique.to_unique_indices)
         out = Points(RealCoords(xyz, offsets=unique_offsets), down_features,
                      voxel_size=downsample_voxel_size)
     if return_to_unique:

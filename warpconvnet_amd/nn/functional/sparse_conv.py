@@ -34,6 +34,7 @@ from ...geometry.coords.search.search_results import IntSearchResult
 from ...geometry.coords.search.torch_discrete import generate_kernel_map
 from ...geometry.types.voxels import Voxels
 from ...utils.ntuple import ntuple
+from ...utils.gather import take_rows
 
 
 class STRIDED_CONV_MODE(enum.Enum):
@@ -472,7 +473,7 @@ def generate_output_coords_and_kernel_map(
     if not _is_random_order(order):
         code = encode(out_coords[:, 1:].contiguous(), batch_offsets=out_offsets, order=order,
                       return_perm=True)
-        out_coords = out_coords[code.perm].contiguous()
+        out_coords = take_rows(out_coords, code.perm).contiguous()
 
     def make_key(is_transposed, in_off, out_off):
         return IntSearchCacheKey(kernel_size=kernel_size, kernel_dilation=kernel_dilation,

@@ -23,6 +23,7 @@ from ...geometry.coords.search.torch_discrete import generate_kernel_map
 from ...geometry.types.voxels import Voxels
 from ...ops.reductions import REDUCTIONS
 from ...utils.ntuple import ntuple
+from ...utils.gather import take_rows
 
 _MODE = {REDUCTIONS.SUM: 0, REDUCTIONS.MEAN: 1, REDUCTIONS.MAX: 2, REDUCTIONS.MIN: 3}
 
@@ -157,7 +158,7 @@ def sparse_unpool(pooled_voxels: Voxels, unpooled_voxels: Voxels, kernel_size, s
     assert kernel_map is not None
     unpooled_maps, pooled_maps = kernel_map.in_maps, kernel_map.out_maps
     perm = torch.argsort(unpooled_maps)
-    rep_feats = pooled_voxels.feature_tensor[pooled_maps[perm].long()]
+    rep_feats = take_rows(pooled_voxels.feature_tensor, pooled_maps[perm].long())
     if concat_unpooled_voxels:
         rep_feats = torch.cat([unpooled_voxels.feature_tensor, rep_feats], dim=-1)
     return unpooled_voxels.replace(batched_features=rep_feats)

@@ -9,6 +9,7 @@ from torch import Tensor
 from torch.autograd import Function
 
 from .._lib import DTYPE_CODE, check, lib, ptr, require_device, stream_ptr
+from ..utils.gather import take_rows
 
 
 class REDUCTIONS(enum.Enum):
@@ -100,7 +101,7 @@ def segment_reduction(features: Tensor, offsets: Tensor, reduction, indices: Opt
         num_per_row = offsets.diff()
         pick = (torch.rand(len(num_per_row), device=features.device) * num_per_row).floor().long()
         entry = pick + offsets[:-1]
-        return features[indices[entry] if indices is not None else entry]
+        return take_rows(features, indices[entry] if indices is not None else entry)
     raise NotImplementedError(f"reduction {reduction.value!r} is not built")
 
 

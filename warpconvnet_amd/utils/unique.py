@@ -11,6 +11,7 @@ import torch
 from torch import Tensor
 
 from .._lib import check, lib, ptr, require_device, stream_ptr, workspace
+from .gather import take_rows
 
 
 def _run_unique(call, n: int, columns: int, dev, want_inverse: bool, want_representatives: bool):
@@ -163,7 +164,7 @@ class ToUnique:
         return unique, self.unique_info.to_csr_indices, self.unique_info.to_csr_offsets
 
     def to_original(self, unique: Tensor) -> Tensor:
-        return unique[self.unique_info.to_orig_indices]
+        return take_rows(unique, self.unique_info.to_orig_indices)
 
     @property
     def to_unique_indices(self) -> Tensor:
