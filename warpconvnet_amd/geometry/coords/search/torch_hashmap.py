@@ -105,9 +105,9 @@ class TorchHashTable:
     def _grow(self) -> None:
         """Rebuild with four times the slots (after the device reported an overflow).  More slots
         shorten the probe chains and, up to 2^26 slots, mean more bins during the build; beyond
-        that and eight slots per key neither changes and the overflow is final."""
+        that and four slots per key neither changes and the overflow is final."""
         n = self._keys4.shape[0]
-        if self._slots >= (1 << 30) or (self._slots >= (1 << 26) and self._slots >= 8 * n):
+        if self._slots >= (1 << 30) or (self._slots >= (1 << 26) and self._slots >= 4 * n):
             raise WcnError(ERR_TABLE_OVERFLOW, "wcn_table_build")
         self._build(self._slots * 4)
 
