@@ -486,6 +486,8 @@ def main():
     ap.add_argument("--sorted-voxels", action="store_true",
                     help="also time the same step on the voxels sorted along a Morton curve, and the sort "
                          "(config.morton_sorted)")
+    ap.add_argument("--sizes", action="store_true",
+                    help="also time the same layer on 16 and 64 scenes (4 M and 16 M voxels)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -763,6 +765,36 @@ def main():
             "kernel_map_build_ms": float(np.median(maps[10:])),
             "contraction_kernel_ms": float(np.median(kernels[10:])),
             "unsorted_kernel_map_build_ms": map_ms, "unsorted_contraction_kernel_ms": conv_kernel_ms}
+
+    if args.sizes:
+        larger = {}
+        for batch in (16, 64):
+            bc, _, f, _ = make_workload(batch=batch, seed=1)
+            big_coords = torch.as_tensor(bc, device=dev)
+            big_feats = f.to(dev)
+            m = len(bc)
+            maps, kernels = [], []
+            for _ in range(12):
+                cold = big_coords.view(-1, 4)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                k0.record(); k1.record()
+                e0.record()
+                km_b = generate_kernel_map(cold, cold, (1, 1, 1), (3, 3, 3))
+                e1.record()
+                L.wcn_conv_set_timing_events(ctypes.c_void_p(k0.cuda_event), ctypes.c_void_p(k1.cuda_event))
+                sparse_conv_forward(big_feats, weight_d, km_b, m)
+                torch.cuda.synchronize()
+                maps.append(e0.elapsed_time(e1))
+                kernels.append(k0.elapsed_time(k1))
+            map_b, conv_b = float(np.median(maps[4:])), float(np.median(kernels[4:]))
+            larger[f"{batch} scenes"] = {
+                "num_voxels": m, "num_pairs": int(km_b.offsets[-1]),
+                "kernel_map_build_ms": map_b, "contraction_kernel_ms": conv_b,
+                "voxels_per_s_map_plus_kernel": m / ((map_b + conv_b) * 1e-3),
+                "kernel": L.wcn_conv_last_kernel().decode()}
+            del big_coords, big_feats, km_b
+        result["config"]["larger_batches"] = larger
 
     if args.backward:
         from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_backward
