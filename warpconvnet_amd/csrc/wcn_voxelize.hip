@@ -164,12 +164,17 @@ __global__ void __launch_bounds__(256) voxel_rows(PointRows src, int64_t n, int4
 __global__ void __launch_bounds__(256) batch_indexed_rows(const int32_t* __restrict__ coords, int64_t n,
                                                           int dims, BatchStarts starts, int batch_size,
                                                           int32_t* __restrict__ rows) {
+  // the offsets arrive with the launch (scalar registers); lanes search them at different places,
+  // so they are put into LDS first
+  __shared__ int64_t s_start[WCN_VOXEL_MAX_BATCH + 1];
+  if (threadIdx.x <= WCN_VOXEL_MAX_BATCH) s_start[threadIdx.x] = starts.start[threadIdx.x];
+  __syncthreads();
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   int lo = 0, hi = batch_size;  // the item lies in [lo, hi)
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
-    if (starts.start[mid] <= i) lo = mid; else hi = mid;
+    if (s_start[mid] <= i) lo = mid; else hi = mid;
   }
   if (dims == 3) {
     const int32_t* c = coords + 3 * i;
