@@ -58,6 +58,9 @@ def _pad_kernel_args(values: Sequence[int], fill: int):
     return values + [fill] * (3 - len(values))
 
 
+# a map builder's workspace up to this size stays with its map (see _kernel_map_from_table)
+_KEEP_WORKSPACE_BYTES = 256 << 20
+
 # pairs per output row of the last map built for (kernel size, stride, size class of the row count):
 # sizes the buffers the pairs are emitted into before their number is known
 _PAIRS_PER_ROW = {}
@@ -123,15 +126,19 @@ def _kernel_map_from_table(table: TorchHashTable, out_coords: Tensor, kernel_siz
                                            stream_ptr(device)), "wcn_kmap_count_dilated")
         fill(assumed, in_buf, out_buf)
         # By-product the contraction reuses: the per-64-row group starts of every offset, (K, G + 1)
-        # int32, final once the count call's kernels have run.  Only this table is kept with the
-        # map (a copy of about K * M / 16 bytes; the workspace, whose probe results are K * M * 4
-        # bytes, goes back to the allocator).  The copy is enqueued here, before the wait for the
-        # result, so that nothing stands between that wait and what the caller launches next.
-        # The workspace begins with the map's K + 1 offsets as int64, which the scan leaves there for
-        # the fill pass: they ride along in the same copy, for contractions that take their offsets
-        # from device memory (wcn_sparse_conv_fwd_prepared).
+        # int32, final once the count call's kernels have run.  The workspace begins with the map's
+        # K + 1 offsets as int64, which the scan leaves there for the fill pass, and the group starts
+        # follow: this head (about K * M / 16 bytes) is what stays with the map, for the kernels
+        # that walk the map by groups and for contractions that take their offsets from device
+        # memory (wcn_sparse_conv_fwd_prepared).  The probe results behind it are K * M * 4 bytes:
+        # where that is more than _KEEP_WORKSPACE_BYTES the head is copied and the workspace goes
+        # back to the allocator; below, the map keeps the workspace as it is and the step has no
+        # copy in it.  The copy is enqueued here, before the wait for the result, so that nothing
+        # stands between that wait and what the caller launches next.
         begin = L.wcn_kmap_group_start(ptr(ws), M, K) - ws.data_ptr()
-        kept = ws[:begin + 4 * K * ((M + 63) // 64 + 1)].clone()
+        kept = ws[:begin + 4 * K * ((M + 63) // 64 + 1)]
+        if ws.numel() > _KEEP_WORKSPACE_BYTES:
+            kept = kept.clone()
         groups = kept[begin:]
         status = L.wcn_kmap_read_result(ptr(ws), M, K, host_offsets, stream_ptr(device))
         if status == ERR_TABLE_OVERFLOW:
