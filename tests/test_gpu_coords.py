@@ -516,3 +516,47 @@ def test_batch_indexed_coordinates_against_the_formula(dims, counts):
     want = torch.cat([batch.to(torch.int32).unsqueeze(1), coords], dim=1)
     assert got.dtype == torch.int32 and got.shape == want.shape
     assert torch.equal(got.cpu(), want)
+
+
+def test_steps_from_several_host_threads_on_their_own_streams():
+    """The library's state between its calls (the mailbox the pair counts arrive in, the pending
+    result, the table flags) is per thread: four threads, each on a stream of its own, build maps of
+    different scenes and run the contraction over them at the same time, and every thread gets what
+    the main thread got for its scene, bit for bit."""
+    import threading
+    from helpers import kaiming_weight
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    w = kaiming_weight(27, 64, 64, seed=3, dtype=torch.float16).to(DEV)
+    scenes = []
+    for t in range(4):
+        bc = synthetic.batch_indexed([synthetic.indoor_scene(40 + t, 60_000 + 7_000 * t, 0.02)])
+        c = torch.as_tensor(bc, device=DEV)
+        x = torch.randn(len(bc), 64, generator=torch.Generator().manual_seed(t)).half().to(DEV)
+        km = generate_kernel_map(c, c, (1, 1, 1), (3, 3, 3))
+        scenes.append((c, x, km.in_maps.clone(), km.out_maps.clone(), km.offsets.clone(),
+                       sparse_conv_forward(x, w, km, len(bc))))
+    torch.cuda.synchronize()
+    failures = []
+
+    def work(t):
+        c, x, want_in, want_out, want_offsets, want = scenes[t]
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                for _ in range(15):
+                    cold = c.view(-1, 4)  # a new tensor object: table and map are built again
+                    km = generate_kernel_map(cold, cold, (1, 1, 1), (3, 3, 3))
+                    out = sparse_conv_forward(x, w, km, c.shape[0])
+                    if not (torch.equal(km.offsets, want_offsets) and torch.equal(km.in_maps, want_in)
+                            and torch.equal(km.out_maps, want_out) and torch.equal(out, want)):
+                        failures.append(t)
+        except Exception as e:  # a thread's exception would otherwise be lost
+            failures.append((t, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    torch.cuda.synchronize()
+    assert failures == []
