@@ -639,6 +639,8 @@ def main():
             for _ in range(count):
                 _, o, _ = step(probes=False)
             outs.append(o)
+            stream.synchronize()
+        L.wcn_thread_release()  # this thread's pinned mailbox and events
 
     concurrent = {}
     for threads in (2, 4):

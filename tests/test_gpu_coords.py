@@ -525,6 +525,7 @@ def test_steps_from_several_host_threads_on_their_own_streams():
     the main thread got for its scene, bit for bit."""
     import threading
     from helpers import kaiming_weight
+    from warpconvnet_amd._lib import lib
     from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
     from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
     w = kaiming_weight(27, 64, 64, seed=3, dtype=torch.float16).to(DEV)
@@ -552,6 +553,8 @@ def test_steps_from_several_host_threads_on_their_own_streams():
                         failures.append(t)
         except Exception as e:  # a thread's exception would otherwise be lost
             failures.append((t, repr(e)))
+        torch.cuda.synchronize()
+        lib().wcn_thread_release()  # the thread's pinned mailbox and events
 
     threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
     for th in threads:
