@@ -1,0 +1,85 @@
+"""Seeded random sweep over what the fixed cases pin one at a time: batch sizes, voxel counts from one
+to twelve thousand per item (tiny, just below / at / above a 64-row group), sparse to nearly full
+boxes, coordinates far from the origin and negative, kernel sizes 1 to 5 per axis, strides 1 to 3 per
+axis, channel counts on and off the kernels' tile widths, the three element types.  Every case:
+strided coordinates and kernel map bit for bit against the C oracle, features (with a bias, a
+residual and a ReLU in the epilogue now and then) against its double-precision gather-GEMM-scatter
+within the tolerances of test_gpu_conv.py."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import kaiming_weight, normal_features, rel_err, sort_rows
+from warpconvnet_amd.utils import synthetic
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {torch.float32: 1e-5, torch.float16: 1e-2, torch.bfloat16: 1e-2}
+COUNTS = (1, 7, 63, 64, 65, 500, 3000, 12000)
+EXTENTS = (4, 12, 30, 80)
+SHIFTS = (0, -17, 1000, -(1 << 20))
+CHANNELS = (1, 3, 8, 13, 16, 24, 32, 40, 64, 96, 128, 160)
+DTYPES = (torch.float16, torch.bfloat16, torch.float32)
+
+
+def _case(seed):
+    rng = np.random.default_rng(1000 + seed)
+    batch = int(rng.integers(1, 5))
+    extent = int(rng.choice(EXTENTS))
+    items = []
+    for _ in range(batch):
+        n = min(int(rng.choice(COUNTS)), extent ** 3)
+        cells = rng.choice(extent ** 3, size=n, replace=False)
+        c = np.stack([cells // (extent * extent), cells // extent % extent, cells % extent], axis=1)
+        items.append((c + rng.choice(SHIFTS, size=3)).astype(np.int32))
+    ksize = tuple(int(k) for k in rng.integers(1, 6, size=3))
+    stride = (1, 1, 1) if rng.random() < 0.5 else tuple(int(s) for s in rng.integers(1, 4, size=3))
+    c_in, c_out = int(rng.choice(CHANNELS)), int(rng.choice(CHANNELS))
+    dtype = DTYPES[int(rng.integers(0, 3))]
+    epilogue = (rng.random() < 0.5, rng.random() < 0.3, rng.random() < 0.3)  # bias, residual, ReLU
+    return synthetic.batch_indexed(items), batch, ksize, stride, c_in, c_out, dtype, epilogue
+
+
+@pytest.mark.parametrize("seed", range(160))
+def test_random_case_against_the_oracle(oracle, seed):
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    in_coords, batch, ksize, stride, c_in, c_out, dtype, (with_bias, with_residual, relu) = _case(seed)
+    print(f"seed {seed}: {len(in_coords)} voxels in {batch} items, kernel {ksize}, stride {stride}, "
+          f"{c_in} -> {c_out} {dtype}, bias {with_bias}, residual {with_residual}, relu {relu}", flush=True)
+    dev_in = torch.as_tensor(in_coords, device=DEV)
+    if any(s != 1 for s in stride):
+        out_dev, off_dev = stride_coords(dev_in, stride)
+        out_coords = out_dev.cpu().numpy()
+        ref_out, _, ref_off = oracle.stride_coords(in_coords, stride, batch)
+        assert np.array_equal(out_coords, ref_out)
+        assert np.array_equal(off_dev.numpy().astype(np.int64), ref_off)
+    else:
+        out_coords = in_coords
+    km = generate_kernel_map(dev_in, torch.as_tensor(out_coords, device=DEV), stride, ksize)
+    im, om, off, iden = oracle.kernel_map(in_coords, out_coords, ksize, stride)
+    assert km.identity_map_index == iden
+    assert np.array_equal(km.offsets.numpy().astype(np.int64), off)
+    assert np.array_equal(km.in_maps.cpu().numpy(), im)
+    assert np.array_equal(km.out_maps.cpu().numpy(), om)
+    K = ksize[0] * ksize[1] * ksize[2]
+    x = normal_features(len(in_coords), c_in, seed=seed, dtype=dtype)
+    w = kaiming_weight(K, c_in, c_out, seed=seed + 1, dtype=dtype)
+    bias = normal_features(1, c_out, seed=seed + 2, dtype=dtype)[0] if with_bias else None
+    residual = normal_features(len(out_coords), c_out, seed=seed + 3, dtype=dtype) if with_residual else None
+    got = sparse_conv_forward(x.to(DEV), w.to(DEV), km, len(out_coords),
+                              bias=None if bias is None else bias.to(DEV),
+                              residual=None if residual is None else residual.to(DEV), relu=relu)
+    want = oracle.explicit_conv_f64(x.double().numpy(), w.double().numpy(), im, om, off, iden, len(out_coords))
+    if bias is not None:
+        want = want + bias.double().numpy()
+    if residual is not None:
+        want = want + residual.double().numpy()
+    if relu:
+        want = np.maximum(want, 0.0)
+    assert got.shape == want.shape and got.dtype == dtype
+    if np.abs(want).max() > 0:
+        assert rel_err(got.float().cpu().numpy(), want) <= TOL[dtype]
+    else:
+        assert not bool(got.any())
