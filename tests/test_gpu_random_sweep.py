@@ -4,7 +4,7 @@ boxes, coordinates far from the origin and negative, kernel sizes 1 to 5 per axi
 axis, channel counts on and off the kernels' tile widths, the three element types.  Every case:
 strided coordinates and kernel map bit for bit against the C oracle, features (with a bias, a
 residual and a ReLU in the epilogue now and then) against its double-precision gather-GEMM-scatter
-within the tolerances of test_gpu_conv.py."""
+within the tolerances of test_gpu_conv.py; a second sweep does the same for the two gradients."""
 import numpy as np
 import pytest
 import torch
@@ -83,3 +83,38 @@ def test_random_case_against_the_oracle(oracle, seed):
         assert rel_err(got.float().cpu().numpy(), want) <= TOL[dtype]
     else:
         assert not bool(got.any())
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_case_gradients_against_the_oracle(oracle, seed):
+    """Both gradients of the contraction over the same random cases (strided maps included, whose
+    exchanged lists have to be re-ordered for the input gradient), against the torch-CPU restatement
+    of the reference's explicit backward in float64."""
+    from oracle.explicit_conv import explicit_gemm_backward
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_backward
+    in_coords, batch, ksize, stride, c_in, c_out, dtype, _ = _case(500 + seed)
+    print(f"seed {seed}: {len(in_coords)} voxels in {batch} items, kernel {ksize}, stride {stride}, "
+          f"{c_in} -> {c_out} {dtype}", flush=True)
+    dev_in = torch.as_tensor(in_coords, device=DEV)
+    if any(s != 1 for s in stride):
+        out_coords = stride_coords(dev_in, stride)[0].cpu().numpy()
+    else:
+        out_coords = in_coords
+    km = generate_kernel_map(dev_in, torch.as_tensor(out_coords, device=DEV), stride, ksize)
+    im, om, off, iden = oracle.kernel_map(in_coords, out_coords, ksize, stride)
+    assert np.array_equal(km.in_maps.cpu().numpy(), im) and np.array_equal(km.out_maps.cpu().numpy(), om)
+    K = ksize[0] * ksize[1] * ksize[2]
+    x = normal_features(len(in_coords), c_in, seed=seed, dtype=dtype)
+    w = kaiming_weight(K, c_in, c_out, seed=seed + 1, dtype=dtype)
+    gy = normal_features(len(out_coords), c_out, seed=seed + 2, dtype=dtype)
+    gx, gw = sparse_conv_backward(gy.to(DEV), x.to(DEV), w.to(DEV), km)
+    want_x, want_w = explicit_gemm_backward(gy.double(), x.double(), w.double(), torch.as_tensor(im),
+                                            torch.as_tensor(om), off, iden)
+    assert gx.dtype == dtype and gw.dtype == dtype
+    for got, want in ((gx, want_x), (gw, want_w)):
+        if float(want.abs().max()) > 0:
+            assert rel_err(got.float().cpu().numpy(), want.numpy()) <= TOL[dtype]
+        else:
+            assert not bool(got.any())
