@@ -4,7 +4,8 @@ boxes, coordinates far from the origin and negative, kernel sizes 1 to 5 per axi
 axis, channel counts on and off the kernels' tile widths, the three element types.  Every case:
 strided coordinates and kernel map bit for bit against the C oracle, features (with a bias, a
 residual and a ReLU in the epilogue now and then) against its double-precision gather-GEMM-scatter
-within the tolerances of test_gpu_conv.py; a second sweep does the same for the two gradients."""
+within the tolerances of test_gpu_conv.py; a second sweep does the same for the two gradients, a
+third for the pooling reductions and the depthwise convolution over the maps."""
 import numpy as np
 import pytest
 import torch
@@ -118,3 +119,58 @@ def test_random_case_gradients_against_the_oracle(oracle, seed):
             assert rel_err(got.float().cpu().numpy(), want.numpy()) <= TOL[dtype]
         else:
             assert not bool(got.any())
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_case_pooling_and_depthwise_against_the_oracle(oracle, seed):
+    """The consumers of a kernel map over the same random cases: the four pooling reductions against
+    the torch restatement of the reference's sparse_reduce (selections exact, sums within the
+    tolerance), the depthwise convolution and its two gradients against the float64 restatement of
+    the reference's explicit depthwise path."""
+    from oracle.explicit_conv import explicit_depthwise_forward
+    from oracle.pool import pool_over_map
+    from warpconvnet_amd.geometry.coords.ops.stride import stride_coords
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.geometry.types.voxels import Voxels
+    from warpconvnet_amd.nn.functional.sparse_conv_depth import spatially_sparse_depthwise_conv
+    from warpconvnet_amd.nn.functional.sparse_pool import sparse_reduce
+    in_coords, batch, ksize, stride, channels, _, dtype, _ = _case(900 + seed)
+    print(f"seed {seed}: {len(in_coords)} voxels in {batch} items, kernel {ksize}, stride {stride}, "
+          f"{channels} channels {dtype}", flush=True)
+    n = len(in_coords)
+    x = normal_features(n, channels, seed=seed, dtype=dtype)
+    # pooling through the public functional (it strides the coordinates and builds the map itself)
+    counts = np.bincount(in_coords[:, 0], minlength=batch)
+    offsets = torch.as_tensor(np.concatenate([[0], np.cumsum(counts)]))
+    voxels = Voxels(torch.as_tensor(in_coords[:, 1:].copy(), device=DEV), x.to(DEV), offsets=offsets)
+    for reduction in ("max", "min", "mean", "sum"):
+        out = sparse_reduce(voxels, ksize, stride, reduction)
+        out_bc = out.batch_indexed_coordinates.cpu().numpy()
+        im, om, off, _ = oracle.kernel_map(in_coords, out_bc, ksize, stride)
+        want = pool_over_map(x.double(), torch.as_tensor(im), torch.as_tensor(om), len(out_bc), reduction)
+        got = out.feature_tensor.double().cpu()
+        if reduction in ("max", "min"):
+            assert torch.equal(got, want)
+        else:
+            assert rel_err(got.numpy(), want.numpy()) <= TOL[dtype]
+    # depthwise convolution over the map of the same geometry
+    dev_in = torch.as_tensor(in_coords, device=DEV)
+    out_coords = stride_coords(dev_in, stride)[0].cpu().numpy() if any(s != 1 for s in stride) else in_coords
+    km = generate_kernel_map(dev_in, torch.as_tensor(out_coords, device=DEV), stride, ksize)
+    im, om, off, iden = oracle.kernel_map(in_coords, out_coords, ksize, stride)
+    K = ksize[0] * ksize[1] * ksize[2]
+    w = (torch.randn(K, channels, generator=torch.Generator().manual_seed(seed)) * (1.0 / K) ** 0.5).to(dtype)
+    xd, wd = x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    got = spatially_sparse_depthwise_conv(xd, wd, km, len(out_coords))
+    x64, w64 = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    want = explicit_depthwise_forward(x64, w64, torch.as_tensor(im), torch.as_tensor(om), off, iden,
+                                      len(out_coords))
+    assert got.dtype == dtype
+    if float(want.detach().abs().max()) > 0:
+        assert rel_err(got.detach().double().cpu().numpy(), want.detach().numpy()) <= TOL[dtype]
+        gy = normal_features(len(out_coords), channels, seed=seed + 5, dtype=dtype)
+        got.backward(gy.to(DEV))
+        want_gx, want_gw = torch.autograd.grad(want, (x64, w64), gy.double())
+        for g, wg in ((xd.grad, want_gx), (wd.grad, want_gw)):
+            if float(wg.abs().max()) > 0:
+                assert rel_err(g.double().cpu().numpy(), wg.numpy()) <= TOL[dtype]
