@@ -5,7 +5,8 @@ axis, channel counts on and off the kernels' tile widths, the three element type
 strided coordinates and kernel map bit for bit against the C oracle, features (with a bias, a
 residual and a ReLU in the epilogue now and then) against its double-precision gather-GEMM-scatter
 within the tolerances of test_gpu_conv.py; a second sweep does the same for the two gradients, a
-third for the pooling reductions and the depthwise convolution over the maps."""
+third for the pooling reductions and the depthwise convolution over the maps, a fourth for maps
+over one to five spatial dimensions with dilated kernels against a dictionary look-up."""
 import numpy as np
 import pytest
 import torch
@@ -174,3 +175,59 @@ def test_random_case_pooling_and_depthwise_against_the_oracle(oracle, seed):
         for g, wg in ((xd.grad, want_gx), (wd.grad, want_gw)):
             if float(wg.abs().max()) > 0:
                 assert rel_err(g.double().cpu().numpy(), wg.numpy()) <= TOL[dtype]
+
+
+def _brute_force_map(in_rows, out_rows, stride, ksize, dilation):
+    """Kernel map over any number of columns by dictionary look-up: offsets enumerated with the last
+    dimension fastest and centred as the reference centres them (odd sizes about the middle, even
+    sizes from zero), pairs of an offset in ascending output row."""
+    import itertools
+    D = len(ksize)
+    where = {tuple(r): i for i, r in enumerate(in_rows.tolist())}
+    centres = [(k - 1) // 2 if k % 2 == 1 else 0 for k in ksize]
+    ins, outs, offsets = [], [], [0]
+    for idx in itertools.product(*[range(k) for k in ksize]):
+        off = [(i - c) * d for i, c, d in zip(idx, centres, dilation)]
+        for m, r in enumerate(out_rows.tolist()):
+            hit = where.get((r[0],) + tuple(r[1 + d] * stride[d] + off[d] for d in range(D)))
+            if hit is not None:
+                ins.append(hit)
+                outs.append(m)
+        offsets.append(len(ins))
+    return np.array(ins, np.int32), np.array(outs, np.int32), np.array(offsets, np.int64)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_case_dimensions_and_dilation_against_brute_force(seed):
+    """One to five spatial dimensions, dilated kernels, strides: the map against a dictionary
+    look-up over all columns (the C oracle restates the three-dimensional probe only)."""
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    rng = np.random.default_rng(7000 + seed)
+    D = int(rng.integers(1, 6))
+    extent = int(rng.choice((3, 6, 10, 16)))
+    n = int(rng.choice((1, 5, 64, 65, 400, 1500)))
+    rows = rng.integers(-extent // 2, extent // 2 + 1, size=(n, D + 1)).astype(np.int32)
+    rows[:, 0] = rng.integers(0, 3, size=n)
+    rows = np.unique(rows, axis=0)
+    rng.shuffle(rows)
+    top = 5 if D <= 3 else 3
+    ksize = tuple(int(k) for k in rng.integers(1, top + 1, size=D))
+    dilated = rng.random() < 0.5
+    dilation = tuple(int(d) for d in rng.integers(1, 4, size=D)) if dilated else (1,) * D
+    stride = tuple(int(s) for s in rng.integers(1, 3, size=D)) if rng.random() < 0.4 else (1,) * D
+    print(f"seed {seed}: {len(rows)} rows, {D} dimensions, kernel {ksize}, stride {stride}, dilation {dilation}",
+          flush=True)
+    if any(s != 1 for s in stride):
+        coarse = rows.copy()
+        coarse[:, 1:] = np.floor_divide(rows[:, 1:], np.array(stride, dtype=np.int32))
+        out_rows = np.unique(coarse, axis=0)
+    else:
+        out_rows = rows
+    dev = lambda a: torch.as_tensor(np.ascontiguousarray(a), device=DEV)
+    km = generate_kernel_map(dev(rows), dev(out_rows), stride, ksize,
+                             kernel_dilation=dilation if dilated else None,
+                             method="offset" if dilated else "size")
+    want_in, want_out, want_off = _brute_force_map(rows, out_rows, stride, ksize, dilation)
+    assert np.array_equal(km.offsets.numpy().astype(np.int64), want_off)
+    assert np.array_equal(km.in_maps.cpu().numpy(), want_in)
+    assert np.array_equal(km.out_maps.cpu().numpy(), want_out)
