@@ -6,7 +6,8 @@ strided coordinates and kernel map bit for bit against the C oracle, features (w
 residual and a ReLU in the epilogue now and then) against its double-precision gather-GEMM-scatter
 within the tolerances of test_gpu_conv.py; a second sweep does the same for the two gradients, a
 third for the pooling reductions and the depthwise convolution over the maps, a fourth for maps
-over one to five spatial dimensions with dilated kernels against a dictionary look-up."""
+over one to five spatial dimensions with dilated kernels against a dictionary look-up, a fifth for
+points -> voxels against the restatement of the reference's voxelisation."""
 import numpy as np
 import pytest
 import torch
@@ -231,3 +232,38 @@ def test_random_case_dimensions_and_dilation_against_brute_force(seed):
     assert np.array_equal(km.offsets.numpy().astype(np.int64), want_off)
     assert np.array_equal(km.in_maps.cpu().numpy(), want_in)
     assert np.array_equal(km.out_maps.cpu().numpy(), want_out)
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_case_points_to_voxels_against_the_oracle(seed):
+    """Points -> voxels over random batches (ragged and empty items, clouds far from the origin and
+    below zero, voxel sizes from millimetres to metres, 1 to 70 feature channels, every reduction the
+    front-end builds): coordinates and offsets bit for bit, selections exact, sums within 1e-5."""
+    from oracle import voxelize
+    from warpconvnet_amd.geometry.types.points import Points
+    rng = np.random.default_rng(9000 + seed)
+    batch = int(rng.integers(1, 6))
+    counts = [int(rng.choice((0, 1, 2, 63, 65, 1000, 20000))) for _ in range(batch)]
+    if sum(counts) == 0:
+        counts[0] = 5
+    span = float(rng.choice((0.05, 1.0, 30.0)))
+    centre = rng.choice((0.0, -50.0, 1000.0), size=3)
+    pts = ((rng.random((sum(counts), 3)) - 0.5) * span + centre).astype(np.float32)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    voxel_size = float(rng.choice((0.002, 0.02, 0.1, 0.75)))
+    channels = int(rng.choice((1, 3, 7, 16, 33, 70)))
+    reduction = str(rng.choice(("mean", "max", "sum", "min")))
+    print(f"seed {seed}: items {counts}, span {span}, centre {centre.tolist()}, voxel {voxel_size}, "
+          f"{channels} channels, {reduction}", flush=True)
+    feats = normal_features(len(pts), channels, seed=seed)
+    pc = Points(torch.as_tensor(pts, device=DEV), feats.to(DEV), offsets=torch.as_tensor(offsets))
+    st = pc.to_voxels(voxel_size, reduction=reduction)
+    coords, vfeats, voffsets = voxelize.points_to_voxels(pts, feats.double().numpy(), offsets, voxel_size,
+                                                         reduction)
+    assert np.array_equal(st.coordinate_tensor.cpu().numpy(), coords)
+    assert np.array_equal(st.offsets.numpy(), voffsets)
+    got = st.feature_tensor.double().cpu().numpy()
+    if reduction in ("max", "min"):
+        assert np.array_equal(got, vfeats)
+    else:
+        assert rel_err(got, vfeats) <= 1e-5
