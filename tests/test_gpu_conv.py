@@ -683,3 +683,45 @@ def test_dilated_convolution_matches_oracle(oracle):
     assert rel_err(y.feature_tensor.cpu().numpy(), want) <= 1e-5
     km = next(iter(vox.cache.values()))
     assert np.array_equal(km.in_maps.cpu().numpy(), im) and np.array_equal(km.out_maps.cpu().numpy(), om)
+
+
+CHOICE_CASES = [
+    # name, dtype, c_in, c_out, voxels, kernel: shapes the wide-row, narrow-row and pair-packed kernels take by default
+    ("f16_16_16", torch.float16, 16, 16, 6000, (3, 3, 3)),
+    ("bf16_32_32_k5", torch.bfloat16, 32, 32, 3000, (5, 5, 5)),
+    ("f16_64_64", torch.float16, 64, 64, 6000, (3, 3, 3)),
+    ("f32_32_32", torch.float32, 32, 32, 6000, (3, 3, 3)),
+    ("f16_128_128_rows", torch.float16, 128, 128, 26000, (3, 3, 3)),
+    ("bf16_160_96", torch.bfloat16, 160, 96, 3000, (3, 3, 3)),
+]
+
+
+@pytest.mark.parametrize("name,dtype,c_in,c_out,n,ksize", CHOICE_CASES, ids=[c[0] for c in CHOICE_CASES])
+def test_the_kernels_behind_the_environment_switch_agree(oracle, monkeypatch, name, dtype, c_in, c_out, n, ksize):
+    """WCN_CONV_KERNEL=ring keeps every shape on the ring kernel (the documented fallback),
+    WCN_CONV_KERNEL=pack skips the kernels for narrow and for wide rows: all three choices against
+    the oracle, and against each other within two roundings of the element type."""
+    from warpconvnet_amd._lib import lib
+    from warpconvnet_amd.geometry.coords.search.torch_discrete import generate_kernel_map
+    from warpconvnet_amd.nn.functional.sparse_conv import sparse_conv_forward
+    bc = synthetic.random_cloud(77, n, 30)
+    c = torch.as_tensor(bc, device=DEV)
+    km = generate_kernel_map(c, c, (1, 1, 1), ksize)
+    K = int(np.prod(ksize))
+    x = normal_features(len(bc), c_in, seed=11, dtype=dtype)
+    w = kaiming_weight(K, c_in, c_out, seed=12, dtype=dtype)
+    want, _ = _oracle_out(oracle, x, w, bc, bc, ksize, (1, 1, 1))
+    results, kernels = {}, {}
+    for choice in ("", "pack", "ring"):
+        if choice:
+            monkeypatch.setenv("WCN_CONV_KERNEL", choice)
+        else:
+            monkeypatch.delenv("WCN_CONV_KERNEL", raising=False)
+        got = sparse_conv_forward(x.to(DEV), w.to(DEV), km, len(bc))
+        kernels[choice] = lib().wcn_conv_last_kernel().decode()
+        results[choice] = got.float().cpu().numpy()
+        assert rel_err(results[choice], want) <= TOL[dtype], (name, choice, kernels[choice])
+    assert kernels["ring"].startswith(("conv_fwd_ring<", "conv_fwd<")), kernels
+    assert kernels["pack"].startswith(("conv_fwd_pack<", "conv_fwd_ring<", "conv_fwd<")), kernels
+    for choice in ("pack", "ring"):
+        assert rel_err(results[choice], results[""]) <= 2 * TOL[dtype]

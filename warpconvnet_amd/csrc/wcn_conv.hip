@@ -31,6 +31,7 @@
 // (M * C_out * s); the weights (K * C_in * C_out * s) stay cache resident.
 #include <algorithm>
 #include <cstdlib>
+#include <cstring>
 #include <mutex>
 #include <string>
 #include <type_traits>
@@ -1136,10 +1137,9 @@ int launch_conv(const ConvArgs& a, hipStream_t s) {
   // at most 32 channels on both sides to the kernel of wcn_conv_group.hip, rows of up to four
   // k-slices to the pair-packed kernel.  WCN_CONV_KERNEL=ring in the environment keeps everything on
   // the kernels below, WCN_CONV_KERNEL=pack skips the first two of the three (for comparisons).
-  static const int only = [] {
-    const char* e = getenv("WCN_CONV_KERNEL");
-    return !e ? 0 : std::string(e) == "ring" ? 1 : std::string(e) == "pack" ? 2 : 0;
-  }();
+  // (read at every call, a fraction of a microsecond, so that one process can compare them)
+  const char* const choice = getenv("WCN_CONV_KERNEL");
+  const int only = !choice ? 0 : strcmp(choice, "ring") == 0 ? 1 : strcmp(choice, "pack") == 0 ? 2 : 0;
   const bool ring_only = only == 1;
   if (only == 0 && wcn_conv_dense_takes(a, dtype)) {
     if (g_time_start) (void)hipEventRecord(g_time_start, s);
