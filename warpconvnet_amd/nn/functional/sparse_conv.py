@@ -97,16 +97,22 @@ def _prepared_weight(weight: Tensor, make_w, dtype: torch.dtype, c_in: int) -> T
     key = (weight._version, weight.data_ptr(), weight.dtype, dtype, tuple(weight.shape), c_in)
     kept = getattr(weight, "_wcn_prepared", None)
     if kept is not None and kept[0] == key:
+        # made on another stream (another thread's, say): this stream waits for that kernel
+        if kept[3] != stream_ptr(weight.device):
+            torch.cuda.current_stream(weight.device).wait_event(kept[2])
         return kept[1]
     L = lib()
     w = make_w()
     K, c_in, c_out = w.shape
     nbytes = L.wcn_conv_prepared_weight_bytes(K, c_in, c_out, DTYPE_CODE[dtype])
     tiles = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+    stream = stream_ptr(w.device)
     check(L.wcn_conv_prepare_weight(ptr(w), DTYPE_CODE[w.dtype], K, c_in, c_out, DTYPE_CODE[dtype],
-                                    ptr(tiles), nbytes, stream_ptr(w.device)), "wcn_conv_prepare_weight")
+                                    ptr(tiles), nbytes, stream), "wcn_conv_prepare_weight")
+    made = torch.cuda.Event()
+    made.record(torch.cuda.current_stream(w.device))
     try:
-        weight._wcn_prepared = (key, tiles)
+        weight._wcn_prepared = (key, tiles, made, stream)
     except AttributeError:
         pass
     return tiles
