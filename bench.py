@@ -657,7 +657,7 @@ def main():
                 w.join()
             torch.cuda.synchronize()
             elapsed_c = time.perf_counter() - t0
-        assert all(torch.equal(o, out) for o in outs)
+        assert len(outs) == threads and all(torch.equal(o, out) for o in outs)  # no thread gave up
         concurrent[f"{threads} streams"] = {
             "ms_per_step": elapsed_c * 1e3 / (threads * args.steps),
             "voxels_per_s": n * threads * args.steps / elapsed_c}

@@ -15,6 +15,16 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+@pytest.fixture(autouse=True)
+def _enough_memory():
+    """The cases here take up to some 60 GB of device memory."""
+    free, _ = torch.cuda.mem_get_info(0)
+    if free < (96 << 30):
+        pytest.skip(f"{free >> 30} GiB of device memory free; these cases are sized for an MI355X")
+    yield
+    torch.cuda.empty_cache()
+
+
 def _random_voxels(n, extent, seed):
     """n distinct voxels of an extent^3 box in random order, four batch items of n / 4 rows."""
     g = torch.Generator(device=DEV).manual_seed(seed)
