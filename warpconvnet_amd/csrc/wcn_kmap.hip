@@ -366,8 +366,41 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
                                                        int64_t* __restrict__ row_total,
                                                        KmapFinish fin) {
   __shared__ int s_wave[16];
+  __shared__ int s_stat[2][16];
   int32_t* row = groups + (int64_t)blockIdx.x * (G + 1);
   const int lane = wcn_lane(), wave = threadIdx.x >> 6;
+  if (fin.result && blockIdx.x == 0) {
+    // Occupied slots and distinct keys of the table, for the host's one read: the sums of the
+    // bins' counts, final since the table was built.  The first workgroup adds them up with all
+    // its threads while its row's entries are on their way; whichever workgroup finishes last
+    // finds the word in place.
+    const int32_t bins = fin.hdr->bins;
+    const int32_t* stats = reinterpret_cast<const int32_t*>(reinterpret_cast<const char*>(fin.hdr) + fin.hdr->stats_offset);
+    int voxels = 0, occupied = 0;
+    for (int i = threadIdx.x; i < bins; i += 1024) {
+      voxels += stats[2 * i];
+      occupied += stats[2 * i + 1];
+    }
+#pragma unroll
+    for (int sft = 32; sft > 0; sft >>= 1) {
+      voxels += __shfl_xor(voxels, sft, 64);
+      occupied += __shfl_xor(occupied, sft, 64);
+    }
+    if (lane == 0) {
+      s_stat[0][wave] = voxels;
+      s_stat[1][wave] = occupied;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      voxels = occupied = 0;
+      for (int w = 0; w < 16; ++w) {
+        voxels += s_stat[0][w];
+        occupied += s_stat[1][w];
+      }
+      // written before this thread's ticket (and the fence in front of it) further down
+      fin.result[fin.K + 2] = (int64_t)occupied | ((int64_t)(voxels != fin.hdr->num_keys ? 1 : 0) << 32);
+    }
+  }
   int64_t carry = 0;
   constexpr int PER = 4;  // entries per thread and round (one 16-byte load)
   for (int64_t start = 0; start < G; start += 1024 * PER) {
@@ -431,27 +464,12 @@ __global__ void __launch_bounds__(1024) kmap_scan_rows(int32_t* __restrict__ gro
     }
     run += __shfl(v, 63, 64);
   }
-  // occupied slots and distinct keys of the table: the sums of the bins' counts
-  int voxels = 0, occupied = 0;
-  {
-    const int32_t bins = fin.hdr->bins;
-    const int32_t* stats = reinterpret_cast<const int32_t*>(reinterpret_cast<const char*>(fin.hdr) + fin.hdr->stats_offset);
-    for (int i = lane; i < bins; i += 64) {
-      voxels += stats[2 * i];
-      occupied += stats[2 * i + 1];
-    }
-#pragma unroll
-    for (int sft = 32; sft > 0; sft >>= 1) {
-      voxels += __shfl_xor(voxels, sft, 64);
-      occupied += __shfl_xor(occupied, sft, 64);
-    }
-  }
   if (lane == 0) {
     const int64_t status = fin.hdr->status;
-    const int64_t blocks = (int64_t)occupied | ((int64_t)(voxels != fin.hdr->num_keys ? 1 : 0) << 32);
+    // occupied slots | duplicates << 32: left there by the first workgroup (see the top)
+    const int64_t blocks = __hip_atomic_load(&fin.result[fin.K + 2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     fin.result[0] = 0;
     fin.result[fin.K + 1] = status;
-    fin.result[fin.K + 2] = blocks;
     if (fin.mailbox) {
       fin.mailbox[1] = 0;
       fin.mailbox[1 + fin.K + 1] = status;
